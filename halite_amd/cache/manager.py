@@ -1,0 +1,184 @@
+"""The cache manager: groups of pages, block tables, slots and per-request state.
+
+Everything here is host bookkeeping except the page storage and the state rows.  A
+step asks for room for its tokens first (all groups or none), runs, then advances
+the requests' lengths, at which point windowed groups give back the pages that have
+been passed.  When a request ends, all its pages and its slot return.  The idle
+invariant is the reference's ``check_memory``
+(src/halite/transformers/infer/engine/scheduler.py:109-123): every page but the
+reserved one is free and every slot is free.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..parts.base import PagedKVNeed, StateNeed
+from .pages import CacheGroup, LayerPages, NoSpace, PagePool
+from .slots import SlotAllocator, StateStore
+
+
+class CacheManager:
+    def __init__(
+        self,
+        needs: dict[int, PagedKVNeed],
+        borrowed: dict[int, int] | None = None,
+        state_needs: dict[int, dict[str, StateNeed]] | None = None,
+        *,
+        page_size: int,
+        num_pages: int,
+        n_slots: int,
+        dtype: torch.dtype = torch.float32,
+        device="cpu",
+        allocate: bool = True,
+    ):
+        """``needs[run]`` for every run that owns a cache; ``borrowed[run] = owner``
+        for runs that read another run's cache; ``num_pages`` counts the reserved
+        page 0 of each group."""
+        self.page_size = page_size
+        self.num_pages = num_pages
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.groups: list[CacheGroup] = []
+        self.group_of_run: dict[int, int] = {}
+        by_need: dict[PagedKVNeed, CacheGroup] = {}
+        for run in sorted(needs):
+            need = needs[run]
+            if need not in by_need:
+                g = CacheGroup(len(self.groups), need, [], page_size, PagePool(num_pages))
+                by_need[need] = g
+                self.groups.append(g)
+            by_need[need].runs.append(run)
+            self.group_of_run[run] = by_need[need].group_id
+        self.borrowed = dict(borrowed or {})
+        for run, owner in self.borrowed.items():
+            if owner not in self.group_of_run:
+                raise ValueError(f"run {run} borrows the cache of run {owner}, which owns none")
+            self.group_of_run[run] = self.group_of_run[owner]
+        self._pages: dict[int, LayerPages] = {}
+        for g in self.groups:
+            k, d = g.need.n_kv_heads, g.need.head_dim
+            if allocate:
+                g.storage = torch.zeros(
+                    (len(g.runs), 2, num_pages, k * page_size * d), dtype=dtype, device=self.device
+                )
+            for i, run in enumerate(g.runs):
+                if allocate:
+                    kp = g.storage[i, 0].view(num_pages, k, page_size, d)
+                    vp = g.storage[i, 1].view(num_pages, k, d, page_size)
+                else:
+                    kp = vp = None
+                self._pages[run] = LayerPages(g.group_id, kp, vp)
+        for run, owner in self.borrowed.items():
+            self._pages[run] = self._pages[owner]
+        self.slots = SlotAllocator(n_slots)
+        self.state = StateStore(n_slots, state_needs or {}, self.device if allocate else "cpu")
+        self.lengths: dict[int, int] = {}
+
+    # -- sizes ------------------------------------------------------------------
+    @staticmethod
+    def bytes_per_page(needs: dict[int, PagedKVNeed], page_size: int, dtype: torch.dtype) -> int:
+        """Bytes that one page number costs over all groups and runs."""
+        return sum(2 * n.n_kv_heads * n.head_dim * page_size * dtype.itemsize for n in needs.values())
+
+    @property
+    def token_capacity(self) -> int:
+        return (self.num_pages - 1) * self.page_size
+
+    def free_pages(self) -> int:
+        """Free pages of the tightest group."""
+        return min((g.pool.available for g in self.groups), default=0)
+
+    def layer_pages(self, run: int) -> LayerPages | None:
+        return self._pages.get(run)
+
+    def state_of_run(self, run: int) -> dict[str, torch.Tensor]:
+        return self.state.tensors.get(run, {})
+
+    # -- requests -----------------------------------------------------------------
+    def admit(self) -> int:
+        slot = self.slots.alloc()
+        self.lengths[slot] = 0
+        self.state.reset(slot)
+        return slot
+
+    def length(self, slot: int) -> int:
+        return self.lengths[slot]
+
+    def pages_missing(self, spans: list[tuple[int, int]]) -> list[int]:
+        """Per group, the pages that ``reserve`` would take for ``(slot, new
+        length)`` spans (each span starts at the slot's current length)."""
+        return [
+            sum(g.pages_missing(slot, self.lengths[slot], new_len) for slot, new_len in spans)
+            for g in self.groups
+        ]
+
+    def can_reserve(self, spans: list[tuple[int, int]]) -> bool:
+        return all(m <= g.pool.available for m, g in zip(self.pages_missing(spans), self.groups))
+
+    def reserve(self, spans: list[tuple[int, int]]) -> None:
+        """Room for every span in every group, or ``NoSpace`` and nothing taken."""
+        for slot, new_len in spans:
+            if new_len <= self.lengths[slot]:
+                raise ValueError(f"slot {slot}: new length {new_len} does not extend {self.lengths[slot]}")
+        missing = self.pages_missing(spans)
+        for m, g in zip(missing, self.groups):
+            if m > g.pool.available:
+                raise NoSpace(f"group {g.group_id}: {m} pages wanted, {g.pool.available} free")
+        for g in self.groups:
+            for slot, new_len in spans:
+                g.reserve(slot, self.lengths[slot], new_len)
+
+    def advance(self, slot: int, new_len: int) -> None:
+        """The tokens up to ``new_len`` are in the cache now."""
+        self.lengths[slot] = new_len
+        for g in self.groups:
+            g.release_passed(slot, new_len)
+
+    def free(self, slot: int) -> None:
+        for g in self.groups:
+            g.release_all(slot)
+        del self.lengths[slot]
+        self.slots.free(slot)
+
+    # -- what a step reads ----------------------------------------------------------
+    def block_table(self, group_id: int, slots: list[int]) -> np.ndarray:
+        """``[len(slots), P]`` int32, row i the page list of ``slots[i]``, -1 where
+        the request holds no page."""
+        g = self.groups[group_id]
+        width = max((len(g.tables.get(s, ())) for s in slots), default=0)
+        out = np.full((len(slots), max(width, 1)), -1, dtype=np.int32)
+        for i, s in enumerate(slots):
+            t = g.tables.get(s, ())
+            out[i, : len(t)] = t
+        return out
+
+    # -- invariants -------------------------------------------------------------------
+    def check(self) -> None:
+        """No page lost, none held twice; tables only of live slots."""
+        live = self.slots.live()
+        if set(self.lengths) != live:
+            raise AssertionError(f"lengths of {sorted(self.lengths)} but live slots {sorted(live)}")
+        for g in self.groups:
+            seen: dict[int, int] = {}
+            for slot, table in g.tables.items():
+                if slot not in live:
+                    raise AssertionError(f"group {g.group_id}: table of dead slot {slot}")
+                for p in table:
+                    if p < 0:
+                        continue
+                    if p == 0 or p >= g.pool.num_pages:
+                        raise AssertionError(f"group {g.group_id}: slot {slot} holds page {p}")
+                    if p in seen:
+                        raise AssertionError(f"group {g.group_id}: page {p} held by slots {seen[p]} and {slot}")
+                    seen[p] = slot
+            if set(seen) != g.pool.held_pages():
+                raise AssertionError(f"group {g.group_id}: tables and pool disagree on held pages")
+            if len(seen) + g.pool.available != g.pool.capacity:
+                raise AssertionError(f"group {g.group_id}: {len(seen)} held + {g.pool.available} free != {g.pool.capacity}")
+
+    def idle(self) -> bool:
+        return self.slots.available == self.slots.n_slots and all(
+            g.pool.available == g.pool.capacity for g in self.groups
+        )

@@ -1,0 +1,77 @@
+"""Options of the engine, under the reference's names where it has them.
+
+``ServerConfig`` takes the scheduler knobs of the reference's ``infer`` engine
+(src/halite/transformers/infer/types.py:67-81) and the paging and per-step limits of
+its ``tokainfer`` engine (src/halite/transformers/tokainfer/types.py:65-190);
+``ModelConfig`` keeps what src/halite/transformers/infer/types.py:84-113 holds beyond
+the sizes that the model's own configuration already gives.
+"""
+
+from __future__ import annotations
+
+from typing import Literal
+
+from pydantic import BaseModel, ConfigDict, Field, StrictBool, StrictInt
+
+
+class ServerConfig(BaseModel):
+    model_config = ConfigDict(extra="forbid")
+
+    # -- infer/types.py:67-81 ------------------------------------------------
+    max_prefill_tokens: StrictInt = Field(default=16384, gt=0)
+    """Most prompt tokens that one step may hold."""
+    chunked_prefill_size: StrictInt = Field(default=8192, gt=0)
+    """Most tokens of one prompt in one step; longer prompts are cut into portions."""
+    default_init_new_token_ratio: float = 0.7
+    default_min_new_token_ratio_factor: float = 0.14
+    default_new_token_ratio_decay_steps: StrictInt = 600
+    schedule_conservativeness: float = 1.0
+    use_cudagraph: StrictBool = False
+    """Replay decode-only steps from a captured HIP graph."""
+    cudagraph_max_batch_size: StrictInt = 64
+
+    # -- tokainfer/types.py:65-190 -------------------------------------------
+    page_size: StrictInt = Field(default=64, gt=0)
+    kv_cache_num_tokens: StrictInt | None = Field(default=None, gt=0)
+    """Tokens the cache pool holds; ``None`` sizes it from free device memory
+    with ``memory_fraction_static`` (infer/engine/model_runner.py:117-131)."""
+    max_tokens_per_forward: StrictInt = Field(default=8192, gt=0)
+    """Token budget of one step: decoded tokens plus prompt portions."""
+    max_seqs_per_forward: StrictInt = Field(default=256, gt=0)
+    """Most requests that are live (own a slot) at a time."""
+
+    # -- retraction (infer/engine/batch.py:468-527) ----------------------------
+    retract_decode_steps: StrictInt = Field(default=20, gt=0)
+
+
+class ModelConfig(BaseModel):
+    """Run-time options of the model (infer/types.py:84-113).  The sizes that the
+    reference repeats here (heads, layers) come from the model's configuration."""
+
+    model_config = ConfigDict(extra="forbid")
+
+    context_len: StrictInt | None = Field(default=None, gt=0)
+    """Longest request; ``None`` takes the model's ``max_position_embeddings``."""
+    dtype: Literal["bfloat16", "float32"] = "bfloat16"
+    kv_cache_dtype: Literal["auto"] = "auto"
+    memory_fraction_static: float = Field(default=0.88, gt=0, le=1)
+    gpu_id: StrictInt = 0
+    device: str = "cuda"
+
+
+def parse_overrides(pairs: list[str]) -> dict:
+    """``key=value`` command-line overrides (the reference's
+    ``apply_overrides``, scripts/eval_task.py:179-182) as a dict of strings
+    that pydantic then validates and converts."""
+    import json
+
+    out = {}
+    for pair in pairs:
+        if "=" not in pair:
+            raise ValueError(f"override {pair!r} is not of the form key=value")
+        key, value = pair.split("=", 1)
+        try:
+            out[key] = json.loads(value)
+        except json.JSONDecodeError:
+            out[key] = value
+    return out

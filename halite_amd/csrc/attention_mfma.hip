@@ -1,0 +1,286 @@
+// Paged attention on the matrix cores (bf16 operands, float32 accumulation and
+// softmax), for prefill portions and decode tokens alike.  Compiled for one head size,
+// HAL_HEAD_DIM (a multiple of 16, at most 256).
+//
+// The unit of work is a wavefront with one *item*: 16 query rows of one request and
+// one key/value head, against a range of that request's keys.  A query row is a
+// (token, head-in-group) pair, token-major, so the heads that share a key/value head
+// sit in the same tile and every key is loaded once for all of them.  The host lists
+// the items; an item whose key range is not the row's whole range writes a partial
+// result (unnormalised sum, running maximum, running denominator) that the merge
+// kernel combines with the log-sum-exp rule, the same rule that joins two partial
+// attentions in src/halite/transformers/tokainfer/attention_fn.py:147-167.
+//
+// Per 32 keys a wave computes S^T = K Q^T with v_mfma_f32_16x16x32_bf16 (A = 16 keys x
+// 32 dims of K straight from the key page, B = Q^T), the online softmax on the
+// accumulator layout (a lane owns one query row and eight keys), and O^T += V^T P^T
+// (A = 16 dims x 32 keys straight from the transposed value page, B = the lane's own
+// eight probabilities).  The keys of the two 16-key MFMA tiles are interleaved so that
+// a lane's eight probabilities are eight consecutive keys, which is one 16-byte load of
+// the transposed values.  Nothing goes through LDS.
+//
+// scores, causal rule and grouped heads as in src/halite/transformers/attention.py:
+// 647-714 and src/halite/transformers/infer/engine/flashinfer_backend.py:217-261.
+#include "hal_common.h"
+#include "hal_api.h"
+
+#ifndef HAL_HEAD_DIM
+#error "compile with -DHAL_HEAD_DIM=<head size>"
+#endif
+static_assert(HAL_HEAD_DIM % 16 == 0 && HAL_HEAD_DIM >= 16 && HAL_HEAD_DIM <= 256,
+              "head size must be a multiple of 16 up to 256");
+
+#define D HAL_HEAD_DIM
+#define KT ((D + 31) / 32)  // 32-wide steps over the head dimension for Q K^T
+#define DT (D / 16)         // 16-wide tiles of the head dimension for P V
+#define ITEM_INTS 8
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+__device__ __forceinline__ bf16x8 ld16(const bf16_t* p) {
+  return __builtin_bit_cast(bf16x8, *(const u32x4*)p);
+}
+__device__ __forceinline__ bf16x8 zero8() {
+  u32x4 z = {0u, 0u, 0u, 0u};
+  return __builtin_bit_cast(bf16x8, z);
+}
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo).bits | ((uint32_t)f32_to_bf16(hi).bits << 16);
+}
+
+// item: {segment, first row, first key, end key, partial index or -1, 0, 0, 0}
+__global__ void __launch_bounds__(256)
+attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
+                      int out_row_stride, const int* __restrict__ items,
+                      const int* __restrict__ n_items_ptr, const int* __restrict__ seg_q_start,
+                      const int* __restrict__ seg_q_len, const int* __restrict__ seg_kv_len,
+                      const int* __restrict__ block_table, int bt_stride,
+                      const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+                      float* __restrict__ part_o, float* __restrict__ part_ml, int H, int K,
+                      int page_size, float scale_log2e, int window) {
+  const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
+  const int item = blockIdx.x * (blockDim.x / HAL_WAVE) + wave;
+  if (item >= *n_items_ptr) return;
+  const int* it = items + (size_t)item * ITEM_INTS;
+  const int seg = it[0], rho0 = it[1], kv_begin = it[2], kv_end = it[3], partial = it[4];
+  const int g = blockIdx.y;
+  const int G = H / K;
+  const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], kv_len = seg_kv_len[seg];
+  const int pos0 = kv_len - q_len;  // position of the segment's first token
+  const int* bt = block_table + (size_t)seg * bt_stride;
+
+  const int col = lane % 16, quad = lane / 16;
+  // this lane's query row
+  const int rho = rho0 + col;
+  const bool row_ok = rho < q_len * G;
+  const int qi = row_ok ? rho / G : 0;
+  const int hg = row_ok ? rho % G : 0;
+  const int p_row = pos0 + qi;  // the row's position: sees keys <= p_row
+  const int lo_row = (window > 0 && p_row - window + 1 > 0) ? p_row - window + 1 : 0;
+  const int head = g * G + hg;
+
+  // Q^T as the B operand: lane holds Q[row][ks*32 + quad*8 .. +8]
+  bf16x8 bq[KT];
+  {
+    const bf16_t* qp = q + (size_t)(q_start + qi) * q_row_stride + (size_t)head * D;
+#pragma unroll
+    for (int ks = 0; ks < KT; ++ks) {
+      const int d0 = ks * 32 + quad * 8;
+      bq[ks] = (row_ok && d0 < D) ? ld16(qp + d0) : zero8();
+    }
+  }
+
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  const int last_key = kv_len - 1;  // keys beyond it are not written yet
+  for (int j0 = kv_begin & ~31; j0 < kv_end; j0 += 32) {
+    // ---- S^T = K Q^T for 32 keys (two tiles of 16) ------------------------------
+    f32x4 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      // row `col` of tile t is key j0 + (col/4)*8 + t*4 + col%4
+      int j = j0 + (col / 4) * 8 + t * 4 + (col % 4);
+      j = j < kv_begin ? kv_begin : (j > last_key ? last_key : j);  // address only
+      const long long page = bt[j / page_size];
+      const bf16_t* kp = k_pages + (((size_t)page * K + g) * page_size + (j % page_size)) * D;
+      s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KT; ++ks) {
+        const int d0 = ks * 32 + quad * 8;
+        const bf16x8 ka = d0 < D ? ld16(kp + d0) : zero8();
+        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, bq[ks], s[t], 0, 0, 0);
+      }
+    }
+    // ---- mask and online softmax: this lane has keys j0 + quad*8 + e, e = 0..7 ----
+    float sv[8];
+    float m_tile = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = j0 + quad * 8 + e;
+      const bool ok = row_ok && j >= kv_begin && j < kv_end && j >= lo_row && j <= p_row;
+      sv[e] = ok ? s[e / 4][e % 4] * scale_log2e : -INFINITY;
+      m_tile = fmaxf(m_tile, sv[e]);
+    }
+    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, HAL_WAVE));
+    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, HAL_WAVE));
+    const float m_new = fmaxf(m, m_tile);
+    float alpha = 1.f;
+    float pv[8];
+    if (m_new == -INFINITY) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pv[e] = 0.f;
+    } else {
+      alpha = exp2f(m - m_new);  // m = -inf gives 0
+      float psum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        pv[e] = exp2f(sv[e] - m_new);
+        psum += pv[e];
+      }
+      l = l * alpha + psum;
+      m = m_new;
+    }
+    u32x4 praw = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]),
+                  pack2(pv[6], pv[7])};
+    const bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
+
+    // ---- O^T += V^T P^T: lane loads V^T[dim dt*16 + col][keys j0 + quad*8 .. +8] ------
+    int jv = j0 + quad * 8;
+    const bool tail = j0 + 32 > kv_len;  // some of the 32 keys are not written yet
+    if (jv < (kv_begin & ~7)) jv = kv_begin & ~7;
+    if (jv > (last_key & ~7)) jv = last_key & ~7;
+    const long long vpage = bt[jv / page_size];
+    const bf16_t* vp = v_pages + ((size_t)vpage * K + g) * D * page_size + (jv % page_size);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      bf16x8 va = ld16(vp + (size_t)(dt * 16 + col) * page_size);
+      if (tail) {
+        // unwritten slots may hold anything, NaN included: 0 * NaN must not get in
+        u32x4 raw = __builtin_bit_cast(u32x4, va);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const int ja = jv + 2 * w;
+          uint32_t keep = 0u;
+          if (ja <= last_key) keep |= 0x0000ffffu;
+          if (ja + 1 <= last_key) keep |= 0xffff0000u;
+          raw[w] &= keep;
+        }
+        va = __builtin_bit_cast(bf16x8, raw);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, o[dt], 0, 0, 0);
+    }
+  }
+
+  // the denominator is spread over the four lanes that share a row
+  l += __shfl_xor(l, 16, HAL_WAVE);
+  l += __shfl_xor(l, 32, HAL_WAVE);
+
+  if (!row_ok) return;
+  if (partial < 0) {
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint2 w;
+      w.x = pack2(o[dt][0] * inv, o[dt][1] * inv);
+      w.y = pack2(o[dt][2] * inv, o[dt][3] * inv);
+      *(uint2*)(op + dt * 16 + quad * 4) = w;
+    }
+  } else {
+    float* po = part_o + (((size_t)partial * K + g) * 16 + col) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      *(f32x4*)(po + dt * 16 + quad * 4) = o[dt];
+    if (quad == 0) {
+      float* pm = part_ml + (((size_t)partial * K + g) * 16 + col) * 2;
+      pm[0] = m;
+      pm[1] = l;
+    }
+  }
+}
+
+// merge item: {segment, first row, first partial, number of partials}
+__global__ void attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
+                                       const int* __restrict__ merges,
+                                       const int* __restrict__ n_merges_ptr,
+                                       const int* __restrict__ seg_q_start,
+                                       const int* __restrict__ seg_q_len,
+                                       const float* __restrict__ part_o,
+                                       const float* __restrict__ part_ml, int H, int K) {
+  const int mi = blockIdx.x;
+  if (mi >= *n_merges_ptr) return;
+  const int g = blockIdx.y;
+  const int G = H / K;
+  const int* mg = merges + (size_t)mi * 4;
+  const int seg = mg[0], rho0 = mg[1], first = mg[2], n = mg[3];
+  const int q_start = seg_q_start[seg], q_len = seg_q_len[seg];
+  // one thread per (row, dim)
+  for (int idx = threadIdx.x; idx < 16 * D; idx += blockDim.x) {
+    const int row = idx / D, d = idx % D;
+    const int rho = rho0 + row;
+    if (rho >= q_len * G) continue;
+    float m_all = -INFINITY;
+    for (int i = 0; i < n; ++i)
+      m_all = fmaxf(m_all, part_ml[(((size_t)(first + i) * K + g) * 16 + row) * 2]);
+    float acc = 0.f, l_all = 0.f;
+    for (int i = 0; i < n; ++i) {
+      const size_t base = ((size_t)(first + i) * K + g) * 16 + row;
+      const float mi_ = part_ml[base * 2], li = part_ml[base * 2 + 1];
+      const float w = (mi_ == -INFINITY) ? 0.f : exp2f(mi_ - m_all);
+      acc += w * part_o[base * D + d];
+      l_all += w * li;
+    }
+    const int qi = rho / G, head = g * G + rho % G;
+    out[(size_t)(q_start + qi) * out_row_stride + (size_t)head * D + d] =
+        f32_to_bf16(l_all > 0.f ? acc / l_all : 0.f);
+  }
+}
+
+extern "C" int hal_attention_mfma_head_dim() { return D; }
+
+// Host arrays are device pointers: items [max_items, 8], merges [max_merges, 4], the
+// live counts in n_items / n_merges (so a captured launch can serve a varying count).
+extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_stride,
+                                  const int* items, const int* n_items, int max_items,
+                                  const int* merges, const int* n_merges, int max_merges,
+                                  const int* seg_q_start, const int* seg_q_len,
+                                  const int* seg_kv_len, const int* block_table, int bt_stride,
+                                  const void* k_pages, const void* v_pages, float* part_o,
+                                  float* part_ml, int H, int K, int head_dim, int page_size,
+                                  float scale, int window, hipStream_t stream) {
+  HAL_REQUIRE(head_dim == D, "hal_attention_mfma: built for head size %d, called with %d", D,
+              head_dim);
+  HAL_REQUIRE(H > 0 && K > 0 && H % K == 0, "hal_attention_mfma: %d heads, %d kv heads", H, K);
+  HAL_REQUIRE(K <= 65535, "hal_attention_mfma: %d kv heads exceed the grid limit", K);
+  HAL_REQUIRE(page_size > 0 && page_size % 8 == 0,
+              "hal_attention_mfma: page size %d must be a multiple of 8", page_size);
+  HAL_REQUIRE(q_row_stride % 8 == 0 && out_row_stride % 4 == 0 && ((uintptr_t)q % 16) == 0 &&
+                  ((uintptr_t)out % 8) == 0,
+              "hal_attention_mfma: q and out rows must be 16-byte aligned");
+  HAL_REQUIRE(window >= 0 && max_items >= 0 && max_merges >= 0, "hal_attention_mfma: bad counts");
+  HAL_REQUIRE(max_merges == 0 || (part_o && part_ml), "hal_attention_mfma: no partial buffers");
+  if (max_items == 0) return 0;
+  const float scale_log2e = scale * 1.4426950408889634f;
+  const int waves = 4;
+  dim3 grid((max_items + waves - 1) / waves, K);
+  hipLaunchKernelGGL(attention_mfma_kernel, grid, dim3(waves * HAL_WAVE), 0, stream,
+                     (const bf16_t*)q, q_row_stride, (bf16_t*)out, out_row_stride, items, n_items,
+                     seg_q_start, seg_q_len, seg_kv_len, block_table, bt_stride,
+                     (const bf16_t*)k_pages, (const bf16_t*)v_pages, part_o, part_ml, H, K,
+                     page_size, scale_log2e, window);
+  HAL_LAUNCH_CHECK();
+  if (max_merges > 0) {
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K), dim3(256), 0, stream,
+                       (bf16_t*)out, out_row_stride, merges, n_merges, seg_q_start, seg_q_len,
+                       part_o, part_ml, H, K);
+    HAL_LAUNCH_CHECK();
+  }
+  return 0;
+}

@@ -1,0 +1,269 @@
+// Embedding lookup, RMSNorm (with the residual add and a row gather fused in),
+// SiLU-gate multiply, and rotary position encoding fused with the append of keys
+// and values to their cache pages.  All arithmetic is float32; T is the element
+// type of activations and cache (float or bf16).
+#include "hal_common.h"
+#include "hal_api.h"
+
+// ---------------------------------------------------------------------------------
+// h[t, :] = table[ids[t], :]  (float32 residual stream)
+// src/halite/transformers/embedding.py:36-44
+// ---------------------------------------------------------------------------------
+template <typename TT>
+__global__ void embedding_kernel(const int* __restrict__ ids, const TT* __restrict__ table,
+                                 float* __restrict__ out, int d, int vocab) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  float* o = out + (size_t)t * d;
+  if (id < 0 || id >= vocab) {
+    // an id outside the table is a caller's fault; make it visible, not a fault
+    for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = __uint_as_float(0x7fc00000u);
+    return;
+  }
+  const TT* row = table + (size_t)id * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = to_f32(row[i]);
+}
+
+extern "C" int hal_embedding(const int* ids, const void* table, int table_dtype, float* out,
+                             int n_tokens, int d, int vocab, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && d > 0 && vocab > 0, "hal_embedding: bad sizes T=%d d=%d V=%d",
+              n_tokens, d, vocab);
+  if (n_tokens == 0) return 0;
+  const int threads = d >= 1024 ? 256 : 64;
+  if (table_dtype == HAL_F32)
+    hipLaunchKernelGGL(embedding_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream, ids,
+                       (const float*)table, out, d, vocab);
+  else if (table_dtype == HAL_BF16)
+    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream, ids,
+                       (const bf16_t*)table, out, d, vocab);
+  else
+    return hal_fail("hal_embedding: unknown table dtype %d", table_dtype);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------
+// RMSNorm over the float32 residual stream.
+//   x = h[src] (+ delta[src]);  h[src] = x when update_h
+//   out[r] = w * T(x * rsqrt(mean(x^2) + eps))
+// src = rows[r] if rows is given, else r.  The statistics and the scaling are
+// float32; the normalised value is rounded to T before the weight multiplies it,
+// as src/halite/nn/normalization.py:43-57 does.
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                               const int* __restrict__ rows, const void* __restrict__ w,
+                               int w_dtype, float eps, T* __restrict__ out, int d, int update_h) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float* hr = h + (size_t)src * d;
+  const T* dr = delta ? delta + (size_t)src * d : nullptr;
+  T* o = out + (size_t)r * d;
+
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float x = hr[i];
+    if (dr) x += to_f32(dr[i]);
+    ss += x * x;
+  }
+  const float total = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(total / (float)d + eps);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float x = hr[i];
+    if (dr) {
+      x += to_f32(dr[i]);
+      if (update_h) hr[i] = x;
+    }
+    const T n = from_f32<T>(x * rstd);
+    o[i] = from_f32<T>(load_as_f32(w, w_dtype, i) * to_f32(n));
+  }
+}
+
+extern "C" int hal_rmsnorm(float* h, const void* delta, const int* rows, const void* w,
+                           int w_dtype, float eps, void* out, int dtype, int n_rows, int d,
+                           int update_h, hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && d > 0, "hal_rmsnorm: bad sizes rows=%d d=%d", n_rows, d);
+  HAL_REQUIRE(w_dtype == HAL_F32 || w_dtype == HAL_BF16, "hal_rmsnorm: weight dtype %d", w_dtype);
+  HAL_REQUIRE(!(rows && update_h && delta),
+              "hal_rmsnorm: a gathered call must not update the residual stream");
+  if (n_rows == 0) return 0;
+  const int threads = d >= 2048 ? 512 : (d >= 512 ? 256 : 64);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(n_rows), dim3(threads), 0, stream, h,
+                       (const float*)delta, rows, w, w_dtype, eps, (float*)out, d, update_h);
+  else if (dtype == HAL_BF16)
+    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(n_rows), dim3(threads), 0, stream, h,
+                       (const bf16_t*)delta, rows, w, w_dtype, eps, (bf16_t*)out, d, update_h);
+  else
+    return hal_fail("hal_rmsnorm: unknown dtype %d", dtype);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// h += delta (float32 stream, delta of type T); used for the last pending delta.
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ h, const T* __restrict__ delta, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) h[i] += to_f32(delta[i]);
+}
+
+extern "C" int hal_residual_add(float* h, const void* delta, int dtype, long long n,
+                                hipStream_t stream) {
+  HAL_REQUIRE(n >= 0, "hal_residual_add: n=%lld", n);
+  if (n == 0) return 0;
+  const int threads = 256;
+  const int blocks = (int)((n + threads - 1) / threads < 4096 ? (n + threads - 1) / threads : 4096);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(residual_add_kernel<float>, dim3(blocks), dim3(threads), 0, stream, h,
+                       (const float*)delta, (size_t)n);
+  else if (dtype == HAL_BF16)
+    hipLaunchKernelGGL(residual_add_kernel<bf16_t>, dim3(blocks), dim3(threads), 0, stream, h,
+                       (const bf16_t*)delta, (size_t)n);
+  else
+    return hal_fail("hal_residual_add: unknown dtype %d", dtype);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------
+// out[t, f] = up[t, f] * silu(gate[t, f]); gate and up are the two halves of one
+// row of `gu` ([T, 2F], gate first).  silu(x) = x * sigmoid(x) in float32.
+// src/halite/transformers/feedforward.py:204-212
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_tokens,
+                                int F) {
+  const size_t n = (size_t)n_tokens * F;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    const size_t t = i / F, f = i % F;
+    const float g = to_f32(gu[t * 2 * F + f]);
+    const float u = to_f32(gu[t * 2 * F + F + f]);
+    const float s = g / (1.0f + expf(-g));
+    out[i] = from_f32<T>(u * s);
+  }
+}
+
+extern "C" int hal_silu_mul(const void* gu, void* out, int dtype, int n_tokens, int F,
+                            hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && F > 0, "hal_silu_mul: bad sizes T=%d F=%d", n_tokens, F);
+  if (n_tokens == 0) return 0;
+  const size_t n = (size_t)n_tokens * F;
+  const int threads = 256;
+  const size_t want = (n + threads - 1) / threads;
+  const int blocks = (int)(want < 8192 ? want : 8192);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(silu_mul_kernel<float>, dim3(blocks), dim3(threads), 0, stream,
+                       (const float*)gu, (float*)out, n_tokens, F);
+  else if (dtype == HAL_BF16)
+    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, dim3(blocks), dim3(threads), 0, stream,
+                       (const bf16_t*)gu, (bf16_t*)out, n_tokens, F);
+  else
+    return hal_fail("hal_silu_mul: unknown dtype %d", dtype);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------
+// Rotary position encoding of q and k, in place in the packed row
+// [q heads | k heads | v heads], and the append of the rotated k and of v to the
+// cache pages of the token's request.
+//   half-split pairs (j, j + rot/2):  src/halite/transformers/position.py:287-291
+//   adjacent pairs (2j, 2j + 1):      src/halite/transformers/position.py:294-300
+// The angle table is float32 [table_len, rot/2] (position.py:140-167); the
+// rotation is float32 and rounded once to T.
+// Key pages are [page][kv head][slot in page][D]; value pages are transposed,
+// [page][kv head][D][slot in page], so that the attention kernels read eight keys
+// of one dimension with one load.
+// src/halite/transformers/infer/engine/memory_pool.py:139-141 (append after rotation)
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
+                                   const int* __restrict__ positions,
+                                   const int* __restrict__ token_seg,
+                                   const int* __restrict__ block_table, int bt_stride,
+                                   const float* __restrict__ cos_t,
+                                   const float* __restrict__ sin_t, int table_len,
+                                   T* __restrict__ k_pages, T* __restrict__ v_pages, int H,
+                                   int K, int D, int rot, int interleaved, int page_size,
+                                   int n_pages) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  T* row = qkv + (size_t)t * row_stride;
+  const int half = rot / 2;
+  if (rot > 0 && (pos < 0 || pos >= table_len)) return;  // checked on the host; never index outside
+
+  long long page = -1;
+  int off = 0;
+  if (K > 0) {
+    page = block_table[(size_t)token_seg[t] * bt_stride + pos / page_size];
+    off = pos % page_size;
+    if (page < 0 || page >= n_pages) page = -1;  // checked on the host
+  }
+
+  const float* cp = cos_t + (size_t)pos * half;
+  const float* sp = sin_t + (size_t)pos * half;
+  for (int idx = threadIdx.x; idx < (H + K) * half; idx += blockDim.x) {
+    const int head = idx / half, j = idx % half;
+    const int i0 = interleaved ? 2 * j : j;
+    const int i1 = interleaved ? 2 * j + 1 : j + half;
+    T* hp = row + (size_t)head * D;
+    const float c = cp[j], s = sp[j];
+    const float x0 = to_f32(hp[i0]), x1 = to_f32(hp[i1]);
+    const T y0 = from_f32<T>(x0 * c - x1 * s);
+    const T y1 = from_f32<T>(x0 * s + x1 * c);
+    hp[i0] = y0;
+    hp[i1] = y1;
+    if (head >= H && page >= 0) {
+      const int g = head - H;
+      T* kp = k_pages + (((size_t)page * K + g) * page_size + off) * D;
+      kp[i0] = y0;
+      kp[i1] = y1;
+    }
+  }
+  if (page < 0) return;
+  // dimensions of k beyond the rotated ones pass through
+  const int rest = D - rot;
+  for (int idx = threadIdx.x; idx < K * rest; idx += blockDim.x) {
+    const int g = idx / rest, i = rot + idx % rest;
+    k_pages[(((size_t)page * K + g) * page_size + off) * D + i] = row[(size_t)(H + g) * D + i];
+  }
+  for (int idx = threadIdx.x; idx < K * D; idx += blockDim.x) {
+    const int g = idx / D, i = idx % D;
+    v_pages[(((size_t)page * K + g) * D + i) * page_size + off] = row[(size_t)(H + K + g) * D + i];
+  }
+}
+
+extern "C" int hal_rope_append(void* qkv, int dtype, int row_stride, const int* positions,
+                               const int* token_seg, const int* block_table, int bt_stride,
+                               const float* cos_t, const float* sin_t, int table_len,
+                               void* k_pages, void* v_pages, int n_tokens, int H, int K, int D,
+                               int rot, int interleaved, int page_size, int n_pages,
+                               hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && H >= 0 && K >= 0 && D > 0, "hal_rope_append: bad sizes");
+  HAL_REQUIRE(rot >= 0 && rot <= D && rot % 2 == 0, "hal_rope_append: rotary dim %d of %d", rot, D);
+  HAL_REQUIRE(row_stride >= (H + 2 * K) * D, "hal_rope_append: row stride %d < %d", row_stride,
+              (H + 2 * K) * D);
+  HAL_REQUIRE(K == 0 || (k_pages && v_pages && block_table && token_seg && page_size > 0),
+              "hal_rope_append: cache arguments missing");
+  if (n_tokens == 0) return 0;
+  const int work = (H + K) * (rot / 2) > K * D ? (H + K) * (rot / 2) : K * D;
+  const int threads = work >= 1024 ? 256 : (work >= 256 ? 128 : 64);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(rope_append_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream,
+                       (float*)qkv, row_stride, positions, token_seg, block_table, bt_stride,
+                       cos_t, sin_t, table_len, (float*)k_pages, (float*)v_pages, H, K, D, rot,
+                       interleaved, page_size, n_pages);
+  else if (dtype == HAL_BF16)
+    hipLaunchKernelGGL(rope_append_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream,
+                       (bf16_t*)qkv, row_stride, positions, token_seg, block_table, bt_stride,
+                       cos_t, sin_t, table_len, (bf16_t*)k_pages, (bf16_t*)v_pages, H, K, D, rot,
+                       interleaved, page_size, n_pages);
+  else
+    return hal_fail("hal_rope_append: unknown dtype %d", dtype);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}

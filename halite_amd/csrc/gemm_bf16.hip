@@ -1,0 +1,188 @@
+// C[M, N] = X[M, K] * W[N, K]^T for few rows of X (decode batches): bf16 operands,
+// float32 accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16), bound by the
+// one pass over W.  W is a linear layer's weight as stored ([out, in]); it is read
+// straight from memory into the MFMA operand layout, 64 contiguous bytes of a row
+// per load instruction, and never staged.
+//
+// A wavefront owns 16*NT rows of W and 16*MT rows of X and a share of K; the waves
+// of a workgroup split K among them and their partial sums are added in wave order
+// through LDS, so the result is deterministic.  The epilogue writes bf16 or float32,
+// can add into a float32 destination (the residual stream), and in the gated form
+// computes up * silu(gate) from two weights at once
+// (src/halite/transformers/feedforward.py:204-212).
+#include "hal_common.h"
+#include "hal_api.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+__device__ __forceinline__ bf16x8 load_frag(const bf16_t* p, bool valid) {
+  u32x4 raw = {0u, 0u, 0u, 0u};
+  if (valid) raw = *(const u32x4*)p;
+  return __builtin_bit_cast(bf16x8, raw);
+}
+
+enum { SK_OUT_BF16 = 0, SK_OUT_F32 = 1, SK_OUT_F32_ADD = 2 };
+
+template <int NT, int MT, bool GATED>
+__global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
+                                   const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
+                                   int ldw, void* __restrict__ C, int ldc, int out_mode, int M,
+                                   int N, int K) {
+  extern __shared__ float red[];  // [sets][NT*MT][64][4]
+  const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
+  const int n_waves = blockDim.x / HAL_WAVE;
+  const int r = lane % 16, q = lane / 16;
+  const int n_base = blockIdx.x * 16 * NT;
+  constexpr int SETS = GATED ? 2 : 1;
+
+  const int steps = (K + 31) / 32;
+  const int per_wave = (steps + n_waves - 1) / n_waves;
+  const int s_begin = wave * per_wave;
+  const int s_end = s_begin + per_wave < steps ? s_begin + per_wave : steps;
+
+  f32x4 acc[SETS][NT][MT];
+#pragma unroll
+  for (int s = 0; s < SETS; ++s)
+#pragma unroll
+    for (int f = 0; f < NT; ++f)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[s][f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const bf16_t* wrow[NT];
+  const bf16_t* w2row[NT];
+#pragma unroll
+  for (int f = 0; f < NT; ++f) {
+    int n = n_base + f * 16 + r;
+    if (n >= N) n = N - 1;  // rows past the end are computed and dropped
+    wrow[f] = W + (size_t)n * ldw;
+    w2row[f] = GATED ? W2 + (size_t)n * ldw : nullptr;
+  }
+  const bf16_t* xrow[MT];
+  bool xvalid[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + r;
+    xvalid[t] = m < M;
+    xrow[t] = X + (size_t)(xvalid[t] ? m : 0) * ldx;
+  }
+
+#pragma unroll 2
+  for (int step = s_begin; step < s_end; ++step) {
+    const int k = step * 32 + q * 8;
+    const bool kv = k < K;  // K is a multiple of 8
+    bf16x8 a[NT], a2[NT], b[MT];
+#pragma unroll
+    for (int f = 0; f < NT; ++f) {
+      a[f] = load_frag(wrow[f] + k, kv);
+      if (GATED) a2[f] = load_frag(w2row[f] + k, kv);
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) b[t] = load_frag(xrow[t] + k, kv && xvalid[t]);
+#pragma unroll
+    for (int f = 0; f < NT; ++f)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        acc[0][f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[f], b[t], acc[0][f][t], 0, 0, 0);
+        if (GATED)
+          acc[1][f][t] =
+              __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[f], b[t], acc[1][f][t], 0, 0, 0);
+      }
+  }
+
+  // partial sums -> LDS, one wave after the other in wave order (deterministic)
+  for (int w = 0; w < n_waves; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int s = 0; s < SETS; ++s)
+#pragma unroll
+        for (int f = 0; f < NT; ++f)
+#pragma unroll
+          for (int t = 0; t < MT; ++t) {
+            float* dst = red + ((s * NT + f) * MT + t) * 256 + lane * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              if (w == 0) dst[i] = acc[s][f][t][i];
+              else dst[i] += acc[s][f][t][i];
+            }
+          }
+    }
+    __syncthreads();
+  }
+
+  // element (f, t, lane, i) of the accumulator tile is row n_base + f*16 + (lane/16)*4 + i
+  // of W (column of C) and row t*16 + lane%16 of X (row of C)
+  for (int idx = tid; idx < NT * MT * 256; idx += blockDim.x) {
+    const int i = idx % 4, ln = (idx / 4) % 64, ft = idx / 256;
+    const int f = ft / MT, t = ft % MT;
+    const int n = n_base + f * 16 + (ln / 16) * 4 + i;
+    const int m = t * 16 + ln % 16;
+    if (n >= N || m >= M) continue;
+    float v = red[idx];
+    const float v2 = GATED ? red[NT * MT * 256 + idx] : 0.f;
+    if (GATED) v = v2 * (v / (1.0f + expf(-v)));  // set 0 is the gate, set 1 is up
+    const size_t o = (size_t)m * ldc + n;
+    if (out_mode == SK_OUT_BF16)
+      ((bf16_t*)C)[o] = f32_to_bf16(v);
+    else if (out_mode == SK_OUT_F32)
+      ((float*)C)[o] = v;
+    else
+      ((float*)C)[o] += v;
+  }
+}
+
+template <int NT, int MT, bool GATED>
+static int launch_skinny(const bf16_t* X, int ldx, const bf16_t* W, const bf16_t* W2, int ldw,
+                         void* C, int ldc, int out_mode, int M, int N, int K, int waves,
+                         hipStream_t stream) {
+  constexpr int SETS = GATED ? 2 : 1;
+  const size_t smem = (size_t)SETS * NT * MT * 256 * sizeof(float);
+  const int blocks = (N + 16 * NT - 1) / (16 * NT);
+  hipLaunchKernelGGL((skinny_gemm_kernel<NT, MT, GATED>), dim3(blocks), dim3(waves * HAL_WAVE),
+                     smem, stream, X, ldx, W, W2, ldw, C, ldc, out_mode, M, N, K);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// X [M, K] bf16 (M <= 64), W [N, K] bf16, optional W2 [N, K] (gated form: W is the
+// gate's weight, W2 is up's).  out_mode: 0 bf16, 1 float32, 2 add into float32.
+extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const void* W2,
+                                    int ldw, void* C, int ldc, int out_mode, int M, int N, int K,
+                                    hipStream_t stream) {
+  HAL_REQUIRE(M >= 0 && M <= 64, "hal_gemm_bf16_skinny: M=%d (at most 64 rows)", M);
+  HAL_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "hal_gemm_bf16_skinny: N=%d K=%d (K in steps of 8)", N,
+              K);
+  HAL_REQUIRE(ldx >= K && ldw >= K && ldc >= N && ldx % 8 == 0 && ldw % 8 == 0,
+              "hal_gemm_bf16_skinny: leading dimensions %d %d %d", ldx, ldw, ldc);
+  HAL_REQUIRE(out_mode >= 0 && out_mode <= 2, "hal_gemm_bf16_skinny: out_mode %d", out_mode);
+  HAL_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)W2 % 16) == 0,
+              "hal_gemm_bf16_skinny: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  const bf16_t* x = (const bf16_t*)X;
+  const bf16_t* w = (const bf16_t*)W;
+  const bf16_t* w2 = (const bf16_t*)W2;
+  const int mt = (M + 15) / 16;
+  // rows of W per wave grow with the rows of X, so that X is not read more often
+  // than W; the waves of a block split K, more of them when there are few blocks
+  const int nt = mt >= 3 ? 4 : mt;
+  const int blocks = (N + 16 * nt - 1) / (16 * nt);
+  const int steps = (K + 31) / 32;
+  int waves = 4;
+  while (waves < 16 && blocks * waves < 4096 && steps / (waves * 2) >= 8) waves *= 2;
+
+#define SK_CASE(NT_, MT_)                                                                     \
+  if (nt == NT_ && mt == MT_) {                                                               \
+    if (w2)                                                                                   \
+      return launch_skinny<NT_, MT_, true>(x, ldx, w, w2, ldw, C, ldc, out_mode, M, N, K,     \
+                                           waves, stream);                                    \
+    return launch_skinny<NT_, MT_, false>(x, ldx, w, nullptr, ldw, C, ldc, out_mode, M, N, K, \
+                                          waves, stream);                                     \
+  }
+  SK_CASE(1, 1)
+  SK_CASE(2, 2)
+  SK_CASE(4, 3)
+  SK_CASE(4, 4)
+#undef SK_CASE
+  return hal_fail("hal_gemm_bf16_skinny: no kernel for nt=%d mt=%d", nt, mt);
+}

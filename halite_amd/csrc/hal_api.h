@@ -1,0 +1,59 @@
+// The C interface of the kernel library.  Every function launches on the given
+// stream, returns 0 on success and otherwise leaves a message for
+// hal_last_error().  Pointers are device pointers unless a comment says otherwise;
+// dtype codes are HAL_F32 = 0 and HAL_BF16 = 1.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+extern "C" {
+
+const char* hal_last_error();
+int hal_version();
+
+int hal_embedding(const int* ids, const void* table, int table_dtype, float* out, int n_tokens,
+                  int d, int vocab, hipStream_t stream);
+
+int hal_rmsnorm(float* h, const void* delta, const int* rows, const void* w, int w_dtype,
+                float eps, void* out, int dtype, int n_rows, int d, int update_h,
+                hipStream_t stream);
+
+int hal_residual_add(float* h, const void* delta, int dtype, long long n, hipStream_t stream);
+
+int hal_silu_mul(const void* gu, void* out, int dtype, int n_tokens, int F, hipStream_t stream);
+
+int hal_rope_append(void* qkv, int dtype, int row_stride, const int* positions,
+                    const int* token_seg, const int* block_table, int bt_stride,
+                    const float* cos_t, const float* sin_t, int table_len, void* k_pages,
+                    void* v_pages, int n_tokens, int H, int K, int D, int rot, int interleaved,
+                    int page_size, int n_pages, hipStream_t stream);
+
+int hal_attention_simple(const void* q, int q_row_stride, void* out, int out_row_stride,
+                         int dtype, const int* positions, const int* token_seg,
+                         const int* block_table, int bt_stride, const void* k_pages,
+                         const void* v_pages, int n_tokens, int H, int K, int D, int page_size,
+                         int n_pages, float scale, int window, hipStream_t stream);
+
+int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, float* C, int ldc, int M,
+                 int N, int K, hipStream_t stream);
+
+// X [M <= 64, K] bf16, W [N, K] bf16, optional W2 [N, K] (gated: up * silu(gate), W the gate).
+// out_mode: 0 bf16, 1 float32, 2 add into float32.
+int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const void* W2, int ldw, void* C,
+                         int ldc, int out_mode, int M, int N, int K, hipStream_t stream);
+
+int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temperature,
+               const int* top_k, const float* top_p, const float* min_p, const uint64_t* seeds,
+               const int* draw_index, int* out_token, float* out_logprob, hipStream_t stream);
+
+// ---- the head-size-specific library (attention_mfma.hip) ---------------------------------
+int hal_attention_mfma_head_dim();
+int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_stride,
+                       const int* items, const int* n_items, int max_items, const int* merges,
+                       const int* n_merges, int max_merges, const int* seg_q_start,
+                       const int* seg_q_len, const int* seg_kv_len, const int* block_table,
+                       int bt_stride, const void* k_pages, const void* v_pages, float* part_o,
+                       float* part_ml, int H, int K, int head_dim, int page_size, float scale,
+                       int window, hipStream_t stream);
+
+}  // extern "C"

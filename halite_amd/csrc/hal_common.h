@@ -1,0 +1,111 @@
+// Shared device helpers for the gfx950 kernels: element types, conversions,
+// wavefront (64 lanes) and block reductions, and the host-side error record.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#define HAL_WAVE 64
+
+// ---- host-side error record -------------------------------------------------
+// Every entry point returns 0 on success; otherwise it has written a message
+// that hal_last_error() returns.
+extern "C" const char* hal_last_error();
+int hal_fail(const char* fmt, ...);
+
+#define HAL_CHECK_HIP(expr)                                                      \
+  do {                                                                           \
+    hipError_t _e = (expr);                                                      \
+    if (_e != hipSuccess)                                                        \
+      return hal_fail("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e),     \
+                      __FILE__, __LINE__);                                       \
+  } while (0)
+
+#define HAL_REQUIRE(cond, ...)                                                   \
+  do {                                                                           \
+    if (!(cond)) return hal_fail(__VA_ARGS__);                                   \
+  } while (0)
+
+#define HAL_LAUNCH_CHECK() HAL_CHECK_HIP(hipGetLastError())
+
+// ---- element types ------------------------------------------------------------
+// dtype codes shared with the Python side
+enum { HAL_F32 = 0, HAL_BF16 = 1 };
+
+struct bf16_t {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v.bits) << 16);
+}
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  bf16_t r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    r.bits = (uint16_t)((u >> 16) | 0x0040u);
+  } else {
+    u += 0x7fffu + ((u >> 16) & 1u);
+    r.bits = (uint16_t)(u >> 16);
+  }
+  return r;
+}
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return bf16_to_f32(v); }
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float v);
+template <>
+__device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return f32_to_bf16(v); }
+
+// load element i of an array whose element type is given at run time
+__device__ __forceinline__ float load_as_f32(const void* p, int dtype, size_t i) {
+  return dtype == HAL_F32 ? ((const float*)p)[i] : bf16_to_f32(((const bf16_t*)p)[i]);
+}
+
+// ---- reductions -----------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = HAL_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, HAL_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = HAL_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, HAL_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.
+// `scratch` is shared memory for 16 floats.  Safe to call repeatedly with the
+// same scratch.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
+  const int n_waves = (blockDim.x + HAL_WAVE - 1) / HAL_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < n_waves; ++w) total += scratch[w];
+  return total;
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
+  const int n_waves = (blockDim.x + HAL_WAVE - 1) / HAL_WAVE;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = scratch[0];
+  for (int w = 1; w < n_waves; ++w) total = fmaxf(total, scratch[w]);
+  return total;
+}

@@ -1,0 +1,227 @@
+// The sampler: one block per row of float32 logits.
+//   greedy (temperature 0 or top_k 1): first index of the maximum, and its
+//     log-probability under softmax(logits);
+//   otherwise z = logits / temperature, p = softmax(z), the reference's filters
+//     (top-k, top-p, min-p), and the first token, in index order, whose cumulative
+//     kept probability exceeds u * (kept mass).  u comes from a counter-based
+//     generator keyed by (seed, draw index) of the row's request, so a request's
+//     tokens do not depend on what else is in the batch.  The log-probability is
+//     that of the temperature-scaled distribution before filtering.
+// NaN logits count as -1e5.  src/halite/transformers/infer/engine/sampler.py:17-60
+#include "hal_common.h"
+#include "hal_api.h"
+
+#define SAMPLE_THREADS 1024
+
+__device__ __forceinline__ float clean_logit(float x) { return x != x ? -1e5f : x; }
+
+// order-preserving map of a float to an unsigned key
+__device__ __forceinline__ uint32_t sort_key(float x) {
+  const uint32_t u = __float_as_uint(x);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__device__ __forceinline__ float uniform_draw(uint64_t seed, uint32_t index) {
+  uint64_t x = seed * 0x9E3779B97F4A7C15ull + ((uint64_t)index + 1ull) * 0xD1B54A32D192ED03ull;
+  x ^= x >> 30;
+  x *= 0xBF58476D1CE4E5B9ull;
+  x ^= x >> 27;
+  x *= 0x94D049BB133111EBull;
+  x ^= x >> 31;
+  return (float)(x >> 40) * (1.0f / 16777216.0f);
+}
+
+struct ArgMax {
+  float v;
+  int i;
+};
+
+__device__ __forceinline__ ArgMax argmax_merge(ArgMax a, ArgMax b) {
+  if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+  return a;
+}
+
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_kernel(const float* __restrict__ logits, int ld, int V,
+              const float* __restrict__ temperature, const int* __restrict__ top_k,
+              const float* __restrict__ top_p, const float* __restrict__ min_p,
+              const uint64_t* __restrict__ seeds, const int* __restrict__ draw_index,
+              int* __restrict__ out_token, float* __restrict__ out_logprob) {
+  __shared__ float red[16];
+  __shared__ float red2[16];
+  __shared__ ArgMax amax_s[16];
+  __shared__ float chunk_sum[SAMPLE_THREADS];
+  __shared__ int chosen_thread;
+  __shared__ float chosen_before;
+
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
+  const float* x = logits + (size_t)row * ld;
+  const float T = temperature[row];
+  const int k = top_k[row];
+  const bool greedy = (T == 0.f) || (k == 1);
+  const float inv_scale = greedy ? 1.f : T;
+
+  // ---- maximum (and its first index) of z = x / T -----------------------------
+  ArgMax am = {-INFINITY, 0x7fffffff};
+  for (int i = tid; i < V; i += SAMPLE_THREADS) {
+    const ArgMax c = {clean_logit(x[i]) / inv_scale, i};
+    am = argmax_merge(am, c);
+  }
+#pragma unroll
+  for (int off = HAL_WAVE / 2; off > 0; off >>= 1) {
+    ArgMax o;
+    o.v = __shfl_xor(am.v, off, HAL_WAVE);
+    o.i = __shfl_xor(am.i, off, HAL_WAVE);
+    am = argmax_merge(am, o);
+  }
+  if (lane == 0) amax_s[wave] = am;
+  __syncthreads();
+  am = amax_s[0];
+  for (int w = 1; w < SAMPLE_THREADS / HAL_WAVE; ++w) am = argmax_merge(am, amax_s[w]);
+  const float m = am.v;
+
+  // ---- sum of exp(z - m) ---------------------------------------------------------
+  float part = 0.f;
+  for (int i = tid; i < V; i += SAMPLE_THREADS) part += expf(clean_logit(x[i]) / inv_scale - m);
+  const float total = block_sum(part, red);
+
+  if (greedy) {
+    if (tid == 0) {
+      out_token[row] = am.i;
+      out_logprob[row] = -logf(total);  // z_max - m - log(total)
+    }
+    return;
+  }
+
+  // ---- filters: the kept set is { key(z_i) >= key_min } and exp(z_i - m) >= min_p --
+  const float tp = top_p[row];
+  const float mp = min_p[row];
+  uint32_t key_min = 0;
+  float ref_mass = total;
+  if (k > 0 && k < V) {
+    // smallest key with fewer than k elements strictly above it
+    uint32_t lo = 0, hi = 0xffffffffu;  // predicate false below the answer, true at hi
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo) / 2;
+      float cnt = 0.f, mass = 0.f;
+      for (int i = tid; i < V; i += SAMPLE_THREADS) {
+        const float z = clean_logit(x[i]) / inv_scale;
+        if (sort_key(z) > mid) cnt += 1.f;
+      }
+      cnt = block_sum(cnt, red);
+      (void)mass;
+      if (cnt < (float)k) hi = mid; else lo = mid + 1;
+    }
+    key_min = lo;
+    if (mp > 0.f) {
+      // with min_p the reference renormalises after top-k, so top-p refers to
+      // the mass that top-k kept
+      float kept = 0.f;
+      for (int i = tid; i < V; i += SAMPLE_THREADS) {
+        const float z = clean_logit(x[i]) / inv_scale;
+        if (sort_key(z) >= key_min) kept += expf(z - m);
+      }
+      ref_mass = block_sum(kept, red);
+    }
+  }
+  if (tp < 1.f) {
+    // smallest key such that the elements strictly above it hold < top_p of the mass
+    const float thr = tp * ref_mass;
+    uint32_t lo = 0, hi = 0xffffffffu;
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo) / 2;
+      float mass = 0.f;
+      for (int i = tid; i < V; i += SAMPLE_THREADS) {
+        const float z = clean_logit(x[i]) / inv_scale;
+        if (sort_key(z) > mid) mass += expf(z - m);
+      }
+      mass = block_sum(mass, red2);
+      if (mass < thr) hi = mid; else lo = mid + 1;
+    }
+    if (lo > key_min) key_min = lo;
+  }
+
+  // ---- inverse CDF over the kept tokens in index order -----------------------------
+  const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int begin = tid * chunk;
+  const int end = begin + chunk < V ? begin + chunk : V;
+  float mine = 0.f;
+  for (int i = begin; i < end; ++i) {
+    const float z = clean_logit(x[i]) / inv_scale;
+    const float e = expf(z - m);
+    if (sort_key(z) >= key_min && e >= mp) mine += e;
+  }
+  chunk_sum[tid] = mine;
+  __syncthreads();
+  if (tid == 0) {
+    float kept_mass = 0.f;
+    for (int i = 0; i < SAMPLE_THREADS; ++i) kept_mass += chunk_sum[i];
+    const float u = uniform_draw(seeds[row], (uint32_t)draw_index[row]);
+    const float target = u * kept_mass;
+    float run = 0.f;
+    int pick = -1;
+    float before = 0.f;
+    int last_nonempty = 0;
+    float last_before = 0.f;
+    for (int i = 0; i < SAMPLE_THREADS; ++i) {
+      const float c = chunk_sum[i];
+      if (c > 0.f) {
+        last_nonempty = i;
+        last_before = run;
+      }
+      if (pick < 0 && run + c > target && c > 0.f) {
+        pick = i;
+        before = run;
+      }
+      run += c;
+    }
+    if (pick < 0) {  // rounding left the target at the very end
+      pick = last_nonempty;
+      before = last_before;
+    }
+    chosen_thread = pick;
+    chosen_before = before;
+    red2[0] = target;
+  }
+  __syncthreads();
+  if (tid == chosen_thread) {
+    const float target = red2[0];
+    float run = chosen_before;
+    int tok = -1, last_kept = -1;
+    float z_tok = 0.f, z_last = 0.f;
+    for (int i = begin; i < end; ++i) {
+      const float z = clean_logit(x[i]) / inv_scale;
+      const float e = expf(z - m);
+      if (sort_key(z) >= key_min && e >= mp) {
+        run += e;
+        last_kept = i;
+        z_last = z;
+        if (run > target) {
+          tok = i;
+          z_tok = z;
+          break;
+        }
+      }
+    }
+    if (tok < 0) {
+      tok = last_kept;
+      z_tok = z_last;
+    }
+    out_token[row] = tok;
+    out_logprob[row] = z_tok - m - logf(total);
+  }
+}
+
+extern "C" int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temperature,
+                          const int* top_k, const float* top_p, const float* min_p,
+                          const uint64_t* seeds, const int* draw_index, int* out_token,
+                          float* out_logprob, hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "hal_sample: bad sizes rows=%d V=%d ld=%d", n_rows,
+              V, ld);
+  if (n_rows == 0) return 0;
+  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, ld, V,
+                     temperature, top_k, top_p, min_p, seeds, draw_index, out_token, out_logprob);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,212 @@
+"""What one step runs: segments on the host, and their arrays on the device.
+
+A *segment* is the next tokens of one request: a portion of its prompt, cut anywhere,
+or one decoded token.  All segments of a step are one flat batch, as in the
+reference's ``tokainfer`` engine (src/halite/transformers/tokainfer/types.py:521-553;
+tokainfer/engine/input_building.py:138-306): token ids, positions, for every token the
+segment it belongs to, per segment where its queries start and how many keys it has
+after this step, the rows whose logits are wanted, and per cache group the block table
+of the step's requests.  Everything is packed into one int32 buffer and copied to the
+device once.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..kernels import attention as attention_kernels
+
+
+@dataclass
+class Segment:
+    slot: int  # the request's slot in the cache manager
+    start: int  # position of the first token == tokens already cached
+    tokens: np.ndarray  # int32
+    want: list[int] = field(default_factory=list)  # indices into tokens
+
+    def __post_init__(self):
+        self.tokens = np.asarray(self.tokens, dtype=np.int32).reshape(-1)
+
+
+@dataclass
+class GroupStep:
+    group_id: int
+    page_size: int
+    window: int | None
+    block_table: torch.Tensor  # [S, P] int32 on the device
+    block_table_host: np.ndarray
+
+
+class _Staging:
+    """A ring of pinned host buffers for the per-step copy."""
+
+    def __init__(self, device, n=4):
+        self.device = device
+        self.bufs = [None] * n
+        self.events = [None] * n
+        self.i = 0
+
+    def upload(self, flat: np.ndarray) -> torch.Tensor:
+        i = self.i
+        self.i = (self.i + 1) % len(self.bufs)
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        n = flat.size
+        if self.bufs[i] is None or self.bufs[i].numel() < n:
+            self.bufs[i] = torch.empty(max(n, 4096) * 2, dtype=torch.int32, pin_memory=True)
+        self.bufs[i][:n].numpy()[:] = flat
+        dev = self.bufs[i][:n].to(self.device, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self.events[i] = ev
+        return dev
+
+
+class _Packer:
+    def __init__(self):
+        self.parts = []
+        self.offsets = {}
+        self.n = 0
+
+    def add(self, name, arr):
+        arr = np.ascontiguousarray(arr, dtype=np.int32).reshape(-1)
+        pad = (-arr.size) % 4  # keep every piece 16-byte aligned
+        self.offsets[name] = (self.n, arr.size)
+        self.parts.append(arr)
+        if pad:
+            self.parts.append(np.zeros(pad, dtype=np.int32))
+        self.n += arr.size + pad
+
+    def flat(self):
+        return np.concatenate(self.parts) if self.parts else np.zeros(0, dtype=np.int32)
+
+
+class StepContext:
+    """The device-side view of a step that the parts compute on."""
+
+    def __init__(self, segments: list[Segment], cache, device, staging: _Staging | None = None):
+        self.device = torch.device(device)
+        self.segments = segments
+        self.cache = cache
+        S = len(segments)
+        self.n_segs = S
+        lens = np.array([s.tokens.size for s in segments], dtype=np.int32)
+        starts = np.array([s.start for s in segments], dtype=np.int32)
+        self.seg_q_len_host = lens
+        self.seg_pos0_host = starts
+        self.seg_kv_len_host = starts + lens
+        self.seg_q_start_host = np.concatenate(([0], np.cumsum(lens)[:-1])).astype(np.int32)
+        self.seg_slot_host = np.array([s.slot for s in segments], dtype=np.int32)
+        T = int(lens.sum())
+        self.n_tokens = T
+        tokens = np.concatenate([s.tokens for s in segments]) if S else np.zeros(0, np.int32)
+        seg_of = np.repeat(np.arange(S, dtype=np.int32), lens)
+        positions = np.arange(T, dtype=np.int32) - np.repeat(self.seg_q_start_host, lens) + np.repeat(starts, lens)
+        rows = []
+        for s, q0 in zip(segments, self.seg_q_start_host):
+            for w in s.want:
+                if not 0 <= w < s.tokens.size:
+                    raise ValueError(f"wanted row {w} outside a segment of {s.tokens.size} tokens")
+                rows.append(int(q0) + w)
+        self.n_logit_rows = len(rows)
+        self.max_position = int(self.seg_kv_len_host.max()) - 1 if S else 0
+        self.positions_host = positions
+        self.token_seg_host = seg_of
+
+        pk = _Packer()
+        pk.add("tokens", tokens)
+        pk.add("positions", positions)
+        pk.add("token_seg", seg_of)
+        pk.add("token_slot", np.repeat(self.seg_slot_host, lens))
+        pk.add("logit_rows", np.array(rows, dtype=np.int32))
+        pk.add("seg_q_start", self.seg_q_start_host)
+        pk.add("seg_q_len", lens)
+        pk.add("seg_kv_len", self.seg_kv_len_host)
+        slots = [s.slot for s in segments]
+        tables = {}
+        for g in cache.groups:
+            bt = cache.block_table(g.group_id, slots)
+            tables[g.group_id] = bt
+            pk.add(f"bt{g.group_id}", bt)
+        self._packer = pk
+        self._plans: dict = {}
+        self._plan_host: dict = {}
+        self._tables_host = tables
+        self._staging = staging
+        self._dev = None
+        self._groups: dict[int, GroupStep] = {}
+        self.empty_f32 = None
+
+    # The plans of the attention kernel are part of the same upload, so they are
+    # declared before the first device access.
+    def plan_attention(self, group_id: int, n_heads: int, n_kv_heads: int, window: int, late=False) -> None:
+        key = (group_id, n_heads // n_kv_heads, window)
+        if key in self._plan_host:
+            return
+        if self._dev is not None and not late:
+            return
+        plan = attention_kernels.plan_items(
+            self.seg_q_len_host, self.seg_kv_len_host, n_heads // n_kv_heads, n_kv_heads, window
+        )
+        self._plan_host[key] = plan
+        plan.name = f"plan{len(self._plan_host)}"
+        counts = np.array([plan.n_items, plan.n_merges], dtype=np.int32)
+        if self._dev is None:
+            self._packer.add(plan.name + "_items", plan.items)
+            self._packer.add(plan.name + "_merges", plan.merges)
+            self._packer.add(plan.name + "_counts", counts)
+        else:  # declared after the step's upload: a copy of its own
+            dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(self.device)
+            self._plans[key] = (plan, dev(plan.items), dev(plan.merges), dev(counts))
+
+    def _upload(self):
+        if self._dev is not None:
+            return
+        flat = self._packer.flat()
+        if self._staging is not None and self.device.type == "cuda":
+            self._dev = self._staging.upload(flat)
+        else:
+            self._dev = torch.from_numpy(flat).to(self.device)
+        self.empty_f32 = torch.empty((0, 0), dtype=torch.float32, device=self.device)
+
+    def _view(self, name) -> torch.Tensor:
+        self._upload()
+        off, n = self._packer.offsets[name]
+        return self._dev[off : off + n]
+
+    tokens = property(lambda self: self._view("tokens"))
+    positions = property(lambda self: self._view("positions"))
+    token_seg = property(lambda self: self._view("token_seg"))
+    token_slot = property(lambda self: self._view("token_slot"))
+    logit_rows = property(lambda self: self._view("logit_rows"))
+    seg_q_start = property(lambda self: self._view("seg_q_start"))
+    seg_q_len = property(lambda self: self._view("seg_q_len"))
+    seg_kv_len = property(lambda self: self._view("seg_kv_len"))
+
+    def group(self, group_id: int) -> GroupStep:
+        if group_id not in self._groups:
+            host = self._tables_host[group_id]
+            g = self.cache.groups[group_id]
+            self._groups[group_id] = GroupStep(
+                group_id, g.page_size, g.need.window, self._view(f"bt{group_id}").view(host.shape), host
+            )
+        return self._groups[group_id]
+
+    def attention(self, q, q_row_stride, kv, group: GroupStep, n_heads, scale, window) -> torch.Tensor:
+        """Attention of every token of the step over its request's cached keys."""
+        return attention_kernels.paged_attention(self, q, q_row_stride, kv, group, n_heads, scale, window)
+
+    def device_plan(self, group_id: int, group_size: int, window: int):
+        key = (group_id, group_size, window)
+        plan = self._plan_host.get(key)
+        if plan is None:
+            return None
+        if key not in self._plans:
+            items = self._view(plan.name + "_items").view(-1, 8)
+            merges = self._view(plan.name + "_merges").view(-1, 4)
+            counts = self._view(plan.name + "_counts")
+            self._plans[key] = (plan, items, merges, counts)
+        return self._plans[key]

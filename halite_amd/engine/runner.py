@@ -1,0 +1,168 @@
+"""The step function and what it owns: the model, the cache manager, the staging.
+
+``ModelRunner.step`` takes a batch of (request slot, its next tokens, the places whose
+logits are wanted), portions of prompts beside single decoded tokens, cut anywhere; it
+runs exactly those tokens as one batch from the cache that earlier steps left, and
+returns float32 logits at the wanted places.  The reference has one runner per engine
+(src/halite/transformers/infer/engine/model_runner.py:14-252) with separate extend and
+decode passes; the mixed flat batch is the ``tokainfer`` engine's
+(src/halite/transformers/tokainfer/basic_worker.py:56-174).
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager
+from ..config.engine import ModelConfig, ServerConfig
+from ..config.registry import read_config
+from ..parts.decoder import Decoder
+from ..weights import fill_random, load_weights
+from .batch import Segment, StepContext, _Staging
+
+_TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+class StepError(ValueError):
+    pass
+
+
+def require_gpu(device) -> torch.device:
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError(
+            "halite_amd runs on an AMD GPU through its HIP kernels only; no GPU is visible "
+            f"(device {device}) and there is no CPU path"
+        )
+    return device
+
+
+class ModelRunner:
+    def __init__(
+        self,
+        model: Decoder,
+        server_config: ServerConfig | None = None,
+        model_config: ModelConfig | None = None,
+    ):
+        self.model = model
+        self.server_config = server_config or ServerConfig()
+        self.model_config = model_config or ModelConfig(
+            dtype="float32" if model.dtype == torch.float32 else "bfloat16"
+        )
+        self.device = model.device
+        spec = model.spec
+        self.context_len = min(self.model_config.context_len or spec.max_positions, spec.max_positions)
+        self.vocab_size = spec.vocab_size
+
+        needs, borrowed, state_needs = {}, {}, {}
+        for i, run in enumerate(spec.order):
+            mixer = model.mixer_of_run(i)
+            need = mixer.cache_need()
+            if need is not None:
+                if run.cache_from is None:
+                    needs[i] = need
+                else:
+                    borrowed[i] = run.cache_from
+            st = mixer.state_need()
+            if st:
+                state_needs[i] = st
+        page_size = self.server_config.page_size
+        n_slots = self.server_config.max_seqs_per_forward
+        num_pages = self._size_pool(needs, page_size, model.dtype)
+        self.cache = CacheManager(
+            needs, borrowed, state_needs, page_size=page_size, num_pages=num_pages,
+            n_slots=n_slots, dtype=model.dtype, device=self.device,
+        )
+        for run in model.runs:
+            run.kv = self.cache.layer_pages(run.index)
+            run.state = self.cache.state_of_run(run.index)
+        self._staging = _Staging(self.device) if self.device.type == "cuda" else None
+        self.max_total_tokens = self.cache.token_capacity
+
+    def _size_pool(self, needs, page_size, dtype) -> int:
+        tokens = self.server_config.kv_cache_num_tokens
+        if tokens is not None:
+            return -(-tokens // page_size) + 1
+        if not needs:
+            return 2
+        # src/halite/transformers/infer/engine/model_runner.py:117-131
+        free, total = torch.cuda.mem_get_info(self.device)
+        usable = free - total * (1 - self.model_config.memory_fraction_static)
+        per_page = CacheManager.bytes_per_page(needs, page_size, dtype)
+        pages = int(usable // per_page)
+        if pages < 2:
+            raise RuntimeError("no device memory is left for the cache pool")
+        # a request never holds more than context_len tokens; cap the pool at what
+        # max_seqs_per_forward requests of that length could use
+        cap = self.server_config.max_seqs_per_forward * (-(-self.context_len // page_size)) + 1
+        return min(pages, cap)
+
+    # -- construction -------------------------------------------------------------
+    @classmethod
+    def from_pretrained(cls, folder: str, server_config=None, model_config=None) -> "ModelRunner":
+        model_config = model_config or ModelConfig()
+        device = require_gpu(f"{model_config.device}:{model_config.gpu_id}" if model_config.device == "cuda" else model_config.device)
+        arch, cfg = read_config(folder)
+        model = Decoder(arch.to_spec(cfg), _TORCH_DTYPE[model_config.dtype], device)
+        load_weights(model, arch.weight_map(cfg), folder)
+        runner = cls(model, server_config, model_config)
+        runner.arch, runner.config = arch, cfg
+        return runner
+
+    @classmethod
+    def from_random(cls, cfg, seed: int, server_config=None, model_config=None, arch=None) -> "ModelRunner":
+        from ..config.registry import get_architecture
+
+        model_config = model_config or ModelConfig()
+        device = require_gpu(f"{model_config.device}:{model_config.gpu_id}" if model_config.device == "cuda" else model_config.device)
+        arch = arch or get_architecture(cfg.architectures[0])
+        model = Decoder(arch.to_spec(cfg), _TORCH_DTYPE[model_config.dtype], device)
+        fill_random(model, seed)
+        runner = cls(model, server_config, model_config)
+        runner.arch, runner.config = arch, cfg
+        return runner
+
+    # -- requests -------------------------------------------------------------------
+    def admit(self) -> int:
+        return self.cache.admit()
+
+    def free(self, slot: int) -> None:
+        self.cache.free(slot)
+
+    # -- the step ---------------------------------------------------------------------
+    def check_segments(self, segments: list[Segment]) -> None:
+        seen = set()
+        for s in segments:
+            if s.slot in seen:
+                raise StepError(f"slot {s.slot} appears twice in one step")
+            seen.add(s.slot)
+            n = s.tokens.size
+            if n == 0:
+                raise StepError(f"slot {s.slot}: an entry without tokens")
+            have = self.cache.length(s.slot)
+            if s.start != have:
+                raise StepError(f"slot {s.slot}: tokens start at {s.start} but {have} are cached")
+            if s.start + n > self.context_len:
+                raise StepError(f"slot {s.slot}: {s.start + n} tokens exceed the context length {self.context_len}")
+            lo, hi = int(s.tokens.min()), int(s.tokens.max())
+            if lo < 0 or hi >= self.vocab_size:
+                raise StepError(f"slot {s.slot}: token id {lo if lo < 0 else hi} outside the vocabulary of {self.vocab_size}")
+
+    @torch.no_grad()
+    def step(self, segments: list[Segment]) -> torch.Tensor:
+        """Runs the tokens of ``segments`` and returns float32 logits
+        ``[wanted rows, vocab]`` in the order of the segments and of their ``want``.
+        Raises ``NoSpace`` (and changes nothing) if the pages do not suffice."""
+        if not segments:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        self.check_segments(segments)
+        spans = [(s.slot, s.start + s.tokens.size) for s in segments]
+        self.cache.reserve(spans)
+        ctx = StepContext(segments, self.cache, self.device, self._staging)
+        for run in self.model.runs:
+            self.model.mixer_of_run(run.index).prepare(ctx, run)
+        logits = self.model.forward(ctx)
+        for slot, new_len in spans:
+            self.cache.advance(slot, new_len)
+        return logits

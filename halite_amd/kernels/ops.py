@@ -1,0 +1,333 @@
+"""Typed Python wrappers of the kernel library's entry points.
+
+Each wrapper checks on the host what its kernel assumes (device, dtype, layout,
+shapes) before it launches on torch's current stream; a failed check or a failed
+launch raises ``KernelError``.  There is no other implementation behind these
+functions: without a GPU and the built library they raise.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import library
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16, not {dtype}") from None
+
+
+def _ptr(t: torch.Tensor | None):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, msg: str):
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*tensors):
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel arguments must be on the GPU")
+            _need(t.is_contiguous(), "kernel arguments must be contiguous")
+
+
+def _check(lib, rc: int):
+    if rc != 0:
+        raise KernelError(lib.hal_last_error().decode())
+
+
+def _i32(t: torch.Tensor | None, name: str):
+    if t is not None:
+        _need(t.dtype == torch.int32, f"{name} must be int32")
+
+
+# --------------------------------------------------------------------------------
+
+
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None):
+    """``out[t] = table[ids[t]]`` as float32."""
+    lib = library.core_library()
+    _dev(ids, table, out)
+    _i32(ids, "ids")
+    n, (vocab, d) = ids.numel(), table.shape
+    if out is None:
+        out = torch.empty((n, d), dtype=torch.float32, device=table.device)
+    _need(out.dtype == torch.float32 and out.shape == (n, d), "embedding: bad output")
+    _check(
+        lib,
+        lib.hal_embedding(_ptr(ids), _ptr(table), dtype_code(table.dtype), _ptr(out), n, d, vocab, _stream()),
+    )
+    return out
+
+
+def rmsnorm(
+    h: torch.Tensor,
+    weight: torch.Tensor,
+    eps: float,
+    out_dtype: torch.dtype,
+    delta: torch.Tensor | None = None,
+    rows: torch.Tensor | None = None,
+    update_h: bool = True,
+):
+    """RMSNorm of the float32 stream ``h`` (+ ``delta``), optionally only of
+    ``rows``; with ``delta`` and ``update_h`` the sum is written back to ``h``."""
+    lib = library.core_library()
+    _dev(h, weight, delta, rows)
+    _i32(rows, "rows")
+    _need(h.dtype == torch.float32 and h.dim() == 2, "rmsnorm: the stream is float32 [T, d]")
+    n_tokens, d = h.shape
+    _need(weight.shape == (d,), f"rmsnorm: weight {tuple(weight.shape)} for width {d}")
+    if delta is not None:
+        _need(delta.shape == h.shape and delta.dtype == out_dtype, "rmsnorm: bad delta")
+    n_rows = n_tokens if rows is None else rows.numel()
+    if rows is not None:
+        update_h = False
+    out = torch.empty((n_rows, d), dtype=out_dtype, device=h.device)
+    _check(
+        lib,
+        lib.hal_rmsnorm(
+            _ptr(h), _ptr(delta), _ptr(rows), _ptr(weight), dtype_code(weight.dtype),
+            ctypes.c_float(eps), _ptr(out), dtype_code(out_dtype), n_rows, d,
+            1 if (update_h and delta is not None) else 0, _stream(),
+        ),
+    )
+    return out
+
+
+def residual_add(h: torch.Tensor, delta: torch.Tensor):
+    lib = library.core_library()
+    _dev(h, delta)
+    _need(h.dtype == torch.float32 and delta.shape == h.shape, "residual_add: bad shapes")
+    _check(
+        lib,
+        lib.hal_residual_add(_ptr(h), _ptr(delta), dtype_code(delta.dtype), ctypes.c_longlong(h.numel()), _stream()),
+    )
+    return h
+
+
+def silu_mul(gate_up: torch.Tensor):
+    """``up * silu(gate)`` of rows ``[gate | up]``."""
+    lib = library.core_library()
+    _dev(gate_up)
+    n, two_f = gate_up.shape
+    _need(two_f % 2 == 0, "silu_mul: odd row length")
+    out = torch.empty((n, two_f // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _check(
+        lib,
+        lib.hal_silu_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), n, two_f // 2, _stream()),
+    )
+    return out
+
+
+def rope_append(
+    qkv: torch.Tensor,
+    positions: torch.Tensor,
+    cos: torch.Tensor,
+    sin: torch.Tensor,
+    n_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    rotary_dim: int,
+    interleaved: bool,
+    token_seg: torch.Tensor | None = None,
+    block_table: torch.Tensor | None = None,
+    k_pages: torch.Tensor | None = None,
+    v_pages: torch.Tensor | None = None,
+    page_size: int = 0,
+):
+    """Rotate q and k in place in the packed rows ``[q | k | v]`` and append k and
+    v to the pages (``n_kv_heads == 0``: rows hold q only, nothing is appended)."""
+    lib = library.core_library()
+    _dev(qkv, positions, cos, sin, token_seg, block_table, k_pages, v_pages)
+    _i32(positions, "positions"), _i32(token_seg, "token_seg"), _i32(block_table, "block_table")
+    n = qkv.shape[0]
+    _need(positions.numel() == n, "rope_append: one position per row")
+    _need(cos.dtype == torch.float32 and sin.dtype == torch.float32, "rope tables are float32")
+    _need(rotary_dim == 0 or (cos.shape[1] == rotary_dim // 2 and cos.shape == sin.shape), "rope table width")
+    n_pages = 0
+    if n_kv_heads > 0:
+        _need(k_pages is not None and v_pages is not None and block_table is not None, "rope_append: no cache")
+        _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "cache dtype != activation dtype")
+        n_pages = k_pages.shape[0]
+        _need(
+            k_pages.shape == (n_pages, n_kv_heads, page_size, head_dim)
+            and v_pages.shape == (n_pages, n_kv_heads, head_dim, page_size),
+            "rope_append: page shapes",
+        )
+        _need(token_seg.numel() == n and block_table.dim() == 2, "rope_append: segment arrays")
+    _check(
+        lib,
+        lib.hal_rope_append(
+            _ptr(qkv), dtype_code(qkv.dtype), qkv.shape[1], _ptr(positions), _ptr(token_seg),
+            _ptr(block_table), 0 if block_table is None else block_table.shape[1],
+            _ptr(cos), _ptr(sin), cos.shape[0], _ptr(k_pages), _ptr(v_pages),
+            n, n_heads, n_kv_heads, head_dim, rotary_dim, 1 if interleaved else 0,
+            page_size, n_pages, _stream(),
+        ),
+    )
+
+
+def attention_simple(
+    q: torch.Tensor,
+    q_row_stride: int,
+    positions: torch.Tensor,
+    token_seg: torch.Tensor,
+    block_table: torch.Tensor,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    n_heads: int,
+    scale: float,
+    window: int = 0,
+):
+    """Paged attention, one wavefront per (token, head); ``q`` holds the query
+    heads at the start of rows of ``q_row_stride`` elements."""
+    lib = library.core_library()
+    _dev(q, positions, token_seg, block_table, k_pages, v_pages)
+    _i32(positions, "positions"), _i32(token_seg, "token_seg"), _i32(block_table, "block_table")
+    n = positions.numel()
+    n_pages, n_kv, page_size, head_dim = k_pages.shape
+    _need(v_pages.shape == (n_pages, n_kv, head_dim, page_size), "attention: page shapes")
+    _need(k_pages.dtype == q.dtype and v_pages.dtype == q.dtype, "attention: cache dtype")
+    _need(q.numel() >= n * q_row_stride and q_row_stride >= n_heads * head_dim, "attention: q rows")
+    out = torch.empty((n, n_heads * head_dim), dtype=q.dtype, device=q.device)
+    _check(
+        lib,
+        lib.hal_attention_simple(
+            _ptr(q), q_row_stride, _ptr(out), n_heads * head_dim, dtype_code(q.dtype),
+            _ptr(positions), _ptr(token_seg), _ptr(block_table), block_table.shape[1],
+            _ptr(k_pages), _ptr(v_pages), n, n_heads, n_kv, head_dim, page_size, n_pages,
+            ctypes.c_float(scale), window, _stream(),
+        ),
+    )
+    return out
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor):
+    """``a @ w.T`` in true float32 (``a`` [M, K], ``w`` [N, K])."""
+    lib = library.core_library()
+    _dev(a, w)
+    _need(a.dtype == torch.float32 and w.dtype == torch.float32, "gemm_f32 takes float32")
+    m, k = a.shape
+    n, k2 = w.shape
+    _need(k == k2, f"gemm_f32: inner sizes {k} and {k2}")
+    out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    _check(lib, lib.hal_gemm_f32(_ptr(a), k, _ptr(w), k, _ptr(out), n, m, n, k, _stream()))
+    return out
+
+
+def sample(
+    logits: torch.Tensor,
+    temperature: torch.Tensor,
+    top_k: torch.Tensor,
+    top_p: torch.Tensor,
+    min_p: torch.Tensor,
+    seeds: torch.Tensor,
+    draw_index: torch.Tensor,
+):
+    """Next token and log-probability of every row of float32 ``logits``."""
+    lib = library.core_library()
+    _dev(logits, temperature, top_k, top_p, min_p, seeds, draw_index)
+    n, vocab = logits.shape
+    _need(logits.dtype == torch.float32, "sample: logits are float32")
+    _need(temperature.dtype == torch.float32 and top_p.dtype == torch.float32 and min_p.dtype == torch.float32, "sample: float parameters")
+    _i32(top_k, "top_k"), _i32(draw_index, "draw_index")
+    _need(seeds.dtype == torch.int64, "sample: seeds are int64")
+    for t in (temperature, top_k, top_p, min_p, seeds, draw_index):
+        _need(t.numel() == n, "sample: one parameter per row")
+    tokens = torch.empty(n, dtype=torch.int32, device=logits.device)
+    logprobs = torch.empty(n, dtype=torch.float32, device=logits.device)
+    _check(
+        lib,
+        lib.hal_sample(
+            _ptr(logits), vocab, n, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(min_p),
+            _ptr(seeds), _ptr(draw_index), _ptr(tokens), _ptr(logprobs), _stream(),
+        ),
+    )
+    return tokens, logprobs
+
+
+SKINNY_MAX_ROWS = 64
+
+
+def gemm_bf16_skinny(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    w_up: torch.Tensor | None = None,
+    out_dtype: torch.dtype = torch.bfloat16,
+    add_to: torch.Tensor | None = None,
+):
+    """``x @ w.T`` for at most 64 rows of bf16 ``x``; with ``w_up`` the gated form
+    ``(x @ w_up.T) * silu(x @ w.T)``; ``add_to`` (float32) receives ``+=``."""
+    lib = library.core_library()
+    _dev(x, add_to)
+    for t in (w, w_up):
+        if t is not None:
+            _need(t.is_cuda and t.dtype == torch.bfloat16 and t.stride(1) == 1, "skinny gemm: weight layout")
+    _need(x.dtype == torch.bfloat16, "skinny gemm takes bf16")
+    m, k = x.shape
+    n, k2 = w.shape
+    _need(k == k2 and (w_up is None or (w_up.shape == w.shape and w_up.stride(0) == w.stride(0))), "skinny gemm: shapes")
+    _need(m <= SKINNY_MAX_ROWS, f"skinny gemm: {m} rows")
+    if add_to is not None:
+        _need(add_to.dtype == torch.float32 and add_to.shape == (m, n), "skinny gemm: add_to")
+        out, mode = add_to, 2
+    else:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        mode = 0 if out_dtype == torch.bfloat16 else 1
+        _need(out_dtype in (torch.bfloat16, torch.float32), "skinny gemm: output dtype")
+    _check(
+        lib,
+        lib.hal_gemm_bf16_skinny(
+            _ptr(x), k, _ptr(w), _ptr(w_up), w.stride(0), _ptr(out), n, mode, m, n, k, _stream()
+        ),
+    )
+    return out
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``x @ w.T`` for a weight ``[out, in]``.
+
+    float32 weights: the true 32-bit kernel (activations are widened if needed).
+    bf16 weights: the hand-written kernel for up to 64 rows; for more rows the
+    library product that the reference itself uses for its linear layers
+    (src/halite/transformers/infer/attention.py:21-24), except where float32
+    output is asked for, which the hand-written kernel gives in passes of 64 rows.
+    """
+    out_dtype = out_dtype or x.dtype
+    if w.dtype == torch.float32:
+        y = gemm_f32(x if x.dtype == torch.float32 else x.float(), w)
+        return y if out_dtype == torch.float32 else y.to(out_dtype)
+    _need(w.dtype == torch.bfloat16, f"linear: weight dtype {w.dtype}")
+    if x.dtype != torch.bfloat16:
+        x = x.to(torch.bfloat16)
+    m, k = x.shape
+    skinny_ok = k % 8 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
+    if skinny_ok and m <= SKINNY_MAX_ROWS:
+        return gemm_bf16_skinny(x, w, out_dtype=out_dtype)
+    if out_dtype == torch.float32 and skinny_ok:
+        out = torch.empty((m, w.shape[0]), dtype=torch.float32, device=x.device)
+        for r0 in range(0, m, SKINNY_MAX_ROWS):
+            out[r0 : r0 + SKINNY_MAX_ROWS] = gemm_bf16_skinny(
+                x[r0 : r0 + SKINNY_MAX_ROWS], w, out_dtype=torch.float32
+            )
+        return out
+    y = torch.matmul(x, w.t())
+    return y if out_dtype == torch.bfloat16 else y.to(out_dtype)

@@ -1,0 +1,31 @@
+from . import attention, block, embedding, feedforward, norm, rope  # noqa: F401
+from .base import (
+    ARRANGEMENTS,
+    EMBEDDINGS,
+    FEED_FORWARDS,
+    HEADS,
+    MIXERS,
+    NORMS,
+    POSITIONS,
+    BuildContext,
+    Embedding,
+    FeedForward,
+    Head,
+    Mixer,
+    Norm,
+    PagedKVNeed,
+    ParamDecl,
+    Part,
+    PositionEncoding,
+    RunBinding,
+    StateNeed,
+    register_arrangement,
+)
+from .decoder import Decoder
+
+__all__ = [
+    "ARRANGEMENTS", "EMBEDDINGS", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITIONS",
+    "BuildContext", "Decoder", "Embedding", "FeedForward", "Head", "Mixer", "Norm",
+    "PagedKVNeed", "ParamDecl", "Part", "PositionEncoding", "RunBinding", "StateNeed",
+    "register_arrangement",
+]

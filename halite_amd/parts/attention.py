@@ -1,0 +1,105 @@
+"""Grouped-query self-attention over the paged cache
+(src/halite/transformers/infer/attention.py:20-172)."""
+
+from __future__ import annotations
+
+import torch
+from pydantic import BaseModel, Field, StrictInt, model_validator
+
+from ..kernels import attention as attention_kernels
+from ..kernels import ops
+from .base import MIXERS, Mixer, PagedKVNeed, ParamDecl
+
+
+class AttentionParams(BaseModel):
+    hidden_size: StrictInt = Field(gt=0)
+    n_heads: StrictInt = Field(gt=0)
+    n_kv_heads: StrictInt = Field(gt=0)
+    head_dim: StrictInt = Field(gt=0)
+    scale: float = Field(gt=0)
+    position: str | None = None
+    window: StrictInt | None = Field(default=None, gt=0)
+
+    @model_validator(mode="after")
+    def _check(self):
+        if self.n_heads % self.n_kv_heads:
+            raise ValueError(f"{self.n_heads} heads are not a multiple of {self.n_kv_heads} kv heads")
+        return self
+
+
+@MIXERS.register("attention")
+class Attention(Mixer):
+    """q, k, v projections (separate weights, one packed tensor), rotation of q and
+    k, append of k and v to the run's pages, attention of every token over the keys
+    of its request up to itself (and no further back than ``window``), output
+    projection.  Query head ``h`` reads key/value head ``h // (H/K)``.
+    """
+
+    Params = AttentionParams
+
+    def __init__(self, params, build):
+        super().__init__(params, build)
+        self.position = None
+        if params.position is not None:
+            if params.position not in build.positions:
+                raise ValueError(f"attention names position encoding {params.position!r}, which the model does not define")
+            self.position = build.positions[params.position]
+            if self.position.p.head_dim != params.head_dim:
+                raise ValueError("position encoding and attention disagree on head_dim")
+
+    def param_decls(self):
+        p = self.p
+        return {
+            "q.weight": ParamDecl((p.n_heads * p.head_dim, p.hidden_size)),
+            "k.weight": ParamDecl((p.n_kv_heads * p.head_dim, p.hidden_size)),
+            "v.weight": ParamDecl((p.n_kv_heads * p.head_dim, p.hidden_size)),
+            "out.weight": ParamDecl((p.hidden_size, p.n_heads * p.head_dim)),
+        }
+
+    def allocate(self, dtypes):
+        p = self.p
+        if len({dtypes["q.weight"], dtypes["k.weight"], dtypes["v.weight"]}) != 1:
+            raise ValueError("q, k and v weights are stored with different element types")
+        nq, nk = p.n_heads * p.head_dim, p.n_kv_heads * p.head_dim
+        dev = self.build.device
+        self.w_qkv = torch.empty((nq + 2 * nk, p.hidden_size), dtype=dtypes["q.weight"], device=dev)
+        self.w_out = torch.empty((p.hidden_size, nq), dtype=dtypes["out.weight"], device=dev)
+        return {
+            "q.weight": self.w_qkv[:nq],
+            "k.weight": self.w_qkv[nq : nq + nk],
+            "v.weight": self.w_qkv[nq + nk :],
+            "out.weight": self.w_out,
+        }
+
+    def cache_need(self):
+        return PagedKVNeed(self.p.n_kv_heads, self.p.head_dim, self.p.window)
+
+    def prepare(self, ctx, run):
+        group = ctx.cache.groups[run.kv.group_id]
+        if attention_kernels.mfma_supported(self.build.dtype, self.p.head_dim, group.page_size):
+            ctx.plan_attention(group.group_id, self.p.n_heads, self.p.n_kv_heads, self.p.window or 0)
+
+    def forward(self, x, ctx, run):
+        p = self.p
+        kv = run.kv
+        group = ctx.group(kv.group_id)
+        n_q = p.n_heads * p.head_dim
+        if run.appends:
+            qkv = ops.linear(x, self.w_qkv)
+            n_kv_append = p.n_kv_heads
+        else:  # the keys and values are an earlier run's
+            qkv = ops.linear(x, self.w_qkv[:n_q])
+            n_kv_append = 0
+        if self.position is not None:
+            cos, sin = self.position.tables(ctx.max_position + 1)
+            rot, interleaved = self.position.rotary_dim, self.position.interleaved
+        else:
+            cos = sin = ctx.empty_f32
+            rot, interleaved = 0, False
+        ops.rope_append(
+            qkv, ctx.positions, cos, sin, p.n_heads, n_kv_append, p.head_dim, rot, interleaved,
+            token_seg=ctx.token_seg, block_table=group.block_table,
+            k_pages=kv.k, v_pages=kv.v, page_size=group.page_size,
+        )
+        out = ctx.attention(qkv, qkv.shape[1], kv, group, p.n_heads, p.scale, p.window or 0)
+        return ops.linear(out, self.w_out)

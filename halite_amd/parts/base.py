@@ -1,0 +1,193 @@
+"""What every part of a model is, and the registries that hold the kinds of parts.
+
+A part (mixer, feed-forward, norm, position encoding, embedding, head) is built from
+its own validated parameters and a ``BuildContext``; it declares the tensors it owns,
+what cache and what fixed-size per-request state it needs, and computes on the tokens
+of one step.  No part knows which model it is in: the reference composes its blocks
+the same way from interchangeable modules (configs/models/transformer.py:55-196).
+
+Registering a new kind is one decorator; the model builder looks kinds up by the
+``kind`` string of a ``PartSpec``.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import TYPE_CHECKING, Any, ClassVar
+
+import torch
+from pydantic import BaseModel, ValidationError
+
+from ..config.registry import ConfigError
+from ..config.spec import PartSpec
+
+if TYPE_CHECKING:
+    from ..engine.batch import StepContext
+
+
+@dataclass(frozen=True)
+class ParamDecl:
+    """A tensor that a part owns.  ``init`` is what the random-weights mode does
+    with it: ``normal`` (N(0, std) from the seed) or ``ones``."""
+
+    shape: tuple[int, ...]
+    init: str = "normal"
+    integer: bool = False
+
+
+@dataclass(frozen=True)
+class PagedKVNeed:
+    """Keys and values of every token, kept in pages.  Runs whose needs are equal
+    share one group of pages; ``window`` (tokens a query looks back, itself
+    included) lets pages be given back once every later query has passed them."""
+
+    n_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """State of fixed size that a request keeps between steps, one row per live
+    request, zero when the request is admitted."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class BuildContext:
+    dtype: torch.dtype  # element type of activations and cache
+    device: torch.device
+    hidden_size: int
+    positions: dict[str, "Part"] = field(default_factory=dict)
+
+
+@dataclass
+class RunBinding:
+    """What one entry of the run order is bound to at run time."""
+
+    index: int
+    kv: Any = None  # cache.pages.LayerPages of this run (own or borrowed), or None
+    appends: bool = True  # False: the cache belongs to an earlier run
+    state: dict[str, torch.Tensor] = field(default_factory=dict)  # [n_slots, *shape]
+
+
+class Part:
+    """Base of all parts."""
+
+    Params: ClassVar[type[BaseModel]]
+
+    def __init__(self, params: BaseModel, build: BuildContext):
+        self.p = params
+        self.build = build
+
+    # -- declarations ---------------------------------------------------------
+    def param_decls(self) -> dict[str, ParamDecl]:
+        return {}
+
+    def allocate(self, dtypes: dict[str, torch.dtype]) -> dict[str, torch.Tensor]:
+        """Creates the part's tensors on the device with the given element types
+        and returns, for every name of ``param_decls``, the tensor (or the view
+        into a packed tensor) that the loader fills.  The default makes one
+        attribute per name (``q.weight`` becomes ``self.q_weight``)."""
+        out = {}
+        for name, decl in self.param_decls().items():
+            t = torch.empty(decl.shape, dtype=dtypes[name], device=self.build.device)
+            setattr(self, name.replace(".", "_"), t)
+            out[name] = t
+        return out
+
+    def finalize(self) -> None:
+        """Called once after the tensors are filled."""
+
+    def cache_need(self) -> PagedKVNeed | None:
+        return None
+
+    def state_need(self) -> dict[str, StateNeed]:
+        return {}
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a request (attention here)."""
+
+    def prepare(self, ctx: "StepContext", run: RunBinding) -> None:
+        """Called for every run before the step's arrays go to the device; a mixer
+        may add host-built arrays of its own to that one copy."""
+
+    def forward(self, x: torch.Tensor, ctx: "StepContext", run: RunBinding) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def forward(
+        self,
+        h: torch.Tensor,
+        delta: torch.Tensor | None = None,
+        rows: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        """Normalises the float32 stream ``h`` after adding ``delta`` to it (the sum
+        is written back to ``h``); with ``rows`` only those rows, and ``h`` is left
+        as it is."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    pass
+
+
+class Embedding(Part):
+    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self.kinds: dict[str, type[Part]] = {}
+
+    def register(self, kind: str):
+        def deco(cls):
+            self.kinds[kind] = cls
+            cls.kind = kind
+            return cls
+
+        return deco
+
+    def build(self, spec: PartSpec, build: BuildContext) -> Part:
+        if spec.kind not in self.kinds:
+            known = ", ".join(sorted(self.kinds)) or "(none)"
+            raise ConfigError(f"unknown {self.what} kind {spec.kind!r}; known: {known}")
+        cls = self.kinds[spec.kind]
+        try:
+            params = cls.Params(**spec.params())
+        except ValidationError as e:
+            raise ConfigError(f"{self.what} {spec.kind!r}: bad parameters:\n{e}") from e
+        return cls(params, build)
+
+
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+NORMS = Registry("norm")
+POSITIONS = Registry("position encoding")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("head")
+ARRANGEMENTS: dict[str, type] = {}
+
+
+def register_arrangement(kind: str):
+    def deco(cls):
+        ARRANGEMENTS[kind] = cls
+        return cls
+
+    return deco

@@ -1,0 +1,69 @@
+"""The gated feed-forward (src/halite/transformers/feedforward.py:175-225)."""
+
+from __future__ import annotations
+
+import torch
+from pydantic import BaseModel, Field, StrictInt, field_validator
+
+from ..kernels import ops
+from .base import FEED_FORWARDS, FeedForward, ParamDecl
+
+
+class GatedParams(BaseModel):
+    hidden_size: StrictInt = Field(gt=0)
+    intermediate_size: StrictInt = Field(gt=0)
+    activation: str = "silu"
+
+    @field_validator("activation")
+    @classmethod
+    def _known(cls, v):
+        if v != "silu":
+            raise ValueError(f"activation {v!r}: only 'silu' has a kernel")
+        return v
+
+
+@FEED_FORWARDS.register("gated")
+class GatedFeedForward(FeedForward):
+    """``linear_out(linear_proj(x) * silu(linear_gate(x)))`` without biases
+    (feedforward.py:204-212).  Gate and up weights live in one tensor
+    ``[2F, d]`` (gate first) so that one product serves both; the activation and
+    the multiply are float32 on the accumulators or on the product's output."""
+
+    Params = GatedParams
+
+    def param_decls(self):
+        f, d = self.p.intermediate_size, self.p.hidden_size
+        return {
+            "linear_gate.weight": ParamDecl((f, d)),
+            "linear_proj.weight": ParamDecl((f, d)),
+            "linear_out.weight": ParamDecl((d, f)),
+        }
+
+    def allocate(self, dtypes):
+        f, d = self.p.intermediate_size, self.p.hidden_size
+        dev = self.build.device
+        if dtypes["linear_gate.weight"] != dtypes["linear_proj.weight"]:
+            raise ValueError("gate and up weights are stored with different element types")
+        self.w_gate_up = torch.empty((2 * f, d), dtype=dtypes["linear_gate.weight"], device=dev)
+        self.w_out = torch.empty((d, f), dtype=dtypes["linear_out.weight"], device=dev)
+        return {
+            "linear_gate.weight": self.w_gate_up[:f],
+            "linear_proj.weight": self.w_gate_up[f:],
+            "linear_out.weight": self.w_out,
+        }
+
+    def forward(self, x, ctx):
+        f = self.p.intermediate_size
+        w = self.w_gate_up
+        fused = (
+            w.dtype == torch.bfloat16
+            and x.dtype == torch.bfloat16
+            and x.shape[0] <= ops.SKINNY_MAX_ROWS
+            and x.shape[1] % 8 == 0
+            and (f * x.shape[1]) % 8 == 0
+        )
+        if fused:
+            act = ops.gemm_bf16_skinny(x, w[:f], w_up=w[f:])
+        else:
+            act = ops.silu_mul(ops.linear(x, w))
+        return ops.linear(act, self.w_out)
