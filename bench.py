@@ -1,0 +1,229 @@
+"""Benchmark: decode tokens a second and prefill tokens a second at the Llama-3.1-8B
+shape with seeded random weights on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+The default run decodes a batch of 8 requests whose contexts end at the configured
+context length (8,192 tokens); a step is one decode step of the engine: building the
+batch, the forward pass from the paged cache, greedy sampling and reading the tokens
+back.  The same line carries the prefill of one 2,048-token prompt, the decode step's
+fraction of the HBM roofline, and decode rates at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_BYTES_PER_S = 8.0e12
+PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
+
+LLAMA_3_1_8B = dict(
+    architectures=["LlamaForCausalLM"],
+    vocab_size=128256,
+    hidden_size=4096,
+    num_hidden_layers=32,
+    num_attention_heads=32,
+    num_key_value_heads=8,
+    head_dim=128,
+    intermediate_size=14336,
+    rms_norm_eps=1e-5,
+    rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    max_position_embeddings=8192,
+    tie_word_embeddings=False,
+)
+
+
+def layer_params(c) -> int:
+    d, f = c.hidden_size, c.intermediate_size
+    qkv = (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim * d
+    return qkv + c.num_attention_heads * c.head_dim * d + 3 * f * d + 2 * d
+
+
+def decode_bytes(c, n_layers, batch, kv_tokens, elt=2) -> float:
+    """What a decode step has to read: every weight it uses once (layers, final
+    norm, head; of the embedding only the batch's rows) and the cached keys and
+    values of the live requests."""
+    weights = n_layers * layer_params(c) + c.hidden_size + c.vocab_size * c.hidden_size
+    weights += batch * c.hidden_size
+    kv = kv_tokens * 2 * c.num_key_value_heads * c.head_dim * n_layers
+    return (weights + kv) * elt
+
+
+def prefill_flops(c, n_layers, t) -> float:
+    """2 flops per weight and token in the layers, causal attention (half of the
+    T x T scores and weighted sums), and the head for the one wanted row."""
+    linear = 2.0 * t * n_layers * (layer_params(c) - 2 * c.hidden_size)
+    attention = 2.0 * t * t * c.num_attention_heads * c.head_dim * n_layers
+    head = 2.0 * c.vocab_size * c.hidden_size
+    return linear + attention + head
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=None, help="context length at the end of decoding")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration (named in the record)")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import numpy as np
+    import torch
+
+    from halite_amd.config import LlamaConfig, ModelConfig, ServerConfig
+    from halite_amd.engine.batch import Segment
+    from halite_amd.engine.runner import ModelRunner
+    from halite_amd.sampling import Sampler, SamplingParams
+
+    full = LlamaConfig(**LLAMA_3_1_8B)
+    n_layers = args.layers or full.num_hidden_layers
+    cfg = full.model_copy(update={"num_hidden_layers": n_layers})
+    context = args.context or full.max_position_embeddings
+    elt = 2 if args.dtype == "bfloat16" else 4
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    pool_tokens = max(batches) * (context + 64) + 4096
+    runner = ModelRunner.from_random(
+        cfg, seed=0,
+        server_config=ServerConfig(kv_cache_num_tokens=pool_tokens, max_seqs_per_forward=max(batches) + 1,
+                                   max_tokens_per_forward=16384),
+        model_config=ModelConfig(dtype=args.dtype, context_len=context),
+    )
+    sampler = Sampler(runner.device)
+    greedy = SamplingParams(temperature=0.0)
+    gen = torch.Generator().manual_seed(0)
+
+    def sync():
+        torch.cuda.synchronize()
+
+    def decode_run(batch: int, steps: int, warmup: int):
+        """Prefills ``batch`` prompts so that the contexts end at ``context`` after
+        the last timed step, then times ``steps`` decode steps."""
+        prompt_len = context - steps - warmup
+        slots = [runner.admit() for _ in range(batch)]
+        last = []
+        for s in slots:
+            ids = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=gen).numpy().astype(np.int32)
+            pos, tok = 0, None
+            while pos < prompt_len:
+                n = min(4096, prompt_len - pos)
+                logits = runner.step([Segment(s, pos, ids[pos : pos + n], [n - 1] if pos + n == prompt_len else [])])
+                pos += n
+            tok, _ = sampler.forward(logits, [greedy], [0], [0])
+            last.append(int(tok[0]))
+        params, seeds, draws = [greedy] * batch, [0] * batch, [0] * batch
+
+        def one_step(tokens):
+            segs = [Segment(s, runner.cache.length(s), [t], [0]) for s, t in zip(slots, tokens)]
+            logits = runner.step(segs)
+            toks, _ = sampler.forward(logits, params, seeds, draws)
+            return toks.tolist()
+
+        for _ in range(warmup):
+            last = one_step(last)
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            last = one_step(last)
+        sync()
+        dt = time.perf_counter() - t0
+        kv_tokens = sum(runner.cache.length(s) for s in slots) - batch * steps / 2.0
+        for s in slots:
+            runner.free(s)
+        return dt, kv_tokens
+
+    # -- the headline: batch 8 -------------------------------------------------------
+    results = {}
+    for b in batches:
+        steps = args.steps if b == args.batch else max(8, args.steps // 2)
+        dt, kv_tokens = decode_run(b, steps, args.warmup)
+        results[b] = (b * steps / dt, dt / steps, kv_tokens, steps)
+        print(f"[bench] decode batch {b}: {results[b][0]:.1f} tok/s, {results[b][1] * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    value, step_s, kv_tokens, _ = results[args.batch]
+    need = decode_bytes(cfg, n_layers, args.batch, kv_tokens, elt)
+    achieved = need / step_s
+
+    record = {
+        "metric": "decode tokens per second (Llama-3.1-8B shape, batch 8, context 8192)",
+        "value": round(value, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: seeded uniform-random token ids, random weights N(0, 0.02)",
+        "config": {
+            "model": "Llama-3.1-8B shape",
+            "layers": n_layers,
+            "layers_of_model": full.num_hidden_layers,
+            "hidden_size": cfg.hidden_size,
+            "heads": cfg.num_attention_heads,
+            "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim,
+            "intermediate_size": cfg.intermediate_size,
+            "vocab_size": cfg.vocab_size,
+            "global_batch": args.batch,
+            "seq_len": context,
+            "context_len": context,
+            "prefill_tokens": 2048,
+            "page_size": runner.cache.page_size,
+            "parallelism": "single GPU",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved / 1e9, 1),
+            "peak": HBM_BYTES_PER_S / 1e9,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_BYTES_PER_S, 4),
+        },
+    }
+
+    if not args.no_points:
+        record["points"] = {f"decode_b{b}": round(results[b][0], 2) for b in (1, 64) if b in results}
+        # -- prefill of one 2,048-token prompt ----------------------------------------
+        T = 2048
+        ids = torch.randint(0, cfg.vocab_size, (T,), generator=gen).numpy().astype(np.int32)
+        times = []
+        for i in range(4):
+            s = runner.admit()
+            sync()
+            t0 = time.perf_counter()
+            logits = runner.step([Segment(s, 0, ids, [T - 1])])
+            tok, _ = sampler.forward(logits, [greedy], [0], [0])
+            tok.tolist()
+            sync()
+            times.append(time.perf_counter() - t0)
+            runner.free(s)
+        t = min(times[1:])
+        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+        record["prefill"] = {
+            "value": round(T / t, 1),
+            "tokens": T,
+            "ms": round(t * 1e3, 3),
+            "frac": round(prefill_flops(cfg, n_layers, T) / t / peak, 4),
+        }
+    print(json.dumps(record), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

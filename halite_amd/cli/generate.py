@@ -1,0 +1,86 @@
+"""Generate tokens from a model folder.
+
+In the manner of the reference's scripts (scripts/eval_task.py:161-185): ``--model``
+names the checkpoint folder, and free ``key=value`` words after the options override
+fields of the configuration objects: ``sampling.<field>`` (SamplingParams),
+``server.<field>`` (ServerConfig) and ``model.<field>`` (ModelConfig), e.g.
+
+    python -m halite_amd.cli.generate --model DIR --prompt-ids 1,2,3 \\
+        sampling.temperature=0.8 sampling.max_new_tokens=24 server.page_size=16
+
+Prompts are token ids (``--prompt-ids``, repeatable; ``--prompt-file`` with one JSON
+list a line) or seeded uniform-random ids of given lengths (``--prompt-lens``).
+Results are printed as one JSON object a line.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+
+import torch
+
+from ..config import ModelConfig, ServerConfig, parse_overrides, read_config
+
+
+def parse_args(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--model", type=str, required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--prompt-ids", action="append", default=[], help="comma-separated token ids; repeatable")
+    ap.add_argument("--prompt-file", type=str, help="file with one JSON list of token ids a line")
+    ap.add_argument("--prompt-lens", type=str, help="comma-separated lengths of random prompts")
+    ap.add_argument("--prompt-seed", type=int, default=0)
+    ap.add_argument("--seed", type=int, default=0, help="engine seed for sampling streams")
+    ap.add_argument("--stats", action="store_true", help="print scheduler statistics to stderr")
+    ap.add_argument("opts", default=None, nargs=argparse.REMAINDER, help="key=value overrides")
+    return ap.parse_args(argv)
+
+
+def split_overrides(opts):
+    groups = {"sampling": {}, "server": {}, "model": {}}
+    for key, value in parse_overrides([o for o in (opts or []) if o != "--"]).items():
+        head, _, field = key.partition(".")
+        if head not in groups or not field:
+            raise SystemExit(f"override {key!r}: use sampling.<field>, server.<field> or model.<field>")
+        groups[head][field] = value
+    return groups
+
+
+def main(argv=None) -> int:
+    args = parse_args(argv)
+    over = split_overrides(args.opts)
+    from ..engine import InferenceEngine
+    from ..sampling import SamplingParams
+
+    _, cfg = read_config(args.model)
+    prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
+    if args.prompt_file:
+        with open(args.prompt_file) as f:
+            prompts += [json.loads(line) for line in f if line.strip()]
+    if args.prompt_lens:
+        gen = torch.Generator().manual_seed(args.prompt_seed)
+        for n in args.prompt_lens.split(","):
+            prompts.append(torch.randint(0, cfg.vocab_size, (int(n),), generator=gen).tolist())
+    if not prompts:
+        raise SystemExit("no prompts: give --prompt-ids, --prompt-file or --prompt-lens")
+
+    engine = InferenceEngine.from_pretrained(
+        args.model, ServerConfig(**over["server"]), ModelConfig(**over["model"]), seed=args.seed
+    )
+    params = SamplingParams(**over["sampling"])
+    results = engine.infer_batch([(i, p, params) for i, p in enumerate(prompts)])
+    for r in results:
+        print(json.dumps(r.to_dict()))
+    if args.stats:
+        s = engine.stats
+        print(
+            f"steps {s.steps} prefill tokens {s.prefill_tokens} decode tokens {s.decode_tokens} "
+            f"retractions {s.retractions} elapsed {engine.last_elapsed:.3f} s",
+            file=sys.stderr,
+        )
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
