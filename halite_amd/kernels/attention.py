@@ -20,8 +20,8 @@ from . import library, ops
 
 ROWS_PER_ITEM = 16
 KEYS_PER_BLOCK = 32
-MIN_SPLIT_KEYS = 128
-TARGET_WAVES = 4096
+MIN_SPLIT_KEYS = 256
+TARGET_WAVES = 2048
 
 
 @dataclass
@@ -60,9 +60,12 @@ def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: 
     seg_ids, rho0s = np.concatenate(seg_ids), np.concatenate(rho0s)
     kv_b, kv_e = np.concatenate(kv_b), np.concatenate(kv_e)
     span = kv_e - kv_b
-    total = int(span.sum()) * n_kv_heads
-    chunk = -(-total // TARGET_WAVES)
-    chunk = max(MIN_SPLIT_KEYS, -(-chunk // KEYS_PER_BLOCK) * KEYS_PER_BLOCK)
+    if len(span) * n_kv_heads * 2 >= TARGET_WAVES:
+        chunk = 1 << 30  # enough tiles to fill the GPU: nothing is cut
+    else:
+        total = int(span.sum()) * n_kv_heads
+        chunk = -(-total // TARGET_WAVES)
+        chunk = max(MIN_SPLIT_KEYS, -(-chunk // KEYS_PER_BLOCK) * KEYS_PER_BLOCK)
     base = kv_b - kv_b % KEYS_PER_BLOCK  # pieces end on multiples of 32 keys
     n_pieces = np.maximum(1, -(-(kv_e - base) // chunk))
 

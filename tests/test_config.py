@@ -1,0 +1,125 @@
+import json
+
+import pytest
+
+import tiny
+from halite_amd.config import (
+    ConfigError,
+    LlamaConfig,
+    ModelConfig,
+    ModelSpec,
+    ServerConfig,
+    get_architecture,
+    parse_config,
+    parse_overrides,
+    read_config,
+)
+
+
+def test_parses_both_tiny_configs():
+    for raw in (tiny.TINY_A, tiny.TINY_B, tiny.TINY_C):
+        arch, cfg = parse_config(raw)
+        assert arch.name == "LlamaForCausalLM"
+        assert isinstance(cfg, LlamaConfig)
+        assert cfg.head_dim == raw["head_dim"] and cfg.rms_norm_eps == raw["rms_norm_eps"]
+        assert cfg.rope_theta == raw["rope_theta"]
+    _, b = parse_config(tiny.TINY_B)
+    assert b.rope_scaling.factor == 8.0 and b.rope_scaling.original_max_position_embeddings == 64
+    assert b.tie_word_embeddings is True
+
+
+def test_defaults_that_have_a_meaning():
+    raw = dict(tiny.TINY_A)
+    del raw["num_key_value_heads"], raw["head_dim"]
+    _, cfg = parse_config(raw)
+    assert cfg.num_key_value_heads == 4 and cfg.head_dim == 16 and cfg.rope_scaling is None
+
+
+@pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
+                                 "intermediate_size", "rms_norm_eps", "rope_theta", "max_position_embeddings"])
+def test_no_size_has_a_default_in_code(key):
+    raw = dict(tiny.TINY_A)
+    del raw[key]
+    with pytest.raises(ConfigError, match=key):
+        parse_config(raw)
+
+
+@pytest.mark.parametrize(
+    "change,match",
+    [
+        ({"num_key_value_heads": 3}, "not a multiple"),
+        ({"head_dim": 15}, "odd"),
+        ({"attention_bias": True}, "bias"),
+        ({"mlp_bias": True}, "bias"),
+        ({"hidden_act": "gelu"}, "silu"),
+        ({"rope_scaling": {"rope_type": "yarn", "factor": 2.0}}, "llama3"),
+        ({"rope_scaling": {"rope_type": "llama3", "factor": 2.0}}, "low_freq_factor"),
+        ({"vocab_size": "256"}, "vocab_size"),
+        ({"num_hidden_layers": 0}, "num_hidden_layers"),
+    ],
+)
+def test_validation_errors(change, match):
+    with pytest.raises(ConfigError, match=match):
+        parse_config({**tiny.TINY_A, **change})
+
+
+def test_unknown_architecture_lists_known():
+    with pytest.raises(ConfigError, match="LlamaForCausalLM"):
+        parse_config({**tiny.TINY_A, "architectures": ["MambaForCausalLM"]})
+    with pytest.raises(ConfigError, match="architectures"):
+        parse_config({k: v for k, v in tiny.TINY_A.items() if k != "architectures"})
+
+
+def test_round_trip_through_json(tmp_path):
+    _, cfg = parse_config(tiny.TINY_B)
+    (tmp_path / "config.json").write_text(json.dumps(cfg.to_json_dict()))
+    _, again = read_config(str(tmp_path))
+    assert again == cfg
+    with pytest.raises(ConfigError, match="config.json"):
+        read_config(str(tmp_path / "nothing"))
+
+
+def test_spec_is_data():
+    arch, cfg = parse_config(tiny.TINY_B)
+    spec = arch.to_spec(cfg)
+    assert [r.layer for r in spec.order] == ["0", "1", "2"]
+    att = spec.layers["1"].mixer
+    assert att.kind == "attention" and att.params()["n_kv_heads"] == 1 and att.params()["head_dim"] == 32
+    assert abs(att.params()["scale"] - 32**-0.5) < 1e-12
+    assert spec.positions["rope"].params()["scaling"]["factor"] == 8.0
+    assert spec.head.params()["tied"] is True
+    again = ModelSpec(**json.loads(spec.model_dump_json()))
+    assert again == spec
+    # the run order is validated as data too
+    bad = spec.model_dump()
+    bad["order"][1]["cache_from"] = 2
+    with pytest.raises(ValueError, match="earlier run"):
+        ModelSpec(**bad)
+    bad = spec.model_dump()
+    bad["order"][0]["layer"] = "nope"
+    with pytest.raises(ValueError, match="unknown layer"):
+        ModelSpec(**bad)
+
+
+def test_weight_map_names():
+    arch = get_architecture("LlamaForCausalLM")
+    _, a = parse_config(tiny.TINY_A)
+    _, b = parse_config(tiny.TINY_B)
+    assert arch.weight_map(a)["lm_head.weight"] == "head.weight"
+    assert arch.weight_map(b)["lm_head.weight"] is None
+    assert arch.weight_map(a)["model.layers.#.mlp.up_proj.weight"] == "layers.#.ff.linear_proj.weight"
+
+
+def test_engine_options_and_overrides():
+    s = ServerConfig(**parse_overrides(["page_size=16", "max_tokens_per_forward=512", "use_cudagraph=true"]))
+    assert s.page_size == 16 and s.max_tokens_per_forward == 512 and s.use_cudagraph is True
+    assert s.max_prefill_tokens == 16384 and s.chunked_prefill_size == 8192  # the reference's defaults
+    assert s.default_init_new_token_ratio == 0.7
+    with pytest.raises(ValueError):
+        ServerConfig(page_size=0)
+    with pytest.raises(ValueError):
+        ServerConfig(no_such_option=1)
+    with pytest.raises(ValueError):
+        ModelConfig(dtype="float16")
+    with pytest.raises(ValueError, match="key=value"):
+        parse_overrides(["page_size"])

@@ -1,0 +1,152 @@
+"""Generation through the entry point and the command line, against the plain
+implementation."""
+
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_llama
+import tiny
+from halite_amd.config import ModelConfig, ServerConfig
+from halite_amd.engine import InferenceEngine, InferenceRequest
+from halite_amd.sampling import SamplingParams, request_seed
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name, cfg in (("A", tiny.TINY_A), ("B", tiny.TINY_B)):
+        w = tiny.random_weights(cfg, seed=21, std=0.08)
+        for dtype, store in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+            folder = str(tmp_path_factory.mktemp(f"gen{name}{dtype}"))
+            tiny.write_model_folder(folder, cfg, w, store)
+            out[(name, dtype)] = (folder, *plain_llama.read_model_folder(folder))
+    return out
+
+
+def check_against_plain(pc, pw, prompt, got, params, gap_limit, margin_limit):
+    """Teacher-forced on the engine's own tokens: at every step the plain model's
+    choice must be the engine's, unless the decision is closer than rounding."""
+    ids = list(prompt)
+    for step, tok in enumerate(got):
+        logits = plain_llama.forward(pc, pw, ids)[-1]
+        want, _, margin = plain_llama.sample_token(logits, params, step)
+        if tok != want:
+            if margin is None:
+                assert float(logits[want] - logits[tok]) <= gap_limit, f"token {step}: engine {tok}, plain {want}"
+            else:
+                assert margin <= margin_limit, f"token {step}: engine {tok}, plain {want} (margin {margin})"
+        ids.append(tok)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation(models, dtype):
+    folder, pc, pw = models[("A", dtype)]
+    engine = InferenceEngine.from_pretrained(folder, ServerConfig(kv_cache_num_tokens=1024), ModelConfig(dtype=dtype))
+    prompts = [tiny.random_tokens(tiny.TINY_A, n, 40 + n) for n in (5, 17, 33, 64)]
+    params = {"max_new_tokens": 16, "temperature": 0.0}
+    results = engine.infer_batch([InferenceRequest(f"q{i}", p, params) for i, p in enumerate(prompts)])
+    assert [r.id for r in results] == ["q0", "q1", "q2", "q3"]
+    for r, p in zip(results, prompts):
+        assert r.input_ids == p and len(r.output_ids) == 1 and len(r.output_ids[0]) == 16
+        assert r.finish_reason == ["length"] and len(r.output_logprobs[0]) == 16
+        check_against_plain(pc, pw, p, r.output_ids[0], params, 1e-4 if dtype == "float32" else 0.06, 0)
+        if dtype == "float32":
+            want, lps, _ = plain_llama.generate(pc, pw, p, params)
+            assert r.output_ids[0] == want
+            assert max(abs(a - b) for a, b in zip(r.output_logprobs[0], lps)) < 1e-4
+    # top_k = 1 asks for the same thing, whatever the temperature
+    again = engine.infer_batch([(p, {"max_new_tokens": 16, "top_k": 1, "temperature": 0.7}) for p in prompts])
+    assert [r.output_ids for r in again] == [r.output_ids for r in results]
+    assert engine.model_runner.cache.idle()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_temperature_sampling_with_a_seed(models, dtype):
+    folder, pc, pw = models[("B", dtype)]
+    engine = InferenceEngine.from_pretrained(folder, ServerConfig(kv_cache_num_tokens=1024, page_size=16), ModelConfig(dtype=dtype))
+    prompts = [tiny.random_tokens(tiny.TINY_B, n, 50 + n) for n in (1, 40, 100)]
+    params = SamplingParams(max_new_tokens=24, temperature=0.8, seed=1234)
+    results = engine.infer_batch([(i, p, params) for i, p in enumerate(prompts)])
+    plain_params = {"temperature": 0.8, "seed": request_seed(params, 0), "max_new_tokens": 24}
+    for r, p in zip(results, prompts):
+        assert len(r.output_ids[0]) == 24
+        check_against_plain(pc, pw, p, r.output_ids[0], plain_params, 0, 2e-4 if dtype == "float32" else 2e-2)
+    # the same seed gives the same tokens, alone or beside other requests
+    # (bfloat16 logits move by rounding with the batch, which can flip a draw that
+    # falls next to an interval's edge, so the strict comparison is the 32-bit one)
+    alone = engine.infer_batch([(7, prompts[1], params)])
+    if dtype == "float32":
+        assert alone[0].output_ids == results[1].output_ids
+    else:
+        assert alone[0].output_ids[0][:4] == results[1].output_ids[0][:4]
+    other = engine.infer_batch([(0, prompts[1], SamplingParams(max_new_tokens=24, temperature=0.8, seed=99))])
+    assert other[0].output_ids != results[1].output_ids
+    # n samples of one request draw from different streams
+    many = engine.infer_batch([(0, prompts[1], SamplingParams(max_new_tokens=12, temperature=1.0, seed=5, n=3))])
+    assert len(many[0].output_ids) == 3 and len({tuple(o) for o in many[0].output_ids}) == 3
+
+
+def test_filters_and_stop_tokens_through_the_engine(models):
+    folder, pc, pw = models[("A", "float32")]
+    engine = InferenceEngine.from_pretrained(folder, ServerConfig(kv_cache_num_tokens=512), ModelConfig(dtype="float32"))
+    p = tiny.random_tokens(tiny.TINY_A, 20, 3)
+    params = SamplingParams(max_new_tokens=12, temperature=1.3, top_k=7, top_p=0.9, seed=8)
+    r = engine.infer_batch([(0, p, params)])[0]
+    plain_params = {"temperature": 1.3, "top_k": 7, "top_p": 0.9, "seed": 8}
+    check_against_plain(pc, pw, p, r.output_ids[0], plain_params, 0, 2e-4)
+    greedy, _, _ = plain_llama.generate(pc, pw, p, {"temperature": 0.0, "max_new_tokens": 12})
+    stop = greedy[5]
+    r = engine.infer_batch([(0, p, {"temperature": 0.0, "max_new_tokens": 12, "stop_token_ids": [stop]})])[0]
+    assert r.output_ids[0] == greedy[: greedy.index(stop) + 1] and r.finish_reason == ["stop"]
+    with pytest.raises(ValueError, match="tokenizer"):
+        engine.infer_batch(["some text"])
+
+
+def test_portions_retraction_and_page_reuse_keep_the_tokens(models):
+    """Greedy output does not depend on the budget, on the portions, or on requests
+    being thrown out and run again when pages run out."""
+    folder, pc, pw = models[("A", "float32")]
+    prompts = [tiny.random_tokens(tiny.TINY_A, n, 60 + n) for n in (30, 9, 41, 17, 25, 12)]
+    params = {"max_new_tokens": 40, "temperature": 0.0, "ignore_eos": True}
+    roomy = InferenceEngine.from_pretrained(folder, ServerConfig(kv_cache_num_tokens=2048, page_size=16), ModelConfig(dtype="float32"))
+    want = [r.output_ids[0] for r in roomy.infer_batch([(i, p, params) for i, p in enumerate(prompts)])]
+    tight = InferenceEngine.from_pretrained(
+        folder,
+        ServerConfig(kv_cache_num_tokens=160, page_size=16, max_tokens_per_forward=24, chunked_prefill_size=11,
+                     default_init_new_token_ratio=0.05),
+        ModelConfig(dtype="float32"),
+    )
+    got = tight.infer_batch([(i, p, params) for i, p in enumerate(prompts)])
+    assert tight.stats.retractions > 0
+    assert max(tight.stats.tokens_per_step) <= 24
+    assert [r.output_ids[0] for r in got] == want
+    assert tight.model_runner.cache.idle()
+
+
+def test_command_line(models, tmp_path):
+    folder, pc, pw = models[("B", "float32")]
+    cmd = [sys.executable, "-m", "halite_amd.cli.generate", "--model", folder, "--prompt-ids", "5,17,3,250,9",
+           "--prompt-lens", "12", "--prompt-seed", "4", "--stats",
+           "sampling.temperature=0", "sampling.max_new_tokens=6", "model.dtype=float32", "server.page_size=16"]
+    proc = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [json.loads(l) for l in proc.stdout.strip().split("\n")]
+    assert len(lines) == 2 and lines[0]["input_ids"] == [5, 17, 3, 250, 9]
+    for rec in lines:
+        want, _, _ = plain_llama.generate(pc, pw, rec["input_ids"], {"temperature": 0.0, "max_new_tokens": 6})
+        assert rec["output_ids"] == [want]
+    assert "steps" in proc.stderr
+    out = tmp_path / "rand"
+    cfgfile = tmp_path / "c.json"
+    cfgfile.write_text(json.dumps(tiny.TINY_A))
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "halite_make_random_model"), "--config", str(cfgfile),
+                           "--out", str(out), "--seed", "3", "--dtype", "float32"], capture_output=True, text=True)
+    assert proc.returncode == 0 and (out / "model.safetensors").exists() and (out / "config.json").exists()

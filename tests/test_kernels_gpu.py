@@ -1,0 +1,329 @@
+"""Each kernel alone against its plain reference, at other sizes than the engine's."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+from halite_amd.kernels import attention as attn_kernels
+from halite_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+def close(got, want, tol, what=""):
+    got, want = got.float().cpu(), want.float().cpu()
+    err = float((got - want).abs().max()) / max(1.0, float(want.abs().max()))
+    assert err == err and err <= tol, f"{what}: error {err:.3e} > {tol:.1e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("vocab,d", [(331, 120), (1000, 4096), (17, 8)])
+def test_embedding(gpu, dtype, vocab, d):
+    table = rnd(vocab, d, seed=1).to(DT[dtype])
+    ids = torch.randint(0, vocab, (37,), generator=torch.Generator().manual_seed(2), dtype=torch.int32)
+    out = ops.embedding(ids.to(gpu), table.to(gpu))
+    assert out.dtype == torch.float32
+    assert torch.equal(out.cpu(), P.embed(ids.long(), table.float()))
+    bad = ops.embedding(torch.tensor([vocab], dtype=torch.int32, device=gpu), table.to(gpu))
+    assert torch.isnan(bad).all()  # an id outside the table shows, it does not fault
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("d", [120, 1000, 4096])
+def test_rmsnorm(gpu, dtype, d):
+    dt = DT[dtype]
+    h = rnd(9, d, seed=3, scale=2.0)
+    delta = rnd(9, d, seed=4).to(dt)
+    w = (1 + 0.2 * rnd(d, seed=5)).to(dt)
+    eps = 3e-6
+    tol = 1e-6 if dtype == "float32" else 1e-2
+    # plain: statistics in float32, rounded to the activation type, then the weight
+    x = h + delta.float()
+    want = P.rms_norm(x.to(dt), w, eps) if dtype == "float32" else (w.float() * (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)).to(dt).float())
+    hg = h.to(gpu).clone()
+    out = ops.rmsnorm(hg, w.to(gpu), eps, dt, delta=delta.to(gpu))
+    close(out, want, tol, "norm with add")
+    close(hg, x, 1e-7, "stream after add")
+    # no delta: the stream stays
+    hg = h.to(gpu).clone()
+    out = ops.rmsnorm(hg, w.to(gpu), eps, dt)
+    close(out, P.rms_norm(h, w.float(), eps), tol, "norm")
+    assert torch.equal(hg.cpu(), h)
+    # gathered rows: only those, and the stream stays
+    rows = torch.tensor([7, 0, 7, 3], dtype=torch.int32)
+    hg = h.to(gpu).clone()
+    out = ops.rmsnorm(hg, w.to(gpu), eps, dt, delta=delta.to(gpu), rows=rows.to(gpu))
+    close(out, want[rows.long()], tol, "gathered norm")
+    assert torch.equal(hg.cpu(), h)
+    # a 32-bit weight with bfloat16 activations
+    if dtype == "bfloat16":
+        out = ops.rmsnorm(h.to(gpu).clone(), w.float().to(gpu), eps, dt)
+        close(out, P.rms_norm(h, w.float(), eps), tol, "norm, 32-bit weight")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_silu_mul_and_residual_add(gpu, dtype):
+    dt = DT[dtype]
+    gu = rnd(11, 2 * 352, seed=6, scale=3.0).to(dt)
+    g, u = gu[:, :352].float(), gu[:, 352:].float()
+    close(ops.silu_mul(gu.to(gpu)), u * g * torch.sigmoid(g), 1e-6 if dtype == "float32" else 5e-3)
+    h, d = rnd(5, 77, seed=7), rnd(5, 77, seed=8).to(dt)
+    close(ops.residual_add(h.to(gpu).clone(), d.to(gpu)), h + d.float(), 1e-7)
+
+
+def paged_cache(k, v, page_size, seed, n_extra=3, dtype=torch.float32, poison=True):
+    """Scatters dense keys/values [n, K, D] of ONE request over randomly chosen pages.
+    Returns (k_pages, v_pages, table row) with NaN in every slot that holds nothing."""
+    n, K, D = k.shape
+    n_logical = -(-n // page_size)
+    n_pages = n_logical + n_extra + 1
+    perm = torch.randperm(n_pages - 1, generator=torch.Generator().manual_seed(seed))[:n_logical] + 1
+    fill = float("nan") if poison else 0.0
+    kp = torch.full((n_pages, K, page_size, D), fill)
+    vp = torch.full((n_pages, K, D, page_size), fill)
+    for j in range(n):
+        p, o = int(perm[j // page_size]), j % page_size
+        kp[p, :, o, :] = k[j]
+        vp[p, :, :, o] = v[j]
+    return kp.to(dtype), vp.to(dtype), perm.to(torch.int32)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("H,K,D,rot,page", [(4, 2, 16, 16, 4), (6, 2, 48, 48, 16), (3, 1, 32, 16, 8), (8, 8, 128, 128, 64)])
+def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page):
+    dt = DT[dtype]
+    n_seg, table_w = 3, -(-64 // page)
+    lens, starts = [5, 1, 9], [3, 40, 0]
+    T = sum(lens)
+    qkv = rnd(T, (H + 2 * K) * D, seed=9).to(dt)
+    positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).to(torch.int32)
+    token_seg = torch.cat([torch.full((n,), i) for i, n in enumerate(lens)]).to(torch.int32)
+    n_pages = n_seg * table_w + 8
+    bt = torch.randperm(n_pages - 1, generator=torch.Generator().manual_seed(1))[: n_seg * table_w].view(n_seg, table_w) + 1
+    inv = P.inverse_frequencies(rot, 10000.0)
+    cos, sin = P.rotation_table(torch.arange(64), inv)
+    kp = torch.zeros(n_pages, K, page, D, dtype=dt, device=gpu)
+    vp = torch.zeros(n_pages, K, D, page, dtype=dt, device=gpu)
+    got = qkv.to(gpu).clone()
+    ops.rope_append(got, positions.to(gpu), cos.to(gpu), sin.to(gpu), H, K, D, rot, interleaved,
+                    token_seg=token_seg.to(gpu), block_table=bt.to(torch.int32).to(gpu),
+                    k_pages=kp, v_pages=vp, page_size=page)
+    q = qkv[:, : H * D].float().view(T, H, D)
+    k = qkv[:, H * D : (H + K) * D].float().view(T, K, D)
+    v = qkv[:, (H + K) * D :].float().view(T, K, D)
+    rotate = P.rotate_interleaved if interleaved else P.rotate_half_split
+    c, s = cos[positions.long()], sin[positions.long()]
+    rq = torch.cat((rotate(q[..., :rot], c, s), q[..., rot:]), -1)
+    rk = torch.cat((rotate(k[..., :rot], c, s), k[..., rot:]), -1)
+    tol = 1e-6 if dtype == "float32" else 8e-3
+    close(got[:, : H * D].view(T, H, D), rq, tol, "rotated q")
+    assert torch.equal(got[:, (H + K) * D :].cpu(), qkv[:, (H + K) * D :])  # v untouched
+    kpc, vpc = kp.float().cpu(), vp.float().cpu()
+    written = torch.zeros(n_pages, page, dtype=torch.bool)
+    for t in range(T):
+        pos, seg = int(positions[t]), int(token_seg[t])
+        pg, off = int(bt[seg, pos // page]), pos % page
+        close(kpc[pg, :, off, :], rk[t], tol, "k page")
+        assert torch.equal(vpc[pg, :, :, off], v[t].to(dt).float())
+        written[pg, off] = True
+    assert float(kpc.abs().sum(dim=(1, 3))[~written].sum()) == 0  # nothing else was written
+    assert float(vpc.abs().sum(dim=(1, 2))[~written].sum()) == 0
+
+
+def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use):
+    """``segs``: list of (cached before, new tokens).  Builds one dense sequence per
+    segment, pages it, and compares the rows of the new tokens with plain attention
+    over the whole sequence."""
+    dt = DT[dtype]
+    scale = D**-0.5
+    qs, tables, kps, vps, want, pos, seg_of = [], [], [], [], [], [], []
+    page_base = 0
+    all_k, all_v = [], []
+    for i, (before, new) in enumerate(segs):
+        n = before + new
+        q = rnd(n, H, D, seed=seed + 3 * i).to(dt).float()
+        k = rnd(n, K, D, seed=seed + 3 * i + 1).to(dt).float()
+        v = rnd(n, K, D, seed=seed + 3 * i + 2).to(dt).float()
+        if n > 40:  # one far key stands out: a kernel that drops or misplaces it shows
+            far = 3
+            k[far] = 0
+            k[far, :, 0] = 6.0
+            q[-1, :, :] = 0
+            q[-1, :, 0] = 6.0 * math.sqrt(D) / 6.0 * 2.0
+            v[far] = 5.0
+        ref = P.causal_attention(q, k, v, window=window or None)
+        want.append(ref[before:].reshape(new, H * D))
+        qs.append(q[before:].reshape(new, H * D))
+        kp, vp, row = paged_cache(k, v, page, seed + i, dtype=dt)
+        tables.append(row + page_base)
+        page_base += kp.shape[0]
+        kps.append(kp), vps.append(vp)
+        pos.append(torch.arange(before, n))
+        seg_of.append(torch.full((new,), i))
+    width = max(len(t) for t in tables)
+    bt = torch.full((len(segs), width), -1, dtype=torch.int32)
+    for i, t in enumerate(tables):
+        bt[i, : len(t)] = t
+    k_pages, v_pages = torch.cat(kps).to(gpu), torch.cat(vps).to(gpu)
+    q = torch.cat(qs).to(dt).to(gpu)
+    positions = torch.cat(pos).to(torch.int32).to(gpu)
+    token_seg = torch.cat(seg_of).to(torch.int32).to(gpu)
+    if use == "simple":
+        out = ops.attention_simple(q, H * D, positions, token_seg, bt.to(gpu), k_pages, v_pages, H, scale, window)
+    else:
+        q_len = np.array([n for _, n in segs], dtype=np.int32)
+        kv_len = np.array([b + n for b, n in segs], dtype=np.int32)
+        plan = attn_kernels.plan_items(q_len, kv_len, H // K, K, window)
+        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+
+        class Ctx:
+            n_tokens = int(q_len.sum())
+            seg_q_start = dev(np.concatenate(([0], np.cumsum(q_len)[:-1])).astype(np.int32))
+            seg_q_len = dev(q_len)
+            seg_kv_len = dev(kv_len)
+
+        class Group:
+            block_table = bt.to(gpu)
+
+        class KV:
+            k, v = k_pages, v_pages
+
+        counts = dev(np.array([plan.n_items, plan.n_merges], dtype=np.int32))
+        out = attn_kernels.attention_mfma(q, H * D, (plan, dev(plan.items), dev(plan.merges), counts), Ctx, Group, KV, H, scale, window)
+    close(out, torch.cat(want), 5e-6 if dtype == "float32" else 1.2e-2, f"attention {use}")
+
+
+SHAPES = [(4, 2, 16), (6, 2, 48), (4, 1, 32), (8, 8, 64), (32, 8, 128), (5, 5, 80), (20, 1, 16)]
+SEGS = [[(0, 1)], [(0, 70)], [(63, 1), (0, 33), (64, 64), (129, 2), (200, 1)], [(700, 1), (5, 300)]]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("segs", SEGS)
+@pytest.mark.parametrize("H,K,D", SHAPES[:5])
+def test_attention_simple(gpu, dtype, H, K, D, segs):
+    for page, window in ((1, 0), (4, 0), (16, 0), (64, 0), (16, 37), (4, 1)):
+        attention_case(gpu, dtype, H, K, D, page, segs, window, seed=20, use="simple")
+
+
+@pytest.mark.parametrize("segs", SEGS)
+@pytest.mark.parametrize("H,K,D", SHAPES)
+def test_attention_mfma(gpu, H, K, D, segs):
+    for page, window in ((8, 0), (16, 0), (64, 0), (24, 0), (16, 37), (8, 1), (64, 300)):
+        attention_case(gpu, "bfloat16", H, K, D, page, segs, window, seed=30, use="mfma")
+
+
+def test_attention_mfma_split_keys(gpu):
+    # few rows and many keys: the key range is cut and merged
+    segs = [(3000, 1), (1500, 2), (4000, 1)]
+    plan = attn_kernels.plan_items(np.array([1, 2, 1]), np.array([3001, 1502, 4001]), 4, 2, 0)
+    assert plan.n_merges == 3
+    attention_case(gpu, "bfloat16", 8, 2, 128, 64, segs, 0, seed=40, use="mfma")
+    attention_case(gpu, "bfloat16", 8, 2, 128, 16, segs, 1000, seed=41, use="mfma")
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 256, 64), (5, 331, 120), (64, 200, 352), (130, 96, 1000), (3, 4096, 4096)])
+def test_gemm_f32(gpu, M, N, K):
+    a, w = rnd(M, K, seed=50), rnd(N, K, seed=51)
+    want = (a.double() @ w.double().T).float()
+    close(ops.gemm_f32(a.to(gpu), w.to(gpu)), want, 3e-6, "gemm_f32")
+    # a row's result does not depend on the other rows of the batch
+    alone = ops.gemm_f32(a[:1].to(gpu).contiguous(), w.to(gpu))
+    assert torch.equal(alone.cpu(), ops.gemm_f32(a.to(gpu), w.to(gpu))[:1].cpu())
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("N,K", [(256, 64), (331, 120), (1000, 352), (4096, 4096), (200, 14336)])
+def test_gemm_bf16_skinny(gpu, M, N, K):
+    x = rnd(M, K, seed=60).to(torch.bfloat16)
+    w = rnd(N, K, seed=61, scale=0.05).to(torch.bfloat16)
+    w2 = rnd(N, K, seed=62, scale=0.05).to(torch.bfloat16)
+    want = x.float() @ w.float().T
+    xg, wg, w2g = x.to(gpu), w.to(gpu), w2.to(gpu)
+    close(ops.gemm_bf16_skinny(xg, wg, out_dtype=torch.float32), want, 2e-5, "skinny f32")
+    close(ops.gemm_bf16_skinny(xg, wg), want, 5e-3, "skinny bf16")
+    base = rnd(M, N, seed=63)
+    acc = base.to(gpu).clone()
+    ops.gemm_bf16_skinny(xg, wg, add_to=acc)
+    close(acc, base + want, 2e-5, "skinny add")
+    up = x.float() @ w2.float().T
+    close(ops.gemm_bf16_skinny(xg, wg, w_up=w2g, out_dtype=torch.float32), up * want * torch.sigmoid(want), 3e-5, "skinny gated")
+    with pytest.raises(ops.KernelError):
+        ops.gemm_bf16_skinny(rnd(65, K).to(torch.bfloat16).to(gpu), wg)
+
+
+def test_linear_dispatch(gpu):
+    x = rnd(100, 352, seed=70).to(torch.bfloat16).to(gpu)
+    w = rnd(331, 352, seed=71, scale=0.05)
+    want = x.float().cpu() @ w.to(torch.bfloat16).float().T
+    close(ops.linear(x, w.to(torch.bfloat16).to(gpu)), want, 8e-3, "library product")
+    close(ops.linear(x, w.to(torch.bfloat16).to(gpu), out_dtype=torch.float32), want, 3e-5, "float32 output in passes")
+    # a 32-bit weight under bfloat16 activations runs the 32-bit kernel
+    close(ops.linear(x, w.to(gpu), out_dtype=torch.float32), x.float().cpu() @ w.T, 3e-6, "32-bit weight")
+    assert ops.linear(x, w.to(gpu)).dtype == torch.bfloat16
+
+
+def _sample(gpu, logits, **kw):
+    n = logits.shape[0]
+    f = lambda v, dt: torch.full((n,), v, dtype=dt, device=gpu) if not torch.is_tensor(v) else v.to(gpu)
+    return ops.sample(
+        logits.to(gpu), f(kw.get("temperature", 1.0), torch.float32), f(kw.get("top_k", -1), torch.int32),
+        f(kw.get("top_p", 1.0), torch.float32), f(kw.get("min_p", 0.0), torch.float32),
+        f(kw.get("seed", 7), torch.int64), kw.get("draw", torch.arange(n, dtype=torch.int32)).to(gpu),
+    )
+
+
+@pytest.mark.parametrize("vocab", [331, 1000, 128256])
+def test_sample_greedy(gpu, vocab):
+    logits = rnd(6, vocab, seed=80, scale=2.0)
+    logits[1, 5] = logits[1, 300] = 50.0  # a tie: the first index wins, as torch.argmax
+    logits[2, 17] = float("nan")
+    tok, lp = _sample(gpu, logits, temperature=0.0)
+    clean = torch.where(torch.isnan(logits), torch.full_like(logits, -1e5), logits)
+    assert tok.cpu().tolist() == torch.argmax(clean, -1).tolist() and tok[1] == 5
+    want = torch.log_softmax(clean.double(), -1).gather(1, tok.cpu().long()[:, None])[:, 0]
+    close(lp, want.float(), 1e-5, "greedy logprob")
+    tok2, _ = _sample(gpu, logits, temperature=0.9, top_k=1)
+    assert torch.equal(tok, tok2)
+
+
+@pytest.mark.parametrize("kw", [{}, {"top_k": 5}, {"top_p": 0.7}, {"top_k": 40, "top_p": 0.9}, {"min_p": 0.1},
+                                {"top_k": 9, "top_p": 0.8, "min_p": 0.05}, {"temperature": 0.6, "top_p": 0.5}])
+def test_sample_matches_the_plain_sampler(gpu, kw):
+    vocab, n = 1000, 400
+    base = rnd(1, vocab, seed=81, scale=2.5)[0]
+    logits = base[None].repeat(n, 1)
+    tok, lp = _sample(gpu, logits, seed=11, **kw)
+    params = {"temperature": 1.0, "seed": 11, **kw}
+    probs = P.filtered_probabilities(base, params["temperature"], params.get("top_k", -1), params.get("top_p", 1.0), params.get("min_p", 0.0))
+    agree = 0
+    for i in range(n):
+        t, logprob, margin = P.sample_token(base, params, i)
+        assert probs[int(tok[i])] > 0, "a filtered token was sampled"
+        if margin > 2e-5:
+            assert int(tok[i]) == t, f"draw {i}: kernel {int(tok[i])}, plain {t}"
+            assert abs(float(lp[i]) - logprob) < 1e-4
+            agree += 1
+    assert agree > 0.85 * n
+
+
+def test_sample_rows_are_independent(gpu):
+    logits = rnd(8, 331, seed=82, scale=2.0)
+    temp = torch.tensor([0.0, 1.0, 0.5, 2.0, 1.0, 0.0, 1.0, 0.7])
+    topk = torch.tensor([-1, -1, 10, -1, 1, -1, 50, -1], dtype=torch.int32)
+    seeds = torch.arange(8, dtype=torch.int64) * 1000 + 3
+    draw = torch.tensor([0, 5, 2, 9, 1, 0, 7, 3], dtype=torch.int32)
+    tok, lp = _sample(gpu, logits, temperature=temp, top_k=topk, seed=seeds, draw=draw)
+    for r in range(8):  # the same row alone gives the same token
+        t1, l1 = _sample(gpu, logits[r : r + 1], temperature=temp[r : r + 1], top_k=topk[r : r + 1],
+                         seed=seeds[r : r + 1], draw=draw[r : r + 1])
+        assert int(t1[0]) == int(tok[r]) and abs(float(l1[0]) - float(lp[r])) < 1e-6

@@ -1,0 +1,271 @@
+"""The parts alone, and models put together from parts as data: a windowed layer, a
+layer that runs twice, a layer that reads another layer's cache, and a toy mixer with
+state of its own that is defined here and registered without touching the framework."""
+
+import numpy as np
+import pytest
+import torch
+from pydantic import BaseModel
+
+import plain_llama as P
+import replay
+import tiny
+from halite_amd.config import LayerRun, LayerSpec, ModelConfig, ModelSpec, PartSpec, ServerConfig, parse_config
+from halite_amd.engine.batch import Segment
+from halite_amd.engine.runner import ModelRunner
+from halite_amd.parts import MIXERS, BuildContext, Decoder, Mixer, ParamDecl, StateNeed
+from halite_amd.parts.base import FEED_FORWARDS, NORMS, POSITIONS
+from halite_amd.weights import fill_random
+
+pytestmark = pytest.mark.gpu
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 5e-5, "bfloat16": 2.5e-2}
+
+
+def build(gpu, dtype):
+    return BuildContext(dtype=DT[dtype], device=gpu, hidden_size=0)
+
+
+def fill(part, dtype, seed=0, std=0.05):
+    """Random tensors for one part, returned as float32 CPU copies by name."""
+    decls = part.param_decls()
+    views = part.allocate({n: DT[dtype] for n in decls})
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, d in decls.items():
+        t = 1 + 0.1 * torch.randn(d.shape, generator=g) if d.init == "ones" else std * torch.randn(d.shape, generator=g)
+        views[name].copy_(t)
+        out[name] = views[name].float().cpu()
+    part.finalize()
+    return out
+
+
+@pytest.mark.parametrize("raw", [tiny.TINY_A, tiny.TINY_B, tiny.TINY_C])
+def test_rope_part(gpu, raw):
+    arch, cfg = parse_config(raw)
+    rope = POSITIONS.build(arch.to_spec(cfg).positions["rope"], build(gpu, "float32"))
+    want = P.rope_frequencies_of(raw)
+    assert torch.equal(rope.inv_freq, want)
+    cos, sin = rope.tables(100)
+    c, s = P.rotation_table(torch.arange(cos.shape[0]), want)
+    assert torch.equal(cos.cpu(), c) and torch.equal(sin.cpu(), s)
+    more = rope.tables(cfg.max_position_embeddings)[0]
+    assert more.shape[0] >= cfg.max_position_embeddings and torch.equal(more[:100].cpu(), c[:100])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_norm_and_feed_forward_parts(gpu, dtype):
+    b = build(gpu, dtype)
+    norm = NORMS.build(PartSpec(kind="rmsnorm", size=120, eps=1e-5), b)
+    w = fill(norm, dtype, 1)["weight"]
+    h = torch.randn(70, 120, generator=torch.Generator().manual_seed(2))
+    got = norm.forward(h.to(gpu).clone())
+    err = float((got.float().cpu() - P.rms_norm(h, w, 1e-5)).abs().max())
+    assert err < (1e-5 if dtype == "float32" else 3e-2)
+
+    ff = FEED_FORWARDS.build(PartSpec(kind="gated", hidden_size=120, intermediate_size=200, activation="silu"), b)
+    ws = fill(ff, dtype, 3, std=0.1)
+    for rows in (5, 64, 70):  # the fused small-batch kernel and the large-batch path
+        x = torch.randn(rows, 120, generator=torch.Generator().manual_seed(rows)).to(DT[dtype])
+        want = P.gated_feed_forward(x.float(), ws["linear_gate.weight"], ws["linear_proj.weight"], ws["linear_out.weight"])
+        got = ff.forward(x.to(gpu), None).float().cpu()
+        assert float((got - want).abs().max()) < (2e-5 if dtype == "float32" else 2e-2) * max(1.0, float(want.abs().max()))
+    with pytest.raises(Exception, match="silu"):
+        FEED_FORWARDS.build(PartSpec(kind="gated", hidden_size=8, intermediate_size=8, activation="gelu"), b)
+    with pytest.raises(Exception, match="unknown norm kind"):
+        NORMS.build(PartSpec(kind="layernorm", size=8), b)
+
+
+# -- models from hand-written specs ---------------------------------------------------
+
+
+def toy_spec(layers: dict, order: list, d=64, vocab=97, head_dim=16, rot=16, interleaved=False, max_pos=512):
+    norm = PartSpec(kind="rmsnorm", size=d, eps=1e-5)
+    return ModelSpec(
+        architecture="toy", vocab_size=vocab, hidden_size=d, max_positions=max_pos,
+        embedding=PartSpec(kind="embedding", vocab_size=vocab, size=d),
+        positions={"rope": PartSpec(kind="rope", head_dim=head_dim, rotary_dim=rot, theta=10000.0,
+                                    interleaved=interleaved, max_positions=max_pos)},
+        layers={
+            name: LayerSpec(mixer_norm=norm, mixer=mixer, ff_norm=norm,
+                            ff=PartSpec(kind="gated", hidden_size=d, intermediate_size=2 * d + 8, activation="silu"))
+            for name, mixer in layers.items()
+        },
+        order=order, final_norm=norm, head=PartSpec(kind="linear_head", vocab_size=vocab, size=d, tied=True),
+    )
+
+
+def attention_spec(d=64, heads=4, kv=2, head_dim=16, window=None, position="rope"):
+    return PartSpec(kind="attention", hidden_size=d, n_heads=heads, n_kv_heads=kv, head_dim=head_dim,
+                    scale=head_dim**-0.5, position=position, window=window)
+
+
+def make_runner(gpu, spec, dtype, tokens=1024, page=16):
+    model = Decoder(spec, DT[dtype], gpu)
+    fill_random(model, seed=5, std=0.08)
+    return ModelRunner(model, ServerConfig(kv_cache_num_tokens=tokens, page_size=page, max_seqs_per_forward=8),
+                       ModelConfig(dtype=dtype))
+
+
+def plain_attention_layer(att, x, positions, rope_p, cached_kv=None):
+    """One attention mixer from the plain functions; returns (output, (k, v))."""
+    p = att.p
+    w = att.w_qkv.float().cpu()
+    nq, nk = p.n_heads * p.head_dim, p.n_kv_heads * p.head_dim
+    n = x.shape[0]
+    q = (x @ w[:nq].T).view(n, p.n_heads, p.head_dim)
+    if p.position is not None:
+        inv = P.inverse_frequencies(rope_p["rotary_dim"], rope_p["theta"])
+        cos, sin = P.rotation_table(positions, inv)
+        rotate = P.rotate_interleaved if rope_p["interleaved"] else P.rotate_half_split
+        rot = rope_p["rotary_dim"]
+        q = torch.cat((rotate(q[..., :rot], cos, sin), q[..., rot:]), -1)
+    if cached_kv is None:
+        k = (x @ w[nq : nq + nk].T).view(n, p.n_kv_heads, p.head_dim)
+        v = (x @ w[nq + nk :].T).view(n, p.n_kv_heads, p.head_dim)
+        if p.position is not None:
+            k = torch.cat((rotate(k[..., :rot], cos, sin), k[..., rot:]), -1)
+    else:
+        k, v = cached_kv
+    a = P.causal_attention(q, k, v, window=p.window)
+    return a.reshape(n, nq) @ att.w_out.float().cpu().T, (k, v)
+
+
+def plain_model(model, ids, mixers: dict):
+    """The whole toy model from plain functions; ``mixers[layer name]`` is a function
+    ``(mixer part, x, positions, run index, memo) -> delta`` ."""
+    spec = model.spec
+    ids = torch.as_tensor(ids)
+    positions = torch.arange(len(ids))
+    h = P.embed(ids, model.embedding.weight.float().cpu())
+    memo = {}
+    for i, run in enumerate(spec.order):
+        blk = model.layers[run.layer]
+        x = P.rms_norm(h, blk.mixer_norm.weight.float().cpu(), blk.mixer_norm.p.eps)
+        h = h + mixers[run.layer](blk.mixer, x, positions, i, run, memo)
+        x = P.rms_norm(h, blk.ff_norm.weight.float().cpu(), blk.ff_norm.p.eps)
+        f = blk.ff.p.intermediate_size
+        wgu = blk.ff.w_gate_up.float().cpu()
+        h = h + P.gated_feed_forward(x, wgu[:f], wgu[f:], blk.ff.w_out.float().cpu())
+    h = P.rms_norm(h, model.final_norm.weight.float().cpu(), model.final_norm.p.eps)
+    return P.output_head(h, model.embedding.weight.float().cpu())
+
+
+def replay_all(runner, requests, ref, tol, vocab):
+    for make in (replay.whole, replay.tail_one_by_one, replay.portions, replay.mixed):
+        trace = make(requests)
+        rows = replay.collect(trace, replay.run_trace(runner, trace), vocab)
+        replay.compare(rows, ref, tol)
+    assert runner.cache.idle()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_window_partial_rotation_and_a_layer_without_positions(gpu, dtype):
+    """Three different mixers in one model: a window of 20 tokens with the adjacent
+    pairing on half of the head, full attention, and attention without positions.
+    The windowed layers have pages of their own, and give them back."""
+    rope_p = dict(rotary_dim=8, theta=10000.0, interleaved=True)
+    spec = toy_spec(
+        {"win": attention_spec(window=20), "full": attention_spec(kv=4), "nopos": attention_spec(kv=1, position=None)},
+        [LayerRun(layer="win"), LayerRun(layer="full"), LayerRun(layer="nopos"), LayerRun(layer="win")],
+        rot=8, interleaved=True,
+    )
+    runner = make_runner(gpu, spec, dtype, tokens=640)
+    assert len(runner.cache.groups) == 3 and runner.cache.groups[0].runs == [0, 3]
+
+    def att(part, x, positions, i, run, memo):
+        return plain_attention_layer(part, x, positions, rope_p)[0]
+
+    requests = {f"r{i}": [int(t) % 97 for t in tiny.random_tokens(tiny.TINY_A, n, 70 + i)] for i, n in enumerate([90, 33, 150, 7])}
+    ref = {rid: plain_model(runner.model, toks, {"win": att, "full": att, "nopos": att}) for rid, toks in requests.items()}
+    replay_all(runner, requests, ref, TOL[dtype], 97)
+    # a long request holds only the window's pages in the windowed group
+    s = runner.admit()
+    runner.step([Segment(s, 0, requests["r2"], [])])
+    win, full = runner.cache.groups[0], runner.cache.groups[1]
+    assert sum(p >= 0 for p in win.tables[s]) <= 20 // 16 + 2 < sum(p >= 0 for p in full.tables[s]) == -(-150 // 16)
+    runner.free(s)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_twice_and_a_borrowed_cache(gpu, dtype):
+    """The run order names layer ``a`` twice (each run has a cache of its own) and
+    lets the last run of ``b`` read the keys and values that run 1 wrote."""
+    rope_p = dict(rotary_dim=16, theta=10000.0, interleaved=False)
+    spec = toy_spec(
+        {"a": attention_spec(), "b": attention_spec(heads=8, kv=2, head_dim=16)},
+        [LayerRun(layer="a"), LayerRun(layer="b"), LayerRun(layer="a"), LayerRun(layer="b", cache_from=1)],
+    )
+    runner = make_runner(gpu, spec, dtype)
+    assert sorted(runner.cache.group_of_run) == [0, 1, 2, 3]
+    assert runner.model.runs[3].kv is runner.model.runs[1].kv and not runner.model.runs[3].appends
+    assert runner.model.runs[2].kv is not runner.model.runs[0].kv
+
+    def att(part, x, positions, i, run, memo):
+        if run.cache_from is not None:
+            return plain_attention_layer(part, x, positions, rope_p, cached_kv=memo[run.cache_from])[0]
+        out, memo[i] = plain_attention_layer(part, x, positions, rope_p)
+        return out
+
+    requests = {f"r{i}": [int(t) % 97 for t in tiny.random_tokens(tiny.TINY_A, n, 80 + i)] for i, n in enumerate([70, 5, 41])}
+    ref = {rid: plain_model(runner.model, toks, {"a": att, "b": att}) for rid, toks in requests.items()}
+    replay_all(runner, requests, ref, TOL[dtype], 97)
+
+
+# -- a toy mixer with state of its own, defined and registered here ---------------------
+
+
+class RunningMeanParams(BaseModel):
+    hidden_size: int
+
+
+@MIXERS.register("running_mean")
+class RunningMean(Mixer):
+    """``y_t = W * mean(x_0 .. x_t)``: no cache pages, but a per-request state (the sum
+    so far and the count) that carries from one step to the next."""
+
+    Params = RunningMeanParams
+
+    def param_decls(self):
+        return {"w.weight": ParamDecl((self.p.hidden_size, self.p.hidden_size))}
+
+    def state_need(self):
+        return {"sum": StateNeed((self.p.hidden_size,), torch.float32), "count": StateNeed((1,), torch.float32)}
+
+    def forward(self, x, ctx, run):
+        out = torch.empty_like(x, dtype=torch.float32)
+        for seg, q0, n in zip(ctx.segments, ctx.seg_q_start_host, ctx.seg_q_len_host):
+            xs = x[q0 : q0 + n].float()
+            total = run.state["sum"][seg.slot] + torch.cumsum(xs, 0)
+            count = run.state["count"][seg.slot] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)[:, None]
+            out[q0 : q0 + n] = total / count
+            run.state["sum"][seg.slot] = total[-1]
+            run.state["count"][seg.slot] = count[-1]
+        return (out @ self.w_weight.float().T).to(x.dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped(gpu, dtype):
+    spec = toy_spec(
+        {"mean": PartSpec(kind="running_mean", hidden_size=64), "att": attention_spec()},
+        [LayerRun(layer="mean"), LayerRun(layer="att"), LayerRun(layer="mean")],
+    )
+    runner = make_runner(gpu, spec, dtype)
+    assert len(runner.cache.groups) == 1 and runner.cache.groups[0].runs == [1]
+    assert set(runner.cache.state.tensors) == {0, 2}  # each run of the layer has its own state rows
+    rope_p = dict(rotary_dim=16, theta=10000.0, interleaved=False)
+
+    def mean(part, x, positions, i, run, memo):
+        m = torch.cumsum(x, 0) / torch.arange(1, x.shape[0] + 1)[:, None]
+        return m @ part.w_weight.float().cpu().T
+
+    def att(part, x, positions, i, run, memo):
+        return plain_attention_layer(part, x, positions, rope_p)[0]
+
+    requests = {f"r{i}": [int(t) % 97 for t in tiny.random_tokens(tiny.TINY_A, n, 90 + i)] for i, n in enumerate([60, 3, 35, 18])}
+    ref = {rid: plain_model(runner.model, toks, {"mean": mean, "att": att}) for rid, toks in requests.items()}
+    replay_all(runner, requests, ref, TOL[dtype], 97)
+    # a slot starts from zero again when the next request takes it
+    s = runner.admit()
+    assert float(runner.cache.state.tensors[0]["sum"][s].abs().sum()) == 0
+    runner.free(s)

@@ -1,0 +1,246 @@
+"""Pins of the plain implementation: what fixes each formula beside the reference's
+text.  Each check is chosen so that a plausible mistake (a wrong sign or pairing, a
+norm in the wrong place, a wrong head mapping) fails it.  The reference holds no test
+vectors for generation (its ``test/`` scripts print text for a human), so library
+special cases and invariants stand in for them."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_llama as P
+import tiny
+
+
+def test_inverse_frequencies_closed_form():
+    f = P.inverse_frequencies(16, 10000.0)
+    want = torch.tensor([10000.0 ** (-2 * j / 16) for j in range(8)])
+    assert torch.allclose(f, want, rtol=1e-6)
+    assert f[0] == 1.0 and f.shape == (8,)
+
+
+def test_llama3_scaling_bands():
+    # tiny B: original context 64, factor 8, low 1, high 4: all three bands occur
+    f = P.inverse_frequencies(32, 500000.0)
+    g = P.llama3_scaled_frequencies(f, 8.0, 1.0, 4.0, 64)
+    wl = 2 * math.pi / f
+    high, low = wl < 64 / 4.0, wl > 64 / 1.0
+    mid = ~high & ~low
+    assert high.any() and low.any() and mid.any()
+    assert torch.equal(g[high], f[high])  # short wavelengths untouched
+    assert torch.allclose(g[low], f[low] / 8.0, rtol=1e-6)  # long ones divided
+    assert ((g[mid] < f[mid]) & (g[mid] > f[mid] / 8.0)).all()  # between, strictly
+    assert (g[:-1] > g[1:]).all()  # still decreasing: no jump at a band's edge
+    # factor 1 is the identity
+    assert torch.allclose(P.llama3_scaled_frequencies(f, 1.0, 1.0, 4.0, 64), f, rtol=1e-6)
+
+
+def test_llama3_scaling_matches_two_where_form():
+    # the reference's vectorised form (src/halite/transformers/position.py:264-284)
+    f = P.inverse_frequencies(64, 500000.0)
+    orig, factor, lo, hi = 8192, 8.0, 1.0, 4.0
+    wl = 2 * math.pi / f
+    a = torch.where(wl > orig / lo, f / factor, f)
+    s = (orig / wl - lo) / (hi - lo)
+    b = (1 - s) * a / factor + s * a
+    want = torch.where(~(wl < orig / hi) & ~(wl > orig / lo), b, a)
+    assert torch.allclose(P.llama3_scaled_frequencies(f, factor, lo, hi, orig), want, rtol=1e-6)
+
+
+def _qk(n=7, heads=3, d=16, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(n, heads, d, generator=g), torch.randn(n, heads, d, generator=g)
+
+
+@pytest.mark.parametrize("rotate", [P.rotate_half_split, P.rotate_interleaved])
+def test_rotation_is_a_rotation(rotate):
+    q, _ = _qk()
+    f = P.inverse_frequencies(16, 10000.0)
+    cos, sin = P.rotation_table(torch.arange(7), f)
+    r = rotate(q, cos, sin)
+    assert torch.allclose(r[0], q[0], atol=1e-6)  # position 0: identity
+    assert torch.allclose(r.norm(dim=-1), q.norm(dim=-1), rtol=1e-5)  # norms kept
+    assert not torch.allclose(r[3], q[3], atol=1e-3)
+
+
+@pytest.mark.parametrize("rotate", [P.rotate_half_split, P.rotate_interleaved])
+def test_rotation_scores_depend_on_distance_only(rotate):
+    q, k = _qk()
+    f = P.inverse_frequencies(16, 10000.0)
+    scores = []
+    for shift in (0, 5, 40):
+        cos, sin = P.rotation_table(torch.arange(7) + shift, f)
+        rq, rk = rotate(q, cos, sin), rotate(k, cos, sin)
+        scores.append(torch.einsum("ihd,jhd->hij", rq, rk))
+    assert torch.allclose(scores[0], scores[1], atol=1e-4)
+    assert torch.allclose(scores[0], scores[2], atol=1e-4)
+
+
+def test_rotation_sign_and_pairing():
+    # one pair, angle pi/2: (1, 0) -> (0, 1); a flipped sign gives (0, -1)
+    x = torch.zeros(1, 1, 4)
+    x[0, 0, 0] = 1.0
+    cos, sin = torch.zeros(1, 2), torch.zeros(1, 2)
+    cos[0, 1] = 1.0
+    sin[0, 0] = 1.0
+    h = P.rotate_half_split(x, cos, sin)
+    assert torch.allclose(h[0, 0], torch.tensor([0.0, 0.0, 1.0, 0.0]))  # partner of 0 is 2
+    i = P.rotate_interleaved(x, cos, sin)
+    assert torch.allclose(i[0, 0], torch.tensor([0.0, 1.0, 0.0, 0.0]))  # partner of 0 is 1
+
+
+def test_two_pairings_agree_under_the_permutation():
+    # the adjacent pairing on x equals the half-split pairing on x with its
+    # dimensions reordered [0, 2, 4, ..., 1, 3, 5, ...]
+    q, _ = _qk(d=16)
+    f = P.inverse_frequencies(16, 10000.0)
+    cos, sin = P.rotation_table(torch.arange(7) + 3, f)
+    perm = torch.cat((torch.arange(0, 16, 2), torch.arange(1, 16, 2)))
+    a = P.rotate_interleaved(q, cos, sin)[..., perm]
+    b = P.rotate_half_split(q[..., perm], cos, sin)
+    assert torch.allclose(a, b, atol=1e-6)
+
+
+def test_complex_form_equals_the_interleaved_rotation():
+    # src/halite/transformers/position.py:294-300 multiplies complex numbers
+    q, _ = _qk()
+    f = P.inverse_frequencies(16, 10000.0)
+    ang = torch.outer(torch.arange(7).float(), f)
+    cis = torch.polar(torch.ones_like(ang), ang).unsqueeze(1)
+    want = torch.view_as_real(torch.view_as_complex(q.reshape(7, 3, 8, 2)) * cis).flatten(-2)
+    assert torch.allclose(P.rotate_interleaved(q, ang.cos(), ang.sin()), want, atol=1e-6)
+
+
+def test_rms_norm():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(5, 24, generator=g) * 3
+    w = torch.randn(24, generator=g)
+    want = F.rms_norm(x, (24,), None, 1e-5) * w
+    assert torch.allclose(P.rms_norm(x, w, 1e-5), want, atol=1e-6)
+    # invariant to the scale of x (for a small eps); the mean is over the width
+    assert torch.allclose(P.rms_norm(7 * x, w, 1e-12), P.rms_norm(x, w, 1e-12), atol=1e-5)
+    unit = x / x.pow(2).mean(-1, keepdim=True).sqrt()
+    assert torch.allclose(P.rms_norm(unit, torch.ones(24), 1e-12), unit, atol=1e-5)
+    # eps is inside the root
+    tiny_x = torch.full((1, 4), 1e-4)
+    assert torch.allclose(P.rms_norm(tiny_x, torch.ones(4), 1.0), tiny_x / math.sqrt(1e-8 + 1.0), rtol=1e-5)
+
+
+def test_gated_feed_forward():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(4, 8, generator=g)
+    wg, wu, wd = (torch.randn(s, generator=g) for s in ((12, 8), (12, 8), (8, 12)))
+    want = F.linear(F.silu(F.linear(x, wg)) * F.linear(x, wu), wd)
+    assert torch.allclose(P.gated_feed_forward(x, wg, wu, wd), want, atol=1e-5)
+    # gate and up are not interchangeable
+    assert not torch.allclose(P.gated_feed_forward(x, wu, wg, wd), want, atol=1e-3)
+
+
+@pytest.mark.parametrize("heads,kv", [(4, 4), (4, 2), (6, 1), (6, 2)])
+def test_attention_reduces_to_sdpa(heads, kv):
+    g = torch.Generator().manual_seed(3)
+    n, d = 9, 8
+    q = torch.randn(n, heads, d, generator=g)
+    k = torch.randn(n, kv, d, generator=g)
+    v = torch.randn(n, kv, d, generator=g)
+    want = F.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None], is_causal=True, enable_gqa=True
+    )[0].transpose(0, 1)
+    assert torch.allclose(P.causal_attention(q, k, v), want, atol=1e-5)
+
+
+def test_attention_special_cases():
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn(6, 4, 8, generator=g)
+    k = torch.randn(6, 2, 8, generator=g)
+    v = torch.randn(6, 2, 8, generator=g)
+    out = P.causal_attention(q, k, v)
+    # the first token sees itself only: its output is its value, per group
+    assert torch.allclose(out[0, 0], v[0, 0], atol=1e-6) and torch.allclose(out[0, 3], v[0, 1], atol=1e-6)
+    # later keys never change an earlier row
+    k2, v2 = k.clone(), v.clone()
+    k2[4:] += 5.0
+    v2[4:] -= 3.0
+    assert torch.allclose(P.causal_attention(q, k2, v2)[:4], out[:4], atol=1e-6)
+    # the same value everywhere comes out unchanged
+    same = v[:1].expand(6, 2, 8)
+    assert torch.allclose(P.causal_attention(q, k, same), same.repeat_interleave(2, 1), atol=1e-5)
+    # a window of 1 sees only the token itself; a window beyond the length changes nothing
+    assert torch.allclose(P.causal_attention(q, k, v, window=1), v.repeat_interleave(2, 1), atol=1e-6)
+    assert torch.allclose(P.causal_attention(q, k, v, window=6), out, atol=1e-6)
+    assert not torch.allclose(P.causal_attention(q, k, v, window=2), out, atol=1e-3)
+
+
+def test_attention_scale_is_inverse_root_of_head_size():
+    # one query against two keys: probabilities follow from the scaled scores
+    q = torch.tensor([[[0.0] * 16], [[2.0] + [0.0] * 15]])
+    k = torch.tensor([[[4.0] + [0.0] * 15], [[0.0] * 16]])
+    v = torch.tensor([[[1.0] + [0.0] * 15], [[0.0] * 16]])
+    out = P.causal_attention(q, k, v)
+    p = torch.softmax(torch.tensor([2.0 * 4.0 / 4.0, 0.0]), 0)[0]
+    assert torch.allclose(out[1, 0, 0], p, atol=1e-6)
+
+
+def test_model_shift_invariance_and_causality():
+    cfg = tiny.TINY_B
+    w = tiny.random_weights(cfg, 7, std=0.05)
+    ids = tiny.random_tokens(cfg, 12, 1)
+    a = P.forward(cfg, w, ids)
+    b = P.forward(cfg, w, ids, position_offset=17)
+    assert torch.allclose(a, b, atol=2e-5)  # only distances count
+    c = P.forward(cfg, w, ids[:8])
+    assert torch.allclose(a[:8], c, atol=1e-5)  # a prefix's logits do not see the rest
+    # tied head: the logits are hidden @ embedding^T
+    assert "lm_head.weight" not in w
+
+
+def test_norm_weight_position_matters():
+    cfg = tiny.TINY_A
+    w = tiny.random_weights(cfg, 8, std=0.05)
+    ids = tiny.random_tokens(cfg, 6, 2)
+    a = P.forward(cfg, w, ids)
+    w2 = dict(w)
+    w2["model.layers.0.input_layernorm.weight"], w2["model.layers.0.post_attention_layernorm.weight"] = (
+        w["model.layers.0.post_attention_layernorm.weight"],
+        w["model.layers.0.input_layernorm.weight"],
+    )
+    assert not torch.allclose(a, P.forward(cfg, w2, ids), atol=1e-4)
+
+
+def test_uniform_draw_is_a_uniform_stream():
+    us = [P.uniform_draw(123, i) for i in range(4000)]
+    assert all(0.0 <= u < 1.0 for u in us)
+    assert abs(sum(us) / len(us) - 0.5) < 0.02
+    assert len(set(us)) > 3990
+    assert P.uniform_draw(123, 5) == P.uniform_draw(123, 5) != P.uniform_draw(124, 5)
+
+
+def test_filters():
+    logits = torch.log(torch.tensor([0.5, 0.2, 0.2, 0.06, 0.04]))
+    p = P.filtered_probabilities(logits, 1.0)
+    assert torch.allclose(p, torch.tensor([0.5, 0.2, 0.2, 0.06, 0.04], dtype=p.dtype), atol=1e-6)
+    p = P.filtered_probabilities(logits, 1.0, top_k=2)  # the tie at 0.2 stays whole
+    assert (p > 0).tolist() == [True, True, True, False, False]
+    p = P.filtered_probabilities(logits, 1.0, top_p=0.6)
+    assert (p > 0).tolist() == [True, True, True, False, False]
+    p = P.filtered_probabilities(logits, 1.0, top_p=0.45)
+    assert (p > 0).tolist() == [True, False, False, False, False]
+    p = P.filtered_probabilities(logits, 1.0, min_p=0.2)  # p >= 0.2 * 0.5
+    assert (p > 0).tolist() == [True, True, True, False, False]
+    assert abs(float(p.sum()) - 1.0) < 1e-9
+    hot = P.filtered_probabilities(logits, 0.05)
+    assert hot[0] > 0.999  # temperature -> 0 approaches the maximum
+
+
+def test_sample_token_greedy_and_draw():
+    logits = torch.tensor([0.1, 2.0, 2.0, -1.0])
+    tok, lp, _ = P.sample_token(logits, {"temperature": 0.0}, 0)
+    assert tok == 1 and abs(lp - float(torch.log_softmax(logits.double(), -1)[1])) < 1e-9
+    assert P.sample_token(logits, {"top_k": 1, "temperature": 0.7}, 0)[0] == 1
+    counts = torch.zeros(4)
+    for i in range(3000):
+        counts[P.sample_token(logits, {"temperature": 1.0, "seed": 9}, i)[0]] += 1
+    want = torch.softmax(logits, -1) * 3000
+    assert ((counts - want).abs() < 4 * want.sqrt() + 5).all()

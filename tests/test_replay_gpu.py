@@ -1,0 +1,170 @@
+"""Replay on the GPU: the same requests whole, with the last 32 tokens decoded one by
+one, in portions of changing size, and mixed with other requests so that pages are used
+again; in 32-bit and in bfloat16; each compared with the plain implementation run on
+the whole sequence.  A difference that shows in one way of cutting only is a fault of
+the cache or the batch."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama
+import replay
+import tiny
+from halite_amd.config import ModelConfig, ServerConfig
+from halite_amd.engine.runner import ModelRunner
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TOL = {"float32": 5e-5, "bfloat16": 2.5e-2}  # of the largest logit
+CONFIGS = {"A": tiny.TINY_A, "B": tiny.TINY_B, "C": tiny.TINY_C}
+LENGTHS = {"A": [5, 17, 33, 64, 100, 128], "B": [1, 40, 100, 2, 256, 65], "C": [130, 64, 31, 200, 3, 97]}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    """One model folder per configuration and stored type, and the plain logits of
+    every request's whole sequence (from the stored, i.e. rounded, weights)."""
+    out = {}
+    for name, cfg in CONFIGS.items():
+        weights = tiny.random_weights(cfg, seed=11 + len(name), std=0.06)
+        requests = {f"r{i}": tiny.random_tokens(cfg, n, 100 + i) for i, n in enumerate(LENGTHS[name])}
+        for dtype, store in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+            folder = str(tmp_path_factory.mktemp(f"{name}_{dtype}"))
+            tiny.write_model_folder(folder, cfg, weights, store)
+            pc, pw = plain_llama.read_model_folder(folder)
+            ref = {rid: plain_llama.forward(pc, pw, toks) for rid, toks in requests.items()}
+            out[(name, dtype)] = (folder, requests, ref)
+    return out
+
+
+def make_runner(folder, dtype, tokens, page_size=64):
+    server = ServerConfig(kv_cache_num_tokens=tokens, page_size=page_size, max_seqs_per_forward=8)
+    return ModelRunner.from_pretrained(folder, server, ModelConfig(dtype=dtype))
+
+
+SCHEDULES = {
+    "whole": replay.whole,
+    "tail": replay.tail_one_by_one,
+    "portions": replay.portions,
+    "mixed": replay.mixed,
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("schedule", list(SCHEDULES))
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_schedules(folders, name, schedule, dtype):
+    folder, requests, ref = folders[(name, dtype)]
+    trace = SCHEDULES[schedule](requests)
+    page = 16 if name == "B" else 64
+    # exactly as many pages as the trace needs at its peak: they are used again
+    runner = make_runner(folder, dtype, replay.peak_tokens(trace, page), page)
+    # whatever free or not yet written slots hold must never reach a result
+    for g in runner.cache.groups:
+        g.storage.fill_(float("nan"))
+    logits = replay.run_trace(runner, trace)
+    rows = replay.collect(trace, logits, CONFIGS[name]["vocab_size"])
+    assert sum(len(v) for v in rows.values()) > 0
+    replay.compare(rows, ref, TOL[dtype])
+    assert runner.cache.idle()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cuts_agree_with_each_other(folders, dtype):
+    """The logits at a position do not depend on how the tokens were cut, beyond
+    rounding: far tighter than the distance to the plain implementation in bf16."""
+    folder, requests, _ = folders[("C", dtype)]
+    results = []
+    for schedule in ("whole", "tail", "portions"):
+        trace = SCHEDULES[schedule](requests)
+        runner = make_runner(folder, dtype, replay.peak_tokens(trace))
+        results.append(replay.collect(trace, replay.run_trace(runner, trace), 331))
+    tol = 2e-5 if dtype == "float32" else 1.5e-2
+    for other in results[1:]:
+        for rid in results[0]:
+            a = torch.stack([results[0][rid][p] for p in sorted(results[0][rid])])
+            b = torch.stack([other[rid][p] for p in sorted(other[rid])])
+            assert float((a - b).abs().max()) <= tol * max(1.0, float(a.abs().max()))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_small_pages_and_other_page_sizes(folders, dtype):
+    folder, requests, ref = folders[("A", dtype)]
+    trace = replay.mixed(requests, seed=3)
+    for page in ([1, 4, 8, 16] if dtype == "float32" else [8, 16, 32]):
+        runner = make_runner(folder, dtype, replay.peak_tokens(trace, page), page)
+        rows = replay.collect(trace, replay.run_trace(runner, trace), 256)
+        replay.compare(rows, ref, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_and_long_decoding(folders, dtype):
+    folder, requests, ref = folders[("C", dtype)]
+    rid = "r3"  # 200 tokens
+    toks = requests[rid]
+    # every token on its own, from an empty cache
+    trace = [{"step": i, "entries": [{"id": rid, "tokens": [t], "want": [0]}], "end": [rid] if i == len(toks) - 1 else []}
+             for i, t in enumerate(toks)]
+    runner = make_runner(folder, dtype, 256)
+    rows = replay.collect(trace, replay.run_trace(runner, trace), 331)
+    replay.compare(rows, ref, TOL[dtype])
+    # the first tokens of a sequence: one token, two tokens
+    for n in (1, 2):
+        trace = [{"step": 0, "entries": [{"id": rid, "tokens": toks[:n], "want": list(range(n))}], "end": [rid]}]
+        rows = replay.collect(trace, replay.run_trace(runner, trace), 331)
+        replay.compare(rows, ref, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(folders, dtype, tmp_path):
+    """The program itself, as a user runs it: JSON lines in, <step>.f32 files out."""
+    folder, requests, ref = folders[("B", dtype)]
+    trace = replay.mixed(requests, seed=1)
+    out = tmp_path / "out"
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+           "--out", str(out), "--max-tokens", str(replay.peak_tokens(trace))]
+    proc = subprocess.run(cmd, input="\n".join(json.dumps(s) for s in trace) + "\n", text=True,
+                          capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.split("\n") if l] == [f"done {s['step']}" for s in trace]
+    logits = {}
+    for s in trace:
+        n_want = sum(len(e["want"]) for e in s["entries"])
+        path = out / f"{s['step']}.f32"
+        if n_want == 0:
+            assert not path.exists()
+            continue
+        logits[s["step"]] = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(n_want, 512))
+    rows = replay.collect(trace, logits, 512)
+    replay.compare(rows, ref, TOL[dtype])
+
+
+def test_refusals(folders):
+    from halite_amd.cache import NoSpace
+    from halite_amd.engine.batch import Segment
+    from halite_amd.engine.runner import StepError
+
+    folder, requests, _ = folders[("A", "float32")]
+    runner = make_runner(folder, "float32", 128)
+    s = runner.admit()
+    with pytest.raises(StepError, match="outside the vocabulary"):
+        runner.step([Segment(s, 0, [5, 256], [0])])
+    with pytest.raises(StepError, match="are cached"):
+        runner.step([Segment(s, 3, [5], [0])])
+    with pytest.raises(StepError, match="twice"):
+        runner.step([Segment(s, 0, [5], [0]), Segment(s, 1, [6], [0])])
+    with pytest.raises(StepError, match="context length"):
+        runner.step([Segment(s, 0, list(range(129)), [])])
+    runner.step([Segment(s, 0, list(range(100)), [])])
+    s2 = runner.admit()
+    with pytest.raises(NoSpace):
+        runner.step([Segment(s2, 0, list(range(100)), [])])  # 2 pages of 64 in all
+    assert runner.cache.length(s2) == 0
+    runner.cache.check()
