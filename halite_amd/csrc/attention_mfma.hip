@@ -98,23 +98,71 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   float m = -INFINITY, l = 0.f;
 
   const int last_key = kv_len - 1;  // keys beyond it are not written yet
-  for (int j0 = kv_begin & ~31; j0 < kv_end; j0 += 32) {
+
+  // This lane's key of tile t in the block of 32 keys at j0: row `col` of tile t is
+  // key j0 + (col/4)*8 + t*4 + col%4; its eight keys for the values are j0 + quad*8 .. +8.
+  // Keys outside [kv_begin, last_key] are clamped for the address only; their scores
+  // are masked and their values cleared.  Page numbers are looked up one block ahead
+  // of the loads that need them, so that no load waits for a table entry.
+  auto key_index = [&](int j0, int t) {
+    const int j = j0 + (col / 4) * 8 + t * 4 + (col % 4);
+    return j < kv_begin ? kv_begin : (j > last_key ? last_key : j);
+  };
+  auto value_index = [&](int j0) {
+    int jv = j0 + quad * 8;
+    if (jv < (kv_begin & ~7)) jv = kv_begin & ~7;
+    if (jv > (last_key & ~7)) jv = last_key & ~7;
+    return jv;
+  };
+  auto load_keys = [&](int j0, const int (&pages)[2], bf16x8 (&kf)[2][KT]) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int j = key_index(j0, t);
+      const bf16_t* kp = k_pages + (((size_t)pages[t] * K + g) * page_size + (j % page_size)) * D;
+#pragma unroll
+      for (int ks = 0; ks < KT; ++ks) {
+        const int d0 = ks * 32 + quad * 8;
+        kf[t][ks] = d0 < D ? ld16(kp + d0) : zero8();
+      }
+    }
+  };
+
+  const int j_first = kv_begin & ~31;
+  bf16x8 kcur[2][KT], knext[2][KT];
+  int kpage[2], vpage;  // pages of the NEXT key block and of THIS value block
+  if (j_first < kv_end) {
+    kpage[0] = bt[key_index(j_first, 0) / page_size];
+    kpage[1] = bt[key_index(j_first, 1) / page_size];
+    vpage = bt[value_index(j_first) / page_size];
+    load_keys(j_first, kpage, kcur);
+    kpage[0] = bt[key_index(j_first + 32, 0) / page_size];
+    kpage[1] = bt[key_index(j_first + 32, 1) / page_size];
+  }
+
+  for (int j0 = j_first; j0 < kv_end; j0 += 32) {
+    // ---- issue this block's value loads and the next block's key loads first --------
+    // lane loads V^T[dim dt*16 + col][keys jv .. jv+8]
+    const int jv = value_index(j0);
+    const bool tail = j0 + 32 > kv_len;  // some of the 32 keys are not written yet
+    const bf16_t* vp = v_pages + ((size_t)vpage * K + g) * D * page_size + (jv % page_size);
+    bf16x8 vf[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) vf[dt] = ld16(vp + (size_t)(dt * 16 + col) * page_size);
+    if (j0 + 32 < kv_end) {
+      load_keys(j0 + 32, kpage, knext);
+      vpage = bt[value_index(j0 + 32) / page_size];
+      kpage[0] = bt[key_index(j0 + 64, 0) / page_size];
+      kpage[1] = bt[key_index(j0 + 64, 1) / page_size];
+    }
+
     // ---- S^T = K Q^T for 32 keys (two tiles of 16) ------------------------------
     f32x4 s[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      // row `col` of tile t is key j0 + (col/4)*8 + t*4 + col%4
-      int j = j0 + (col / 4) * 8 + t * 4 + (col % 4);
-      j = j < kv_begin ? kv_begin : (j > last_key ? last_key : j);  // address only
-      const long long page = bt[j / page_size];
-      const bf16_t* kp = k_pages + (((size_t)page * K + g) * page_size + (j % page_size)) * D;
       s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < KT; ++ks) {
-        const int d0 = ks * 32 + quad * 8;
-        const bf16x8 ka = d0 < D ? ld16(kp + d0) : zero8();
-        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, bq[ks], s[t], 0, 0, 0);
-      }
+      for (int ks = 0; ks < KT; ++ks)
+        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][ks], bq[ks], s[t], 0, 0, 0);
     }
     // ---- mask and online softmax: this lane has keys j0 + quad*8 + e, e = 0..7 ----
     float sv[8];
@@ -149,33 +197,30 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                   pack2(pv[6], pv[7])};
     const bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
 
-    // ---- O^T += V^T P^T: lane loads V^T[dim dt*16 + col][keys j0 + quad*8 .. +8] ------
-    int jv = j0 + quad * 8;
-    const bool tail = j0 + 32 > kv_len;  // some of the 32 keys are not written yet
-    if (jv < (kv_begin & ~7)) jv = kv_begin & ~7;
-    if (jv > (last_key & ~7)) jv = last_key & ~7;
-    const long long vpage = bt[jv / page_size];
-    const bf16_t* vp = v_pages + ((size_t)vpage * K + g) * D * page_size + (jv % page_size);
+    // ---- O^T += V^T P^T ------------------------------------------------------------
+    // unwritten slots may hold anything, NaN included, and 0 * NaN must not get in:
+    // in the last block of the request the values of keys past the end are cleared
+    uint32_t keep[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int ja = jv + 2 * w;
+      keep[w] = tail ? ((ja <= last_key ? 0x0000ffffu : 0u) | (ja + 1 <= last_key ? 0xffff0000u : 0u))
+                     : 0xffffffffu;
+    }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      bf16x8 va = ld16(vp + (size_t)(dt * 16 + col) * page_size);
-      if (tail) {
-        // unwritten slots may hold anything, NaN included: 0 * NaN must not get in
-        u32x4 raw = __builtin_bit_cast(u32x4, va);
+      u32x4 raw = __builtin_bit_cast(u32x4, vf[dt]);
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const int ja = jv + 2 * w;
-          uint32_t keep = 0u;
-          if (ja <= last_key) keep |= 0x0000ffffu;
-          if (ja + 1 <= last_key) keep |= 0xffff0000u;
-          raw[w] &= keep;
-        }
-        va = __builtin_bit_cast(bf16x8, raw);
-      }
+      for (int w = 0; w < 4; ++w) raw[w] &= keep[w];
+      const bf16x8 va = __builtin_bit_cast(bf16x8, raw);
 #pragma unroll
       for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
       o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, o[dt], 0, 0, 0);
     }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int ks = 0; ks < KT; ++ks) kcur[t][ks] = knext[t][ks];
   }
 
   // the denominator is spread over the four lanes that share a row
@@ -207,6 +252,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 }
 
 // merge item: {segment, first row, first partial, number of partials}
+// One block per (merge item, kv head); a thread owns four dimensions of one row.
 __global__ void attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
                                        const int* __restrict__ merges,
                                        const int* __restrict__ n_merges_ptr,
@@ -221,25 +267,29 @@ __global__ void attention_merge_kernel(bf16_t* __restrict__ out, int out_row_str
   const int* mg = merges + (size_t)mi * 4;
   const int seg = mg[0], rho0 = mg[1], first = mg[2], n = mg[3];
   const int q_start = seg_q_start[seg], q_len = seg_q_len[seg];
-  // one thread per (row, dim)
-  for (int idx = threadIdx.x; idx < 16 * D; idx += blockDim.x) {
-    const int row = idx / D, d = idx % D;
+  for (int idx = threadIdx.x; idx < 16 * (D / 4); idx += blockDim.x) {
+    const int row = idx / (D / 4), d = (idx % (D / 4)) * 4;
     const int rho = rho0 + row;
     if (rho >= q_len * G) continue;
     float m_all = -INFINITY;
     for (int i = 0; i < n; ++i)
       m_all = fmaxf(m_all, part_ml[(((size_t)(first + i) * K + g) * 16 + row) * 2]);
-    float acc = 0.f, l_all = 0.f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f}, l_all = 0.f;
     for (int i = 0; i < n; ++i) {
       const size_t base = ((size_t)(first + i) * K + g) * 16 + row;
       const float mi_ = part_ml[base * 2], li = part_ml[base * 2 + 1];
       const float w = (mi_ == -INFINITY) ? 0.f : exp2f(mi_ - m_all);
-      acc += w * part_o[base * D + d];
+      float v[4];
+      load4(part_o + base * D + d, v);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] += w * v[e];
       l_all += w * li;
     }
+    const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] *= inv;
     const int qi = rho / G, head = g * G + rho % G;
-    out[(size_t)(q_start + qi) * out_row_stride + (size_t)head * D + d] =
-        f32_to_bf16(l_all > 0.f ? acc / l_all : 0.f);
+    store4(out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D + d, acc);
   }
 }
 

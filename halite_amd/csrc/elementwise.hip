@@ -24,20 +24,49 @@ __global__ void embedding_kernel(const int* __restrict__ ids, const TT* __restri
   for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = to_f32(row[i]);
 }
 
+// four elements per access; d is a multiple of 4
+template <typename TT>
+__global__ void embedding_vec_kernel(const int* __restrict__ ids, const TT* __restrict__ table,
+                                     float* __restrict__ out, int d, int vocab) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  float* o = out + (size_t)t * d;
+  const bool ok = id >= 0 && id < vocab;
+  const TT* row = table + (size_t)(ok ? id : 0) * d;
+  for (int i = threadIdx.x * 4; i < d; i += blockDim.x * 4) {
+    float v[4];
+    load4(row + i, v);
+    if (!ok) v[0] = v[1] = v[2] = v[3] = __uint_as_float(0x7fc00000u);
+    store4(o + i, v);
+  }
+}
+
 extern "C" int hal_embedding(const int* ids, const void* table, int table_dtype, float* out,
                              int n_tokens, int d, int vocab, hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && d > 0 && vocab > 0, "hal_embedding: bad sizes T=%d d=%d V=%d",
               n_tokens, d, vocab);
   if (n_tokens == 0) return 0;
+  HAL_REQUIRE(table_dtype == HAL_F32 || table_dtype == HAL_BF16,
+              "hal_embedding: unknown table dtype %d", table_dtype);
+  if (d % 4 == 0) {
+    int threads = ((d / 4 + 63) / 64) * 64;
+    if (threads > 1024) threads = 1024;
+    if (table_dtype == HAL_F32)
+      hipLaunchKernelGGL(embedding_vec_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream,
+                         ids, (const float*)table, out, d, vocab);
+    else
+      hipLaunchKernelGGL(embedding_vec_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream,
+                         ids, (const bf16_t*)table, out, d, vocab);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   const int threads = d >= 1024 ? 256 : 64;
   if (table_dtype == HAL_F32)
     hipLaunchKernelGGL(embedding_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream, ids,
                        (const float*)table, out, d, vocab);
-  else if (table_dtype == HAL_BF16)
+  else
     hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream, ids,
                        (const bf16_t*)table, out, d, vocab);
-  else
-    return hal_fail("hal_embedding: unknown table dtype %d", table_dtype);
   HAL_LAUNCH_CHECK();
   return 0;
 }
@@ -80,6 +109,82 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delt
   }
 }
 
+// The same with the row held in registers: one pass over memory, four elements per
+// access, all loads issued before the first use.  d is a multiple of 4 and at most
+// 4 * RMS_MAXV * blockDim.x.
+#define RMS_MAXV 8
+template <typename T>
+__global__ void rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                                   const int* __restrict__ rows, const void* __restrict__ w,
+                                   int w_dtype, float eps, T* __restrict__ out, int d,
+                                   int update_h) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float* hr = h + (size_t)src * d;
+  const T* dr = delta ? delta + (size_t)src * d : nullptr;
+  T* o = out + (size_t)r * d;
+  const int nv = d / 4;
+
+  float x[RMS_MAXV][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < RMS_MAXV; ++u) {
+    const int v = threadIdx.x + u * blockDim.x;
+    if (v < nv) load4(hr + v * 4, x[u]);
+  }
+  if (dr) {
+#pragma unroll
+    for (int u = 0; u < RMS_MAXV; ++u) {
+      const int v = threadIdx.x + u * blockDim.x;
+      if (v < nv) {
+        float dv[4];
+        load4(dr + v * 4, dv);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[u][i] += dv[i];
+        if (update_h) store4(hr + v * 4, x[u]);
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < RMS_MAXV; ++u) {
+    const int v = threadIdx.x + u * blockDim.x;
+    if (v < nv) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ss += x[u][i] * x[u][i];
+    }
+  }
+  const float total = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(total / (float)d + eps);
+#pragma unroll
+  for (int u = 0; u < RMS_MAXV; ++u) {
+    const int v = threadIdx.x + u * blockDim.x;
+    if (v < nv) {
+      float wv[4], y[4];
+      load4_any(w, w_dtype, (size_t)v * 4, wv);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y[i] = wv[i] * to_f32(from_f32<T>(x[u][i] * rstd));
+      store4(o + v * 4, y);
+    }
+  }
+}
+
+template <typename T>
+static void launch_rmsnorm(float* h, const void* delta, const int* rows, const void* w,
+                           int w_dtype, float eps, void* out, int n_rows, int d, int update_h,
+                           hipStream_t stream) {
+  if (d % 4 == 0 && d / 4 <= RMS_MAXV * 1024) {
+    int threads = ((d / 4 + 63) / 64) * 64;
+    if (threads > 1024) threads = 1024;
+    hipLaunchKernelGGL(rmsnorm_vec_kernel<T>, dim3(n_rows), dim3(threads), 0, stream, h,
+                       (const T*)delta, rows, w, w_dtype, eps, (T*)out, d, update_h);
+  } else {
+    const int threads = d >= 2048 ? 512 : (d >= 512 ? 256 : 64);
+    hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(n_rows), dim3(threads), 0, stream, h,
+                       (const T*)delta, rows, w, w_dtype, eps, (T*)out, d, update_h);
+  }
+}
+
 extern "C" int hal_rmsnorm(float* h, const void* delta, const int* rows, const void* w,
                            int w_dtype, float eps, void* out, int dtype, int n_rows, int d,
                            int update_h, hipStream_t stream) {
@@ -88,13 +193,10 @@ extern "C" int hal_rmsnorm(float* h, const void* delta, const int* rows, const v
   HAL_REQUIRE(!(rows && update_h && delta),
               "hal_rmsnorm: a gathered call must not update the residual stream");
   if (n_rows == 0) return 0;
-  const int threads = d >= 2048 ? 512 : (d >= 512 ? 256 : 64);
   if (dtype == HAL_F32)
-    hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(n_rows), dim3(threads), 0, stream, h,
-                       (const float*)delta, rows, w, w_dtype, eps, (float*)out, d, update_h);
+    launch_rmsnorm<float>(h, delta, rows, w, w_dtype, eps, out, n_rows, d, update_h, stream);
   else if (dtype == HAL_BF16)
-    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(n_rows), dim3(threads), 0, stream, h,
-                       (const bf16_t*)delta, rows, w, w_dtype, eps, (bf16_t*)out, d, update_h);
+    launch_rmsnorm<bf16_t>(h, delta, rows, w, w_dtype, eps, out, n_rows, d, update_h, stream);
   else
     return hal_fail("hal_rmsnorm: unknown dtype %d", dtype);
   HAL_LAUNCH_CHECK();
@@ -237,6 +339,115 @@ __global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
   }
 }
 
+// Eight elements per work item (rot a multiple of 16, or of 8 for adjacent pairs; D a
+// multiple of 8): all loads of an item are issued before its arithmetic.
+template <typename T>
+__global__ void rope_append_vec_kernel(T* __restrict__ qkv, int row_stride,
+                                       const int* __restrict__ positions,
+                                       const int* __restrict__ token_seg,
+                                       const int* __restrict__ block_table, int bt_stride,
+                                       const float* __restrict__ cos_t,
+                                       const float* __restrict__ sin_t, int table_len,
+                                       T* __restrict__ k_pages, T* __restrict__ v_pages, int H,
+                                       int K, int D, int rot, int interleaved, int page_size,
+                                       int n_pages) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  T* row = qkv + (size_t)t * row_stride;
+  const int half = rot / 2;
+  if (rot > 0 && (pos < 0 || pos >= table_len)) return;
+  long long page = -1;
+  int off = 0;
+  if (K > 0) {
+    page = block_table[(size_t)token_seg[t] * bt_stride + pos / page_size];
+    off = pos % page_size;
+    if (page < 0 || page >= n_pages) page = -1;
+  }
+  const float* cp = cos_t + (size_t)pos * half;
+  const float* sp = sin_t + (size_t)pos * half;
+
+  if (!interleaved) {
+    const int cph = half / 8;
+    for (int idx = threadIdx.x; idx < (H + K) * cph; idx += blockDim.x) {
+      const int head = idx / cph, j = (idx % cph) * 8;
+      T* hp = row + (size_t)head * D;
+      float a[2][4], b[2][4], c[2][4], sn[2][4], y0[2][4], y1[2][4];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        load4(hp + j + 4 * u, a[u]);
+        load4(hp + j + half + 4 * u, b[u]);
+        load4(cp + j + 4 * u, c[u]);
+        load4(sp + j + 4 * u, sn[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          y0[u][i] = a[u][i] * c[u][i] - b[u][i] * sn[u][i];
+          y1[u][i] = a[u][i] * sn[u][i] + b[u][i] * c[u][i];
+        }
+      T* kp = (head >= H && page >= 0)
+                  ? k_pages + (((size_t)page * K + (head - H)) * page_size + off) * D
+                  : nullptr;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        store4(hp + j + 4 * u, y0[u]);
+        store4(hp + j + half + 4 * u, y1[u]);
+        if (kp) {
+          store4(kp + j + 4 * u, y0[u]);
+          store4(kp + j + half + 4 * u, y1[u]);
+        }
+      }
+    }
+  } else {
+    const int cph = rot / 8;
+    for (int idx = threadIdx.x; idx < (H + K) * cph; idx += blockDim.x) {
+      const int head = idx / cph, e0 = (idx % cph) * 8, j = e0 / 2;
+      T* hp = row + (size_t)head * D;
+      float a[2][4], c[4], sn[4], y[2][4];
+      load4(hp + e0, a[0]);
+      load4(hp + e0 + 4, a[1]);
+      load4(cp + j, c);
+      load4(sp + j, sn);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float x0 = a[i / 2][(2 * i) % 4], x1 = a[i / 2][(2 * i) % 4 + 1];
+        y[i / 2][(2 * i) % 4] = x0 * c[i] - x1 * sn[i];
+        y[i / 2][(2 * i) % 4 + 1] = x0 * sn[i] + x1 * c[i];
+      }
+      store4(hp + e0, y[0]);
+      store4(hp + e0 + 4, y[1]);
+      if (head >= H && page >= 0) {
+        T* kp = k_pages + (((size_t)page * K + (head - H)) * page_size + off) * D;
+        store4(kp + e0, y[0]);
+        store4(kp + e0 + 4, y[1]);
+      }
+    }
+  }
+  if (page < 0) return;
+  const int rest8 = (D - rot) / 8;
+  for (int idx = threadIdx.x; idx < K * rest8; idx += blockDim.x) {
+    const int g = idx / rest8, i = rot + (idx % rest8) * 8;
+    float a[2][4];
+    load4(row + (size_t)(H + g) * D + i, a[0]);
+    load4(row + (size_t)(H + g) * D + i + 4, a[1]);
+    T* kp = k_pages + (((size_t)page * K + g) * page_size + off) * D + i;
+    store4(kp, a[0]);
+    store4(kp + 4, a[1]);
+  }
+  const int d8 = D / 8;
+  for (int idx = threadIdx.x; idx < K * d8; idx += blockDim.x) {
+    const int g = idx / d8, i = (idx % d8) * 8;
+    const T* vr = row + (size_t)(H + K + g) * D + i;
+    T vals[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) vals[e] = vr[e];
+    T* vp = v_pages + (((size_t)page * K + g) * D + i) * page_size + off;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) vp[(size_t)e * page_size] = vals[e];
+  }
+}
+
 extern "C" int hal_rope_append(void* qkv, int dtype, int row_stride, const int* positions,
                                const int* token_seg, const int* block_table, int bt_stride,
                                const float* cos_t, const float* sin_t, int table_len,
@@ -250,6 +461,26 @@ extern "C" int hal_rope_append(void* qkv, int dtype, int row_stride, const int* 
   HAL_REQUIRE(K == 0 || (k_pages && v_pages && block_table && token_seg && page_size > 0),
               "hal_rope_append: cache arguments missing");
   if (n_tokens == 0) return 0;
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_rope_append: unknown dtype %d", dtype);
+  const bool vec = D % 8 == 0 && row_stride % 8 == 0 && (interleaved ? rot % 8 == 0 : rot % 16 == 0);
+  if (vec) {
+    int items = (H + K) * (rot / 8) / (interleaved ? 1 : 2);
+    if (K * (D / 8) > items) items = K * (D / 8);
+    int threads = ((items + 63) / 64) * 64;
+    threads = threads < 64 ? 64 : (threads > 512 ? 512 : threads);
+    if (dtype == HAL_F32)
+      hipLaunchKernelGGL(rope_append_vec_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream,
+                         (float*)qkv, row_stride, positions, token_seg, block_table, bt_stride,
+                         cos_t, sin_t, table_len, (float*)k_pages, (float*)v_pages, H, K, D, rot,
+                         interleaved, page_size, n_pages);
+    else
+      hipLaunchKernelGGL(rope_append_vec_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream,
+                         (bf16_t*)qkv, row_stride, positions, token_seg, block_table, bt_stride,
+                         cos_t, sin_t, table_len, (bf16_t*)k_pages, (bf16_t*)v_pages, H, K, D,
+                         rot, interleaved, page_size, n_pages);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   const int work = (H + K) * (rot / 2) > K * D ? (H + K) * (rot / 2) : K * D;
   const int threads = work >= 1024 ? 256 : (work >= 256 ? 128 : 64);
   if (dtype == HAL_F32)

@@ -12,6 +12,7 @@
 // (src/halite/transformers/feedforward.py:204-212).
 #include "hal_common.h"
 #include "hal_api.h"
+#include <stdlib.h>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -25,12 +26,12 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* p, bool valid) {
 
 enum { SK_OUT_BF16 = 0, SK_OUT_F32 = 1, SK_OUT_F32_ADD = 2 };
 
-template <int NT, int MT, bool GATED>
+template <int NT, int MT, bool GATED, int U>
 __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
                                    const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
                                    int ldw, void* __restrict__ C, int ldc, int out_mode, int M,
                                    int N, int K) {
-  extern __shared__ float red[];  // [sets][NT*MT][64][4]
+  extern __shared__ float red[];  // [waves][sets][NT*MT][64][4]
   const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
   const int n_waves = blockDim.x / HAL_WAVE;
   const int r = lane % 16, q = lane / 16;
@@ -56,8 +57,8 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   for (int f = 0; f < NT; ++f) {
     int n = n_base + f * 16 + r;
     if (n >= N) n = N - 1;  // rows past the end are computed and dropped
-    wrow[f] = W + (size_t)n * ldw;
-    w2row[f] = GATED ? W2 + (size_t)n * ldw : nullptr;
+    wrow[f] = W + (size_t)n * ldw + q * 8;
+    w2row[f] = GATED ? W2 + (size_t)n * ldw + q * 8 : nullptr;
   }
   const bf16_t* xrow[MT];
   bool xvalid[MT];
@@ -65,51 +66,51 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + r;
     xvalid[t] = m < M;
-    xrow[t] = X + (size_t)(xvalid[t] ? m : 0) * ldx;
+    xrow[t] = X + (size_t)(xvalid[t] ? m : 0) * ldx + q * 8;
   }
 
-#pragma unroll 2
-  for (int step = s_begin; step < s_end; ++step) {
-    const int k = step * 32 + q * 8;
-    const bool kv = k < K;  // K is a multiple of 8
-    bf16x8 a[NT], a2[NT], b[MT];
+  // U steps of 32 columns at a time: every load of the group is issued before the
+  // first multiply, so a wave keeps U * (NT + MT) 16-byte loads in flight
+  for (int step = s_begin; step < s_end; step += U) {
+    bf16x8 a[U][NT], a2[U][NT], b[U][MT];
 #pragma unroll
-    for (int f = 0; f < NT; ++f) {
-      a[f] = load_frag(wrow[f] + k, kv);
-      if (GATED) a2[f] = load_frag(w2row[f] + k, kv);
+    for (int u = 0; u < U; ++u) {
+      const int k = (step + u) * 32;
+      const bool kv = (step + u) < s_end && k + q * 8 < K;  // K is a multiple of 8
+#pragma unroll
+      for (int f = 0; f < NT; ++f) {
+        a[u][f] = load_frag(wrow[f] + k, kv);
+        if (GATED) a2[u][f] = load_frag(w2row[f] + k, kv);
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) b[u][t] = load_frag(xrow[t] + k, kv && xvalid[t]);
     }
 #pragma unroll
-    for (int t = 0; t < MT; ++t) b[t] = load_frag(xrow[t] + k, kv && xvalid[t]);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int f = 0; f < NT; ++f)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          acc[0][f][t] =
+              __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][f], b[u][t], acc[0][f][t], 0, 0, 0);
+          if (GATED)
+            acc[1][f][t] =
+                __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[u][f], b[u][t], acc[1][f][t], 0, 0, 0);
+        }
+  }
+
+  // every wave's partial sums -> LDS; then each output element is the sum over the
+  // waves in wave order (deterministic)
+  constexpr int TILE = SETS * NT * MT * 256;
+  float* mine = red + (size_t)wave * TILE;
+#pragma unroll
+  for (int s = 0; s < SETS; ++s)
 #pragma unroll
     for (int f = 0; f < NT; ++f)
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        acc[0][f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[f], b[t], acc[0][f][t], 0, 0, 0);
-        if (GATED)
-          acc[1][f][t] =
-              __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[f], b[t], acc[1][f][t], 0, 0, 0);
-      }
-  }
-
-  // partial sums -> LDS, one wave after the other in wave order (deterministic)
-  for (int w = 0; w < n_waves; ++w) {
-    if (wave == w) {
-#pragma unroll
-      for (int s = 0; s < SETS; ++s)
-#pragma unroll
-        for (int f = 0; f < NT; ++f)
-#pragma unroll
-          for (int t = 0; t < MT; ++t) {
-            float* dst = red + ((s * NT + f) * MT + t) * 256 + lane * 4;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              if (w == 0) dst[i] = acc[s][f][t][i];
-              else dst[i] += acc[s][f][t][i];
-            }
-          }
-    }
-    __syncthreads();
-  }
+      for (int t = 0; t < MT; ++t)
+        *(f32x4*)(mine + ((s * NT + f) * MT + t) * 256 + lane * 4) = acc[s][f][t];
+  __syncthreads();
 
   // element (f, t, lane, i) of the accumulator tile is row n_base + f*16 + (lane/16)*4 + i
   // of W (column of C) and row t*16 + lane%16 of X (row of C)
@@ -119,8 +120,11 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
     const int n = n_base + f * 16 + (ln / 16) * 4 + i;
     const int m = t * 16 + ln % 16;
     if (n >= N || m >= M) continue;
-    float v = red[idx];
-    const float v2 = GATED ? red[NT * MT * 256 + idx] : 0.f;
+    float v = 0.f, v2 = 0.f;
+    for (int w = 0; w < n_waves; ++w) {
+      v += red[(size_t)w * TILE + idx];
+      if (GATED) v2 += red[(size_t)w * TILE + NT * MT * 256 + idx];
+    }
     if (GATED) v = v2 * (v / (1.0f + expf(-v)));  // set 0 is the gate, set 1 is up
     const size_t o = (size_t)m * ldc + n;
     if (out_mode == SK_OUT_BF16)
@@ -132,15 +136,16 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   }
 }
 
-template <int NT, int MT, bool GATED>
+template <int NT, int MT, bool GATED, int U>
 static int launch_skinny(const bf16_t* X, int ldx, const bf16_t* W, const bf16_t* W2, int ldw,
                          void* C, int ldc, int out_mode, int M, int N, int K, int waves,
                          hipStream_t stream) {
   constexpr int SETS = GATED ? 2 : 1;
-  const size_t smem = (size_t)SETS * NT * MT * 256 * sizeof(float);
+  const size_t smem = (size_t)waves * SETS * NT * MT * 256 * sizeof(float);
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
-  hipLaunchKernelGGL((skinny_gemm_kernel<NT, MT, GATED>), dim3(blocks), dim3(waves * HAL_WAVE),
-                     smem, stream, X, ldx, W, W2, ldw, C, ldc, out_mode, M, N, K);
+  hipLaunchKernelGGL((skinny_gemm_kernel<NT, MT, GATED, U>), dim3(blocks),
+                     dim3(waves * HAL_WAVE), smem, stream, X, ldx, W, W2, ldw, C, ldc, out_mode,
+                     M, N, K);
   HAL_LAUNCH_CHECK();
   return 0;
 }
@@ -163,26 +168,52 @@ extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const
   const bf16_t* w = (const bf16_t*)W;
   const bf16_t* w2 = (const bf16_t*)W2;
   const int mt = (M + 15) / 16;
-  // rows of W per wave grow with the rows of X, so that X is not read more often
-  // than W; the waves of a block split K, more of them when there are few blocks
-  const int nt = mt >= 3 ? 4 : mt;
+  const int sets = w2 ? 2 : 1;
+  // Rows of W per wave (16 * nt): more of them mean that a fragment of X, which every
+  // block reads again, serves more of W.  The waves of a block split K, more of them
+  // when there are few blocks.  Tunable through the environment for measurements.
+  int nt = mt >= 3 ? 4 : mt;
+  int u = 0, waves = 0;
+  if (const char* e = getenv("HAL_SKINNY_NT")) nt = atoi(e);
+  if (const char* e = getenv("HAL_SKINNY_U")) u = atoi(e);
+  if (const char* e = getenv("HAL_SKINNY_WAVES")) waves = atoi(e);
+  if (nt != 1 && nt != 2 && nt != 4) nt = 4;
+  if (mt >= 3 && nt < 4) nt = 4;
+  if (mt == 2 && nt < 2) nt = 2;
   const int blocks = (N + 16 * nt - 1) / (16 * nt);
   const int steps = (K + 31) / 32;
-  int waves = 4;
-  while (waves < 16 && blocks * waves < 4096 && steps / (waves * 2) >= 8) waves *= 2;
+  if (waves <= 0) {
+    waves = 4;
+    while (waves < 16 && blocks * waves < 4096 && steps / (waves * 2) >= 4) waves *= 2;
+  }
+  while (waves > 1 && (size_t)waves * sets * nt * mt * 1024 > 64 * 1024) waves /= 2;
+  // loads in flight per wave: about 16 fragments of 16 bytes
+  if (u <= 0) u = 8 / (sets * nt);
+  u = u >= 8 ? 8 : (u >= 4 ? 4 : (u >= 2 ? 2 : 1));
 
-#define SK_CASE(NT_, MT_)                                                                     \
-  if (nt == NT_ && mt == MT_) {                                                               \
+#define SK_LAUNCH(NT_, MT_, U_)                                                               \
+  do {                                                                                        \
     if (w2)                                                                                   \
-      return launch_skinny<NT_, MT_, true>(x, ldx, w, w2, ldw, C, ldc, out_mode, M, N, K,     \
-                                           waves, stream);                                    \
-    return launch_skinny<NT_, MT_, false>(x, ldx, w, nullptr, ldw, C, ldc, out_mode, M, N, K, \
-                                          waves, stream);                                     \
+      return launch_skinny<NT_, MT_, true, U_>(x, ldx, w, w2, ldw, C, ldc, out_mode, M, N, K, \
+                                               waves, stream);                                \
+    return launch_skinny<NT_, MT_, false, U_>(x, ldx, w, nullptr, ldw, C, ldc, out_mode, M,   \
+                                              N, K, waves, stream);                           \
+  } while (0)
+#define SK_CASE(NT_, MT_)                                      \
+  if (nt == NT_ && mt == MT_) {                                \
+    if (u == 8) SK_LAUNCH(NT_, MT_, ((NT_ + MT_) <= 2 ? 8 : 4)); \
+    if (u == 4) SK_LAUNCH(NT_, MT_, ((NT_ + MT_) <= 5 ? 4 : 2)); \
+    if (u == 2) SK_LAUNCH(NT_, MT_, 2);                        \
+    SK_LAUNCH(NT_, MT_, 1);                                    \
   }
   SK_CASE(1, 1)
+  SK_CASE(2, 1)
+  SK_CASE(4, 1)
   SK_CASE(2, 2)
+  SK_CASE(4, 2)
   SK_CASE(4, 3)
   SK_CASE(4, 4)
+#undef SK_LAUNCH
 #undef SK_CASE
   return hal_fail("hal_gemm_bf16_skinny: no kernel for nt=%d mt=%d", nt, mt);
 }

@@ -70,6 +70,30 @@ __device__ __forceinline__ float load_as_f32(const void* p, int dtype, size_t i)
   return dtype == HAL_F32 ? ((const float*)p)[i] : bf16_to_f32(((const bf16_t*)p)[i]);
 }
 
+// ---- vectors of four elements as floats (16-byte or 8-byte accesses) ----------------
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+  const float4 t = *(const float4*)p;
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float (&v)[4]) {
+  const uint2 t = *(const uint2*)p;
+  v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+  v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+__device__ __forceinline__ void store4(float* p, const float (&v)[4]) {
+  *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float (&v)[4]) {
+  uint2 t;
+  t.x = (uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16);
+  t.y = (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16);
+  *(uint2*)p = t;
+}
+__device__ __forceinline__ void load4_any(const void* p, int dtype, size_t i, float (&v)[4]) {
+  if (dtype == HAL_F32) load4((const float*)p + i, v);
+  else load4((const bf16_t*)p + i, v);
+}
+
 // ---- reductions -----------------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
