@@ -78,6 +78,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration (named in the record)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -101,7 +102,8 @@ def main() -> int:
     runner = ModelRunner.from_random(
         cfg, seed=0,
         server_config=ServerConfig(kv_cache_num_tokens=pool_tokens, max_seqs_per_forward=max(batches) + 1,
-                                   max_tokens_per_forward=16384),
+                                   max_tokens_per_forward=16384, use_cudagraph=not args.no_graph,
+                                   cudagraph_max_batch_size=max(batches)),
         model_config=ModelConfig(dtype=args.dtype, context_len=context),
     )
     sampler = Sampler(runner.device)
@@ -186,6 +188,7 @@ def main() -> int:
             "context_len": context,
             "prefill_tokens": 2048,
             "page_size": runner.cache.page_size,
+            "hip_graph": not args.no_graph,
             "parallelism": "single GPU",
         },
         "roofline": {

@@ -143,11 +143,12 @@ class CacheManager:
         self.slots.free(slot)
 
     # -- what a step reads ----------------------------------------------------------
-    def block_table(self, group_id: int, slots: list[int]) -> np.ndarray:
+    def block_table(self, group_id: int, slots: list[int], width: int | None = None) -> np.ndarray:
         """``[len(slots), P]`` int32, row i the page list of ``slots[i]``, -1 where
-        the request holds no page."""
+        the request holds no page.  ``P`` is the longest list unless ``width`` fixes it."""
         g = self.groups[group_id]
-        width = max((len(g.tables.get(s, ())) for s in slots), default=0)
+        if width is None:
+            width = max((len(g.tables.get(s, ())) for s in slots), default=0)
         out = np.full((len(slots), max(width, 1)), -1, dtype=np.int32)
         for i, s in enumerate(slots):
             t = g.tables.get(s, ())

@@ -40,6 +40,54 @@ class GroupStep:
     block_table_host: np.ndarray
 
 
+class _Packer:
+    def __init__(self):
+        self.parts = []
+        self.offsets = {}
+        self.n = 0
+
+    def add(self, name, arr, capacity: int | None = None):
+        """Appends ``arr``; with ``capacity`` the piece takes that many ints whatever
+        its length (so that later pieces keep their place from step to step)."""
+        arr = np.ascontiguousarray(arr, dtype=np.int32).reshape(-1)
+        room = arr.size if capacity is None else capacity
+        if arr.size > room:
+            raise ValueError(f"step array {name} has {arr.size} entries, room for {room}")
+        room += (-room) % 4  # keep every piece 16-byte aligned
+        self.offsets[name] = (self.n, arr.size)
+        self.parts.append(arr)
+        if room > arr.size:
+            self.parts.append(np.zeros(room - arr.size, dtype=np.int32))
+        self.n += room
+
+    def flat(self):
+        return np.concatenate(self.parts) if self.parts else np.zeros(0, dtype=np.int32)
+
+
+class StaticLayout:
+    """Fixed capacities and one persistent device buffer, so that every array of a
+    step lies at the same address step after step: what a captured graph needs.
+    Made for decode-only steps of ``n_segs`` requests."""
+
+    def __init__(self, n_segs: int, bt_width: dict[int, int], max_items: int, device):
+        self.n_segs = n_segs
+        self.bt_width = dict(bt_width)
+        self.max_items = max_items
+        self.device = device
+        self.buffer: torch.Tensor | None = None
+        self.size = 0
+
+    def place(self, flat: np.ndarray, staging: "_Staging") -> torch.Tensor:
+        if self.buffer is None:
+            self.size = flat.size
+            self.buffer = torch.zeros(flat.size, dtype=torch.int32, device=self.device)
+        if flat.size != self.size:
+            raise RuntimeError("a static step layout changed its size")
+        self.buffer.copy_(staging.pinned(flat), non_blocking=True)
+        staging.mark()
+        return self.buffer
+
+
 class _Staging:
     """A ring of pinned host buffers for the per-step copy."""
 
@@ -48,8 +96,9 @@ class _Staging:
         self.bufs = [None] * n
         self.events = [None] * n
         self.i = 0
+        self._last = 0
 
-    def upload(self, flat: np.ndarray) -> torch.Tensor:
+    def pinned(self, flat: np.ndarray) -> torch.Tensor:
         i = self.i
         self.i = (self.i + 1) % len(self.bufs)
         if self.events[i] is not None:
@@ -58,39 +107,29 @@ class _Staging:
         if self.bufs[i] is None or self.bufs[i].numel() < n:
             self.bufs[i] = torch.empty(max(n, 4096) * 2, dtype=torch.int32, pin_memory=True)
         self.bufs[i][:n].numpy()[:] = flat
-        dev = self.bufs[i][:n].to(self.device, non_blocking=True)
+        self._last = i
+        return self.bufs[i][:n]
+
+    def mark(self):
         ev = torch.cuda.Event()
         ev.record()
-        self.events[i] = ev
+        self.events[self._last] = ev
+
+    def upload(self, flat: np.ndarray) -> torch.Tensor:
+        dev = self.pinned(flat).to(self.device, non_blocking=True)
+        self.mark()
         return dev
-
-
-class _Packer:
-    def __init__(self):
-        self.parts = []
-        self.offsets = {}
-        self.n = 0
-
-    def add(self, name, arr):
-        arr = np.ascontiguousarray(arr, dtype=np.int32).reshape(-1)
-        pad = (-arr.size) % 4  # keep every piece 16-byte aligned
-        self.offsets[name] = (self.n, arr.size)
-        self.parts.append(arr)
-        if pad:
-            self.parts.append(np.zeros(pad, dtype=np.int32))
-        self.n += arr.size + pad
-
-    def flat(self):
-        return np.concatenate(self.parts) if self.parts else np.zeros(0, dtype=np.int32)
 
 
 class StepContext:
     """The device-side view of a step that the parts compute on."""
 
-    def __init__(self, segments: list[Segment], cache, device, staging: _Staging | None = None):
+    def __init__(self, segments: list[Segment], cache, device, staging: _Staging | None = None,
+                 static: StaticLayout | None = None):
         self.device = torch.device(device)
         self.segments = segments
         self.cache = cache
+        self.static = static
         S = len(segments)
         self.n_segs = S
         lens = np.array([s.tokens.size for s in segments], dtype=np.int32)
@@ -115,6 +154,8 @@ class StepContext:
         self.max_position = int(self.seg_kv_len_host.max()) - 1 if S else 0
         self.positions_host = positions
         self.token_seg_host = seg_of
+        if static is not None and not (S == T == len(rows) == static.n_segs):
+            raise ValueError("a static layout serves decode-only steps of its own batch size")
 
         pk = _Packer()
         pk.add("tokens", tokens)
@@ -128,7 +169,8 @@ class StepContext:
         slots = [s.slot for s in segments]
         tables = {}
         for g in cache.groups:
-            bt = cache.block_table(g.group_id, slots)
+            width = static.bt_width[g.group_id] if static is not None else None
+            bt = cache.block_table(g.group_id, slots, width)
             tables[g.group_id] = bt
             pk.add(f"bt{g.group_id}", bt)
         self._packer = pk
@@ -155,25 +197,32 @@ class StepContext:
         plan.name = f"plan{len(self._plan_host)}"
         counts = np.array([plan.n_items, plan.n_merges], dtype=np.int32)
         if self._dev is None:
-            self._packer.add(plan.name + "_items", plan.items)
-            self._packer.add(plan.name + "_merges", plan.merges)
+            cap = self.static.max_items if self.static is not None else None
+            if cap is not None:
+                plan.cap_items, plan.cap_merges = cap, min(cap, self.n_segs)
+            self._packer.add(plan.name + "_items", plan.items, None if cap is None else cap * 8)
+            self._packer.add(plan.name + "_merges", plan.merges, None if cap is None else plan.cap_merges * 4)
             self._packer.add(plan.name + "_counts", counts)
         else:  # declared after the step's upload: a copy of its own
+            if self.static is not None:
+                raise RuntimeError("a static step needs its attention plans before the upload")
             dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(self.device)
             self._plans[key] = (plan, dev(plan.items), dev(plan.merges), dev(counts))
 
-    def _upload(self):
+    def upload(self):
         if self._dev is not None:
             return
         flat = self._packer.flat()
-        if self._staging is not None and self.device.type == "cuda":
+        if self.static is not None:
+            self._dev = self.static.place(flat, self._staging)
+        elif self._staging is not None and self.device.type == "cuda":
             self._dev = self._staging.upload(flat)
         else:
             self._dev = torch.from_numpy(flat).to(self.device)
         self.empty_f32 = torch.empty((0, 0), dtype=torch.float32, device=self.device)
 
     def _view(self, name) -> torch.Tensor:
-        self._upload()
+        self.upload()
         off, n = self._packer.offsets[name]
         return self._dev[off : off + n]
 
@@ -205,8 +254,15 @@ class StepContext:
         if plan is None:
             return None
         if key not in self._plans:
-            items = self._view(plan.name + "_items").view(-1, 8)
-            merges = self._view(plan.name + "_merges").view(-1, 4)
+            off, _ = self._packer.offsets[plan.name + "_items"]
+            self.upload()
+            items = self._dev[off : off + plan.cap_items * 8].view(-1, 8)
+            off, _ = self._packer.offsets[plan.name + "_merges"]
+            merges = self._dev[off : off + max(plan.cap_merges, 1) * 4].view(-1, 4)
             counts = self._view(plan.name + "_counts")
             self._plans[key] = (plan, items, merges, counts)
         return self._plans[key]
+
+    def fits_static(self) -> bool:
+        """Whether every plan of this step fits the static layout's capacities."""
+        return all(p.n_items <= p.cap_items and p.n_merges <= p.cap_merges for p in self._plan_host.values())

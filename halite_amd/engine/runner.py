@@ -19,7 +19,8 @@ from ..config.engine import ModelConfig, ServerConfig
 from ..config.registry import read_config
 from ..parts.decoder import Decoder
 from ..weights import fill_random, load_weights
-from .batch import Segment, StepContext, _Staging
+from ..kernels import attention as attention_kernels
+from .batch import Segment, StaticLayout, StepContext, _Staging
 
 _TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
@@ -79,6 +80,14 @@ class ModelRunner:
             run.state = self.cache.state_of_run(run.index)
         self._staging = _Staging(self.device) if self.device.type == "cuda" else None
         self.max_total_tokens = self.cache.token_capacity
+        # position tables for the whole context, so that their addresses never change
+        for pos in model.positions.values():
+            if hasattr(pos, "tables"):
+                pos.tables(self.context_len)
+        self._graphs: dict[int, dict] = {}
+        kv_heads = [n.n_kv_heads for n in needs.values()] or [1]
+        self._min_kv_heads = min(kv_heads)
+        self.graph_replays = 0
 
     def _size_pool(self, needs, page_size, dtype) -> int:
         tokens = self.server_config.kv_cache_num_tokens
@@ -159,10 +168,49 @@ class ModelRunner:
         self.check_segments(segments)
         spans = [(s.slot, s.start + s.tokens.size) for s in segments]
         self.cache.reserve(spans)
-        ctx = StepContext(segments, self.cache, self.device, self._staging)
-        for run in self.model.runs:
-            self.model.mixer_of_run(run.index).prepare(ctx, run)
-        logits = self.model.forward(ctx)
+        logits = None
+        if (
+            self.server_config.use_cudagraph
+            and len(segments) <= self.server_config.cudagraph_max_batch_size
+            and all(s.tokens.size == 1 and s.want == [0] for s in segments)
+        ):
+            logits = self._step_graph(segments)
+        if logits is None:
+            ctx = StepContext(segments, self.cache, self.device, self._staging)
+            for run in self.model.runs:
+                self.model.mixer_of_run(run.index).prepare(ctx, run)
+            logits = self.model.forward(ctx)
         for slot, new_len in spans:
             self.cache.advance(slot, new_len)
         return logits
+
+    def _step_graph(self, segments: list[Segment]):
+        """A decode-only step through a captured HIP graph, one graph per batch size
+        (the reference captures its decode pass per padded batch size,
+        src/halite/transformers/infer/engine/model_runner.py:159-239).  The step's
+        arrays live in one persistent buffer that is refilled before every replay;
+        the kernels' grids are sized for the layout's capacities and read the live
+        counts from that buffer.  The first step of a batch size runs eagerly and
+        records the graph; the returned logits are overwritten by the next replay."""
+        B = len(segments)
+        entry = self._graphs.get(B)
+        if entry is None:
+            width = {g.group_id: -(-self.context_len // g.page_size) for g in self.cache.groups}
+            cap = attention_kernels.TARGET_WAVES // self._min_kv_heads + 2 * B + 8
+            entry = self._graphs[B] = {"layout": StaticLayout(B, width, cap, self.device), "graph": None}
+        ctx = StepContext(segments, self.cache, self.device, self._staging, static=entry["layout"])
+        for run in self.model.runs:
+            self.model.mixer_of_run(run.index).prepare(ctx, run)
+        if not ctx.fits_static():
+            return None
+        ctx.upload()
+        if entry["graph"] is None:
+            logits = self.model.forward(ctx)  # this step, for real
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                entry["logits"] = self.model.forward(ctx)  # recorded, not run
+            entry["graph"], entry["ctx"] = graph, ctx
+            return logits
+        entry["graph"].replay()
+        self.graph_replays += 1
+        return entry["logits"]

@@ -32,6 +32,13 @@ class AttentionPlan:
     n_merges: int
     n_partials: int
     name: str = ""
+    # room in the device arrays (larger than the live counts under a static layout)
+    cap_items: int = 0
+    cap_merges: int = 0
+
+    def __post_init__(self):
+        self.cap_items = max(self.cap_items, self.n_items)
+        self.cap_merges = max(self.cap_merges, self.n_merges)
 
 
 def mfma_supported(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
@@ -99,13 +106,14 @@ def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, wi
     n = ctx.n_tokens
     out = torch.empty((n, n_heads * head_dim), dtype=torch.bfloat16, device=q.device)
     part_o = part_ml = None
-    if plan.n_partials:
-        part_o = torch.empty((plan.n_partials, n_kv, 16, head_dim), dtype=torch.float32, device=q.device)
-        part_ml = torch.empty((plan.n_partials, n_kv, 16, 2), dtype=torch.float32, device=q.device)
+    n_part = plan.cap_items if plan.cap_items > plan.n_items else plan.n_partials
+    if n_part and plan.cap_merges:
+        part_o = torch.empty((n_part, n_kv, 16, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n_part, n_kv, 16, 2), dtype=torch.float32, device=q.device)
     P = ops._ptr
     rc = lib.hal_attention_mfma(
         P(q), q_row_stride, P(out), n_heads * head_dim,
-        P(items), P(counts[0:1]), plan.n_items, P(merges), P(counts[1:2]), plan.n_merges,
+        P(items), P(counts[0:1]), plan.cap_items, P(merges), P(counts[1:2]), plan.cap_merges,
         P(ctx.seg_q_start), P(ctx.seg_q_len), P(ctx.seg_kv_len),
         P(group.block_table), group.block_table.shape[1], P(kv.k), P(kv.v), P(part_o), P(part_ml),
         n_heads, n_kv, head_dim, page_size, ctypes.c_float(scale), window, ops._stream(),

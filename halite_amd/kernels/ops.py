@@ -264,7 +264,9 @@ def sample(
     return tokens, logprobs
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 64  # what the kernel takes
+SKINNY_ROWS = 16  # up to here it beats the library product
+_MM_OUT_DTYPE = None  # whether torch.mm takes out_dtype (found at first use)
 
 
 def gemm_bf16_skinny(
@@ -320,14 +322,24 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
         x = x.to(torch.bfloat16)
     m, k = x.shape
     skinny_ok = k % 8 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
-    if skinny_ok and m <= SKINNY_MAX_ROWS:
+    if skinny_ok and m <= SKINNY_ROWS:
         return gemm_bf16_skinny(x, w, out_dtype=out_dtype)
-    if out_dtype == torch.float32 and skinny_ok:
-        out = torch.empty((m, w.shape[0]), dtype=torch.float32, device=x.device)
-        for r0 in range(0, m, SKINNY_MAX_ROWS):
-            out[r0 : r0 + SKINNY_MAX_ROWS] = gemm_bf16_skinny(
-                x[r0 : r0 + SKINNY_MAX_ROWS], w, out_dtype=torch.float32
-            )
-        return out
+    if out_dtype == torch.float32:
+        global _MM_OUT_DTYPE
+        if _MM_OUT_DTYPE is None:
+            try:
+                torch.mm(x[:1], w[:8].t(), out_dtype=torch.float32)
+                _MM_OUT_DTYPE = True
+            except (TypeError, RuntimeError):
+                _MM_OUT_DTYPE = False
+        if _MM_OUT_DTYPE:  # float32 accumulators written out unrounded
+            return torch.mm(x, w.t(), out_dtype=torch.float32)
+        if skinny_ok:
+            out = torch.empty((m, w.shape[0]), dtype=torch.float32, device=x.device)
+            for r0 in range(0, m, SKINNY_MAX_ROWS):
+                out[r0 : r0 + SKINNY_MAX_ROWS] = gemm_bf16_skinny(
+                    x[r0 : r0 + SKINNY_MAX_ROWS], w, out_dtype=torch.float32
+                )
+            return out
     y = torch.matmul(x, w.t())
     return y if out_dtype == torch.bfloat16 else y.to(out_dtype)

@@ -168,3 +168,38 @@ def test_refusals(folders):
         runner.step([Segment(s2, 0, list(range(100)), [])])  # 2 pages of 64 in all
     assert runner.cache.length(s2) == 0
     runner.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_through_a_captured_graph(folders, dtype):
+    """Decode-only steps replayed from a HIP graph: every replay is checked, with
+    eager work (a prompt of another request, a change of the batch size) between
+    replays, against the plain implementation and against the eager engine."""
+    folder, requests, ref = folders[("C", dtype)]
+    server = ServerConfig(kv_cache_num_tokens=1024, page_size=16, max_seqs_per_forward=8, use_cudagraph=True)
+    runner = ModelRunner.from_pretrained(folder, server, ModelConfig(dtype=dtype))
+    a, b, c = requests["r0"], requests["r3"], requests["r1"]  # 130, 200, 64 tokens
+    trace = [{"step": 0, "entries": [{"id": "a", "tokens": a[:60], "want": [59]}, {"id": "b", "tokens": b[:100], "want": []}], "end": []}]
+    pa, pb = 60, 100
+    for i in range(60):
+        entries = [{"id": "a", "tokens": [a[pa]], "want": [0]}, {"id": "b", "tokens": [b[pb]], "want": [0]}]
+        pa, pb = pa + 1, pb + 1
+        trace.append({"step": len(trace), "entries": entries, "end": []})
+        if i == 20:  # an eager prompt between two replays
+            trace.append({"step": len(trace), "entries": [{"id": "c", "tokens": c, "want": [63]}], "end": ["c"]})
+    trace[-1]["end"] = ["a"]
+    for i in range(30):  # the batch shrinks to one request: another graph
+        trace.append({"step": len(trace), "entries": [{"id": "b", "tokens": [b[pb]], "want": [0]}], "end": []})
+        pb += 1
+    trace[-1]["end"] = ["b"]
+    logits = replay.run_trace(runner, trace)
+    assert runner.graph_replays >= 80 and sorted(runner._graphs) == [1, 2]
+    rows = replay.collect(trace, logits, 331)
+    ref2 = {"a": ref["r0"], "b": ref["r3"], "c": ref["r1"]}
+    replay.compare(rows, ref2, TOL[dtype])
+    eager = make_runner(folder, dtype, 1024, 16)
+    rows_eager = replay.collect(trace, replay.run_trace(eager, trace), 331)
+    for rid in rows:
+        for p in rows[rid]:
+            d = float((rows[rid][p] - rows_eager[rid][p]).abs().max())
+            assert d <= (1e-6 if dtype == "float32" else 2e-2), (rid, p, d)
