@@ -252,14 +252,16 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 }
 
 // merge item: {segment, first row, first partial, number of partials}
-// One block per (merge item, kv head); a thread owns four dimensions of one row.
-__global__ void attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
-                                       const int* __restrict__ merges,
-                                       const int* __restrict__ n_merges_ptr,
-                                       const int* __restrict__ seg_q_start,
-                                       const int* __restrict__ seg_q_len,
-                                       const float* __restrict__ part_o,
-                                       const float* __restrict__ part_ml, int H, int K) {
+// One block per (merge item, kv head); a wave owns a row at a time, a lane two
+// dimensions.  The weights exp2(m_i - max) of up to 64 partials are computed one per
+// lane and handed round with shuffles, so that the loads of the partial sums do not
+// wait for one another.
+__global__ void __launch_bounds__(256)
+attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
+                       const int* __restrict__ merges, const int* __restrict__ n_merges_ptr,
+                       const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
+                       const float* __restrict__ part_o, const float* __restrict__ part_ml, int H,
+                       int K) {
   const int mi = blockIdx.x;
   if (mi >= *n_merges_ptr) return;
   const int g = blockIdx.y;
@@ -267,29 +269,53 @@ __global__ void attention_merge_kernel(bf16_t* __restrict__ out, int out_row_str
   const int* mg = merges + (size_t)mi * 4;
   const int seg = mg[0], rho0 = mg[1], first = mg[2], n = mg[3];
   const int q_start = seg_q_start[seg], q_len = seg_q_len[seg];
-  for (int idx = threadIdx.x; idx < 16 * (D / 4); idx += blockDim.x) {
-    const int row = idx / (D / 4), d = (idx % (D / 4)) * 4;
+  const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
+  const int n_waves = blockDim.x / HAL_WAVE;
+  for (int row = wave; row < 16; row += n_waves) {
     const int rho = rho0 + row;
-    if (rho >= q_len * G) continue;
+    if (rho >= q_len * G) break;  // rows are in order: the rest are invalid too
+    // the largest running maximum of the row
     float m_all = -INFINITY;
-    for (int i = 0; i < n; ++i)
+    for (int i = lane; i < n; i += HAL_WAVE)
       m_all = fmaxf(m_all, part_ml[(((size_t)(first + i) * K + g) * 16 + row) * 2]);
-    float acc[4] = {0.f, 0.f, 0.f, 0.f}, l_all = 0.f;
-    for (int i = 0; i < n; ++i) {
-      const size_t base = ((size_t)(first + i) * K + g) * 16 + row;
-      const float mi_ = part_ml[base * 2], li = part_ml[base * 2 + 1];
-      const float w = (mi_ == -INFINITY) ? 0.f : exp2f(mi_ - m_all);
-      float v[4];
-      load4(part_o + base * D + d, v);
+    m_all = wave_max(m_all);
+    float acc[D / 128 + 1][2];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[e] += w * v[e];
-      l_all += w * li;
+    for (int c = 0; c < D / 128 + 1; ++c) acc[c][0] = acc[c][1] = 0.f;
+    float l_all = 0.f;
+    for (int i0 = 0; i0 < n; i0 += HAL_WAVE) {
+      float w = 0.f;
+      if (i0 + lane < n) {
+        const size_t base = ((size_t)(first + i0 + lane) * K + g) * 16 + row;
+        const float mi_ = part_ml[base * 2], li = part_ml[base * 2 + 1];
+        w = (mi_ == -INFINITY) ? 0.f : exp2f(mi_ - m_all);
+        l_all += w * li;
+      }
+      const int cnt = n - i0 < HAL_WAVE ? n - i0 : HAL_WAVE;
+#pragma unroll 8
+      for (int i = 0; i < cnt; ++i) {
+        const float wi = __shfl(w, i, HAL_WAVE);
+        const float* po = part_o + (((size_t)(first + i0 + i) * K + g) * 16 + row) * D;
+#pragma unroll
+        for (int c = 0; c < D / 128 + 1; ++c) {
+          const int d = c * 128 + lane * 2;
+          if (d < D) {
+            const float2 v = *(const float2*)(po + d);
+            acc[c][0] += wi * v.x;
+            acc[c][1] += wi * v.y;
+          }
+        }
+      }
     }
+    l_all = wave_sum(l_all);
     const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) acc[e] *= inv;
     const int qi = rho / G, head = g * G + rho % G;
-    store4(out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D + d, acc);
+    bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
+#pragma unroll
+    for (int c = 0; c < D / 128 + 1; ++c) {
+      const int d = c * 128 + lane * 2;
+      if (d < D) *(uint32_t*)(op + d) = pack2(acc[c][0] * inv, acc[c][1] * inv);
+    }
   }
 }
 

@@ -52,7 +52,7 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
   __shared__ ArgMax amax_s[16];
   __shared__ float chunk_sum[SAMPLE_THREADS];
   __shared__ int chosen_thread;
-  __shared__ float chosen_before;
+  __shared__ int last_thread;
 
   const int row = blockIdx.x, tid = threadIdx.x;
   const int lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
@@ -62,12 +62,34 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
   const bool greedy = (T == 0.f) || (k == 1);
   const float inv_scale = greedy ? 1.f : T;
 
-  // ---- maximum (and its first index) of z = x / T -----------------------------
+  // ---- one pass: maximum (with its first index) and sum of exp(z - max), z = x / T ----
+  // Each thread keeps a running maximum and a sum relative to it (the online form of
+  // softmax's denominator); four logits per load where the row allows it.
   ArgMax am = {-INFINITY, 0x7fffffff};
-  for (int i = tid; i < V; i += SAMPLE_THREADS) {
-    const ArgMax c = {clean_logit(x[i]) / inv_scale, i};
-    am = argmax_merge(am, c);
+  float part = 0.f;
+  auto take = [&](float xv, int i) {
+    const float z = clean_logit(xv) / inv_scale;
+    if (z > am.v) {
+      part = part * expf(am.v - z) + 1.f;  // am.v = -inf gives part * 0
+      am.v = z;
+      am.i = i;
+    } else {
+      part += expf(z - am.v);
+    }
+  };
+  if (ld % 4 == 0 && ((uintptr_t)logits % 16) == 0) {
+    const int n4 = V / 4;
+#pragma unroll 4
+    for (int v = tid; v < n4; v += SAMPLE_THREADS) {
+      const float4 q = *(const float4*)(x + 4 * v);
+      take(q.x, 4 * v), take(q.y, 4 * v + 1), take(q.z, 4 * v + 2), take(q.w, 4 * v + 3);
+    }
+    for (int i = 4 * n4 + tid; i < V; i += SAMPLE_THREADS) take(x[i], i);
+  } else {
+    for (int i = tid; i < V; i += SAMPLE_THREADS) take(x[i], i);
   }
+  // combine the threads: the block's maximum, then the sums rescaled to it
+  ArgMax mine_am = am;
 #pragma unroll
   for (int off = HAL_WAVE / 2; off > 0; off >>= 1) {
     ArgMax o;
@@ -80,10 +102,7 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
   am = amax_s[0];
   for (int w = 1; w < SAMPLE_THREADS / HAL_WAVE; ++w) am = argmax_merge(am, amax_s[w]);
   const float m = am.v;
-
-  // ---- sum of exp(z - m) ---------------------------------------------------------
-  float part = 0.f;
-  for (int i = tid; i < V; i += SAMPLE_THREADS) part += expf(clean_logit(x[i]) / inv_scale - m);
+  part = (mine_am.v == -INFINITY) ? 0.f : part * expf(mine_am.v - m);
   const float total = block_sum(part, red);
 
   if (greedy) {
@@ -104,13 +123,12 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
     uint32_t lo = 0, hi = 0xffffffffu;  // predicate false below the answer, true at hi
     while (lo < hi) {
       const uint32_t mid = lo + (hi - lo) / 2;
-      float cnt = 0.f, mass = 0.f;
+      float cnt = 0.f;
       for (int i = tid; i < V; i += SAMPLE_THREADS) {
         const float z = clean_logit(x[i]) / inv_scale;
         if (sort_key(z) > mid) cnt += 1.f;
       }
       cnt = block_sum(cnt, red);
-      (void)mass;
       if (cnt < (float)k) hi = mid; else lo = mid + 1;
     }
     key_min = lo;
@@ -143,50 +161,45 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
   }
 
   // ---- inverse CDF over the kept tokens in index order -----------------------------
+  // A thread owns a contiguous run of tokens; a block-wide prefix sum of the runs'
+  // kept mass finds the run that holds the target, and its thread walks it.
   const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
   const int begin = tid * chunk;
   const int end = begin + chunk < V ? begin + chunk : V;
   float mine = 0.f;
+#pragma unroll 4
   for (int i = begin; i < end; ++i) {
     const float z = clean_logit(x[i]) / inv_scale;
     const float e = expf(z - m);
     if (sort_key(z) >= key_min && e >= mp) mine += e;
   }
-  chunk_sum[tid] = mine;
-  __syncthreads();
+  float incl = mine;
+#pragma unroll
+  for (int off = 1; off < HAL_WAVE; off <<= 1) {
+    const float up = __shfl_up(incl, off, HAL_WAVE);
+    if (lane >= off) incl += up;
+  }
   if (tid == 0) {
-    float kept_mass = 0.f;
-    for (int i = 0; i < SAMPLE_THREADS; ++i) kept_mass += chunk_sum[i];
-    const float u = uniform_draw(seeds[row], (uint32_t)draw_index[row]);
-    const float target = u * kept_mass;
-    float run = 0.f;
-    int pick = -1;
-    float before = 0.f;
-    int last_nonempty = 0;
-    float last_before = 0.f;
-    for (int i = 0; i < SAMPLE_THREADS; ++i) {
-      const float c = chunk_sum[i];
-      if (c > 0.f) {
-        last_nonempty = i;
-        last_before = run;
-      }
-      if (pick < 0 && run + c > target && c > 0.f) {
-        pick = i;
-        before = run;
-      }
-      run += c;
-    }
-    if (pick < 0) {  // rounding left the target at the very end
-      pick = last_nonempty;
-      before = last_before;
-    }
-    chosen_thread = pick;
-    chosen_before = before;
-    red2[0] = target;
+    chosen_thread = 0x7fffffff;
+    last_thread = -1;
+  }
+  if (lane == HAL_WAVE - 1) red2[wave] = incl;
+  __syncthreads();
+  float before = incl - mine, kept_mass = 0.f;
+  for (int w = 0; w < SAMPLE_THREADS / HAL_WAVE; ++w) {
+    if (w < wave) before += red2[w];
+    kept_mass += red2[w];
+  }
+  const float target = uniform_draw(seeds[row], (uint32_t)draw_index[row]) * kept_mass;
+  if (mine > 0.f) {
+    atomicMax(&last_thread, tid);
+    if (before + mine > target) atomicMin(&chosen_thread, tid);
   }
   __syncthreads();
-  if (tid == chosen_thread) {
-    const float target = red2[0];
+  int pick = chosen_thread;
+  if (pick == 0x7fffffff) pick = last_thread;  // rounding left the target at the very end
+  const float chosen_before = before;
+  if (tid == pick) {
     float run = chosen_before;
     int tok = -1, last_kept = -1;
     float z_tok = 0.f, z_last = 0.f;
