@@ -40,6 +40,12 @@ class ServerConfig(BaseModel):
     max_seqs_per_forward: StrictInt = Field(default=256, gt=0)
     """Most requests that are live (own a slot) at a time."""
 
+    # -- ours -----------------------------------------------------------------
+    decode_weight_copy: Literal["auto", "on", "off"] = "auto"
+    """A second copy of the bf16 matrices in the small-batch kernel's tiled order
+    (steps of up to 16 tokens then read contiguous memory).  ``auto`` keeps it when
+    two copies of the weights take less than a third of the device's memory."""
+
     # -- retraction (infer/engine/batch.py:468-527) ----------------------------
     retract_decode_steps: StrictInt = Field(default=20, gt=0)
 

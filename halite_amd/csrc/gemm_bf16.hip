@@ -55,11 +55,22 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   const bf16_t* w2row[NT];
 #pragma unroll
   for (int f = 0; f < NT; ++f) {
-    int n = n_base + f * 16 + r;
-    if (n >= N) n = N - 1;  // rows past the end are computed and dropped
-    wrow[f] = W + (size_t)n * ldw + q * 8;
-    w2row[f] = GATED ? W2 + (size_t)n * ldw + q * 8 : nullptr;
+    if (ldw == 0) {
+      // tiled weights: [16-row tile][32-column step][lane][8], zero-padded, so that a
+      // wave's load instruction reads one contiguous KiB
+      int tile = blockIdx.x * NT + f;
+      const int n_tiles = (N + 15) / 16;
+      if (tile >= n_tiles) tile = n_tiles - 1;
+      wrow[f] = W + ((size_t)tile * steps * 64 + lane) * 8;
+      w2row[f] = GATED ? W2 + ((size_t)tile * steps * 64 + lane) * 8 : nullptr;
+    } else {
+      int n = n_base + f * 16 + r;
+      if (n >= N) n = N - 1;  // rows past the end are computed and dropped
+      wrow[f] = W + (size_t)n * ldw + q * 8;
+      w2row[f] = GATED ? W2 + (size_t)n * ldw + q * 8 : nullptr;
+    }
   }
+  const int kstride = ldw == 0 ? 512 : 32;  // elements from one step to the next
   const bf16_t* xrow[MT];
   bool xvalid[MT];
 #pragma unroll
@@ -77,10 +88,11 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
     for (int u = 0; u < U; ++u) {
       const int k = (step + u) * 32;
       const bool kv = (step + u) < s_end && k + q * 8 < K;  // K is a multiple of 8
+      const size_t kw = (size_t)(step + u) * kstride;
 #pragma unroll
       for (int f = 0; f < NT; ++f) {
-        a[u][f] = load_frag(wrow[f] + k, kv);
-        if (GATED) a2[u][f] = load_frag(w2row[f] + k, kv);
+        a[u][f] = load_frag(wrow[f] + kw, kv);
+        if (GATED) a2[u][f] = load_frag(w2row[f] + kw, kv);
       }
 #pragma unroll
       for (int t = 0; t < MT; ++t) b[u][t] = load_frag(xrow[t] + k, kv && xvalid[t]);
@@ -158,7 +170,7 @@ extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const
   HAL_REQUIRE(M >= 0 && M <= 64, "hal_gemm_bf16_skinny: M=%d (at most 64 rows)", M);
   HAL_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "hal_gemm_bf16_skinny: N=%d K=%d (K in steps of 8)", N,
               K);
-  HAL_REQUIRE(ldx >= K && ldw >= K && ldc >= N && ldx % 8 == 0 && ldw % 8 == 0,
+  HAL_REQUIRE(ldx >= K && (ldw >= K || ldw == 0) && ldc >= N && ldx % 8 == 0 && ldw % 8 == 0,
               "hal_gemm_bf16_skinny: leading dimensions %d %d %d", ldx, ldw, ldc);
   HAL_REQUIRE(out_mode >= 0 && out_mode <= 2, "hal_gemm_bf16_skinny: out_mode %d", out_mode);
   HAL_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)W2 % 16) == 0,

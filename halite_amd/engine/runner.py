@@ -108,12 +108,24 @@ class ModelRunner:
         return min(pages, cap)
 
     # -- construction -------------------------------------------------------------
+    @staticmethod
+    def _want_tiled(spec, dtype, device, server_config) -> bool:
+        mode = (server_config or ServerConfig()).decode_weight_copy
+        if dtype != torch.bfloat16 or mode == "off":
+            return False
+        if mode == "on":
+            return True
+        probe = Decoder(spec, dtype, "cpu")
+        _, total = torch.cuda.mem_get_info(device)
+        return 2 * probe.param_bytes() < total / 3
+
     @classmethod
     def from_pretrained(cls, folder: str, server_config=None, model_config=None) -> "ModelRunner":
         model_config = model_config or ModelConfig()
         device = require_gpu(f"{model_config.device}:{model_config.gpu_id}" if model_config.device == "cuda" else model_config.device)
         arch, cfg = read_config(folder)
-        model = Decoder(arch.to_spec(cfg), _TORCH_DTYPE[model_config.dtype], device)
+        spec, dtype = arch.to_spec(cfg), _TORCH_DTYPE[model_config.dtype]
+        model = Decoder(spec, dtype, device, cls._want_tiled(spec, dtype, device, server_config))
         load_weights(model, arch.weight_map(cfg), folder)
         runner = cls(model, server_config, model_config)
         runner.arch, runner.config = arch, cfg
@@ -126,7 +138,8 @@ class ModelRunner:
         model_config = model_config or ModelConfig()
         device = require_gpu(f"{model_config.device}:{model_config.gpu_id}" if model_config.device == "cuda" else model_config.device)
         arch = arch or get_architecture(cfg.architectures[0])
-        model = Decoder(arch.to_spec(cfg), _TORCH_DTYPE[model_config.dtype], device)
+        spec, dtype = arch.to_spec(cfg), _TORCH_DTYPE[model_config.dtype]
+        model = Decoder(spec, dtype, device, cls._want_tiled(spec, dtype, device, server_config))
         fill_random(model, seed)
         runner = cls(model, server_config, model_config)
         runner.arch, runner.config = arch, cfg

@@ -269,24 +269,50 @@ SKINNY_ROWS = 16  # up to here it beats the library product
 _MM_OUT_DTYPE = None  # whether torch.mm takes out_dtype (found at first use)
 
 
+def tile_weight(w: torch.Tensor) -> torch.Tensor:
+    """``w`` [N, K] in the small-batch kernel's own order: [16-row tile][32-column
+    step][lane][8 elements], zero-padded, where lane ``l`` of a tile holds row
+    ``l % 16`` and columns ``(l // 16) * 8 ...`` of the step.  A wave's load then reads
+    one contiguous KiB."""
+    n, k = w.shape
+    n_pad, k_pad = -(-n // 16) * 16, -(-k // 32) * 32
+    if (n_pad, k_pad) != (n, k):
+        padded = torch.zeros((n_pad, k_pad), dtype=w.dtype, device=w.device)
+        padded[:n, :k] = w
+        w = padded
+    t = w.view(n_pad // 16, 16, k_pad // 32, 4, 8).permute(0, 2, 3, 1, 4)
+    return t.contiguous().view(-1)
+
+
 def gemm_bf16_skinny(
     x: torch.Tensor,
     w: torch.Tensor,
     w_up: torch.Tensor | None = None,
     out_dtype: torch.dtype = torch.bfloat16,
     add_to: torch.Tensor | None = None,
+    tiled_shape: tuple[int, int] | None = None,
 ):
     """``x @ w.T`` for at most 64 rows of bf16 ``x``; with ``w_up`` the gated form
     ``(x @ w_up.T) * silu(x @ w.T)``; ``add_to`` (float32) receives ``+=``."""
     lib = library.core_library()
     _dev(x, add_to)
-    for t in (w, w_up):
-        if t is not None:
-            _need(t.is_cuda and t.dtype == torch.bfloat16 and t.stride(1) == 1, "skinny gemm: weight layout")
     _need(x.dtype == torch.bfloat16, "skinny gemm takes bf16")
     m, k = x.shape
-    n, k2 = w.shape
-    _need(k == k2 and (w_up is None or (w_up.shape == w.shape and w_up.stride(0) == w.stride(0))), "skinny gemm: shapes")
+    if tiled_shape is not None:  # weights from tile_weight()
+        n, k2 = tiled_shape
+        need = (-(-n // 16) * 16) * (-(-k2 // 32) * 32)
+        for t in (w, w_up):
+            if t is not None:
+                _need(t.is_cuda and t.dtype == torch.bfloat16 and t.numel() == need and t.is_contiguous(), "skinny gemm: tiled weight")
+        ldw = 0
+    else:
+        for t in (w, w_up):
+            if t is not None:
+                _need(t.is_cuda and t.dtype == torch.bfloat16 and t.stride(1) == 1, "skinny gemm: weight layout")
+        n, k2 = w.shape
+        _need(w_up is None or (w_up.shape == w.shape and w_up.stride(0) == w.stride(0)), "skinny gemm: shapes")
+        ldw = w.stride(0)
+    _need(k == k2, "skinny gemm: inner sizes")
     _need(m <= SKINNY_MAX_ROWS, f"skinny gemm: {m} rows")
     if add_to is not None:
         _need(add_to.dtype == torch.float32 and add_to.shape == (m, n), "skinny gemm: add_to")
@@ -298,14 +324,16 @@ def gemm_bf16_skinny(
     _check(
         lib,
         lib.hal_gemm_bf16_skinny(
-            _ptr(x), k, _ptr(w), _ptr(w_up), w.stride(0), _ptr(out), n, mode, m, n, k, _stream()
+            _ptr(x), k, _ptr(w), _ptr(w_up), ldw, _ptr(out), n, mode, m, n, k, _stream()
         ),
     )
     return out
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-    """``x @ w.T`` for a weight ``[out, in]``.
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None,
+           tiled: torch.Tensor | None = None) -> torch.Tensor:
+    """``x @ w.T`` for a weight ``[out, in]``; ``tiled`` is ``tile_weight(w)`` if the
+    model keeps that copy for small batches.
 
     float32 weights: the true 32-bit kernel (activations are widened if needed).
     bf16 weights: the hand-written kernel for up to 64 rows; for more rows the
@@ -322,6 +350,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
         x = x.to(torch.bfloat16)
     m, k = x.shape
     skinny_ok = k % 8 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
+    if m <= SKINNY_ROWS and tiled is not None and k % 8 == 0:
+        return gemm_bf16_skinny(x, tiled, out_dtype=out_dtype, tiled_shape=tuple(w.shape))
     if skinny_ok and m <= SKINNY_ROWS:
         return gemm_bf16_skinny(x, w, out_dtype=out_dtype)
     if out_dtype == torch.float32:

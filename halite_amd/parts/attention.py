@@ -71,6 +71,16 @@ class Attention(Mixer):
             "out.weight": self.w_out,
         }
 
+    def finalize(self):
+        self.t_qkv = self.t_q = self.t_out = None
+        if self.build.tiled_weights and self.w_qkv.dtype == torch.bfloat16 and self.w_qkv.is_cuda:
+            self.t_qkv = ops.tile_weight(self.w_qkv)
+            self.t_out = ops.tile_weight(self.w_out) if self.w_out.dtype == torch.bfloat16 else None
+            n_q = self.p.n_heads * self.p.head_dim
+            if n_q % 16 == 0:  # the q rows are whole tiles at the front
+                steps = -(-self.p.hidden_size // 32)
+                self.t_q = self.t_qkv[: (n_q // 16) * steps * 512]
+
     def cache_need(self):
         return PagedKVNeed(self.p.n_kv_heads, self.p.head_dim, self.p.window)
 
@@ -85,10 +95,10 @@ class Attention(Mixer):
         group = ctx.group(kv.group_id)
         n_q = p.n_heads * p.head_dim
         if run.appends:
-            qkv = ops.linear(x, self.w_qkv)
+            qkv = ops.linear(x, self.w_qkv, tiled=self.t_qkv)
             n_kv_append = p.n_kv_heads
         else:  # the keys and values are an earlier run's
-            qkv = ops.linear(x, self.w_qkv[:n_q])
+            qkv = ops.linear(x, self.w_qkv[:n_q], tiled=self.t_q)
             n_kv_append = 0
         if self.position is not None:
             cos, sin = self.position.tables(ctx.max_position + 1)
@@ -102,4 +112,4 @@ class Attention(Mixer):
             k_pages=kv.k, v_pages=kv.v, page_size=group.page_size,
         )
         out = ctx.attention(qkv, qkv.shape[1], kv, group, p.n_heads, p.scale, p.window or 0)
-        return ops.linear(out, self.w_out)
+        return ops.linear(out, self.w_out, tiled=self.t_out)

@@ -61,6 +61,8 @@ class BuildContext:
     device: torch.device
     hidden_size: int
     positions: dict[str, "Part"] = field(default_factory=dict)
+    # keep a second copy of every bf16 matrix in the small-batch kernel's tiled order
+    tiled_weights: bool = False
 
 
 @dataclass

@@ -39,14 +39,16 @@ class ParamSlot:
 
 
 class Decoder:
-    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device: torch.device | str):
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device: torch.device | str,
+                 tiled_weights: bool = False):
         # the kinds of parts register themselves when their modules are imported
         from . import attention, block, embedding, feedforward, norm, rope  # noqa: F401
 
         self.spec = spec
         self.dtype = dtype
         self.device = torch.device(device)
-        build = BuildContext(dtype=dtype, device=self.device, hidden_size=spec.hidden_size)
+        build = BuildContext(dtype=dtype, device=self.device, hidden_size=spec.hidden_size,
+                             tiled_weights=tiled_weights and dtype == torch.bfloat16)
         for name, pspec in spec.positions.items():
             build.positions[name] = POSITIONS.build(pspec, build)
         self.build = build
@@ -96,6 +98,15 @@ class Decoder:
             self.head.tie(self.embedding)
         for part in self.named_parts().values():
             part.finalize()
+
+    def param_bytes(self) -> int:
+        n = 0
+        for slot in self.param_slots():
+            size = 1
+            for d in slot.decl.shape:
+                size *= d
+            n += size * (4 if slot.decl.integer else self.dtype.itemsize)
+        return n
 
     # -- the forward pass of one step -----------------------------------------------
     def forward(self, ctx) -> torch.Tensor:

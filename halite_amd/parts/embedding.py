@@ -52,5 +52,10 @@ class LinearHead(Head):
     def tie(self, embedding: TokenEmbedding):
         self.weight = embedding.weight
 
+    def finalize(self):
+        self.t_weight = None
+        if self.build.tiled_weights and self.weight.dtype == torch.bfloat16 and self.weight.is_cuda:
+            self.t_weight = ops.tile_weight(self.weight)
+
     def forward(self, x):
-        return ops.linear(x, self.weight, out_dtype=torch.float32)
+        return ops.linear(x, self.weight, out_dtype=torch.float32, tiled=self.t_weight)

@@ -52,9 +52,22 @@ class GatedFeedForward(FeedForward):
             "linear_out.weight": self.w_out,
         }
 
+    def finalize(self):
+        self.t_gate = self.t_up = self.t_out = None
+        f = self.p.intermediate_size
+        if self.build.tiled_weights and self.w_gate_up.is_cuda:
+            if self.w_gate_up.dtype == torch.bfloat16:
+                self.t_gate = ops.tile_weight(self.w_gate_up[:f])
+                self.t_up = ops.tile_weight(self.w_gate_up[f:])
+            if self.w_out.dtype == torch.bfloat16:
+                self.t_out = ops.tile_weight(self.w_out)
+
     def forward(self, x, ctx):
         f = self.p.intermediate_size
         w = self.w_gate_up
+        if self.t_gate is not None and x.dtype == torch.bfloat16 and x.shape[0] <= ops.SKINNY_ROWS and x.shape[1] % 8 == 0:
+            act = ops.gemm_bf16_skinny(x, self.t_gate, w_up=self.t_up, tiled_shape=(f, x.shape[1]))
+            return ops.linear(act, self.w_out, tiled=self.t_out)
         fused = (
             w.dtype == torch.bfloat16
             and x.dtype == torch.bfloat16
@@ -66,4 +79,4 @@ class GatedFeedForward(FeedForward):
             act = ops.gemm_bf16_skinny(x, w[:f], w_up=w[f:])
         else:
             act = ops.silu_mul(ops.linear(x, w))
-        return ops.linear(act, self.w_out)
+        return ops.linear(act, self.w_out, tiled=self.t_out)

@@ -259,6 +259,15 @@ def test_gemm_bf16_skinny(gpu, M, N, K):
     close(ops.gemm_bf16_skinny(xg, wg, w_up=w2g, out_dtype=torch.float32), up * want * torch.sigmoid(want), 3e-5, "skinny gated")
     with pytest.raises(ops.KernelError):
         ops.gemm_bf16_skinny(rnd(65, K).to(torch.bfloat16).to(gpu), wg)
+    # the tiled copy of the weights gives the same sums in the same order
+    tw, tw2 = ops.tile_weight(wg), ops.tile_weight(w2g)
+    assert tw.numel() == (-(-N // 16) * 16) * (-(-K // 32) * 32)
+    a = ops.gemm_bf16_skinny(xg, wg, out_dtype=torch.float32)
+    b = ops.gemm_bf16_skinny(xg, tw, out_dtype=torch.float32, tiled_shape=(N, K))
+    assert torch.equal(a, b)
+    a = ops.gemm_bf16_skinny(xg, wg, w_up=w2g)
+    b = ops.gemm_bf16_skinny(xg, tw, w_up=tw2, tiled_shape=(N, K))
+    assert torch.equal(a, b)
 
 
 def test_linear_dispatch(gpu):

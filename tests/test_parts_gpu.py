@@ -101,7 +101,7 @@ def attention_spec(d=64, heads=4, kv=2, head_dim=16, window=None, position="rope
 
 
 def make_runner(gpu, spec, dtype, tokens=1024, page=16):
-    model = Decoder(spec, DT[dtype], gpu)
+    model = Decoder(spec, DT[dtype], gpu, tiled_weights=True)
     fill_random(model, seed=5, std=0.08)
     return ModelRunner(model, ServerConfig(kv_cache_num_tokens=tokens, page_size=page, max_seqs_per_forward=8),
                        ModelConfig(dtype=dtype))
