@@ -46,11 +46,15 @@ __device__ __forceinline__ bf16x8 zero8() {
   u32x4 z = {0u, 0u, 0u, 0u};
   return __builtin_bit_cast(bf16x8, z);
 }
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-  return (uint32_t)f32_to_bf16(lo).bits | ((uint32_t)f32_to_bf16(hi).bits << 16);
-}
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+// 2^x for x <= 0 (results below the normal range may flush to zero)
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// item: {segment, first row, first key, end key, partial index or -1, 0, 0, 0}
+// item: {segment, first row, first key, end key, first partial slot or -1, 0, 0, 0}
+// A wave works on RT tiles of 16 rows (rows first row .. first row + 16*RT); the keys
+// and values it loads serve all of them.  Row tile rt of an item writes partial slot
+// `first partial slot + rt`.
+template <int RT>
 __global__ void __launch_bounds__(256)
 attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
                       int out_row_stride, const int* __restrict__ items,
@@ -59,7 +63,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                       const int* __restrict__ block_table, int bt_stride,
                       const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                       float* __restrict__ part_o, float* __restrict__ part_ml, int H, int K,
-                      int page_size, float scale_log2e, int window) {
+                      int page_size, int page_shift, float scale_log2e, int window) {
   const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
   const int item = blockIdx.x * (blockDim.x / HAL_WAVE) + wave;
   if (item >= *n_items_ptr) return;
@@ -72,32 +76,48 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   const int* bt = block_table + (size_t)seg * bt_stride;
 
   const int col = lane % 16, quad = lane / 16;
-  // this lane's query row
-  const int rho = rho0 + col;
-  const bool row_ok = rho < q_len * G;
-  const int qi = row_ok ? rho / G : 0;
-  const int hg = row_ok ? rho % G : 0;
-  const int p_row = pos0 + qi;  // the row's position: sees keys <= p_row
-  const int lo_row = (window > 0 && p_row - window + 1 > 0) ? p_row - window + 1 : 0;
-  const int head = g * G + hg;
-
-  // Q^T as the B operand: lane holds Q[row][ks*32 + quad*8 .. +8]
-  bf16x8 bq[KT];
-  {
-    const bf16_t* qp = q + (size_t)(q_start + qi) * q_row_stride + (size_t)head * D;
+  // this lane's query row in every row tile
+  bool row_ok[RT];
+  int qi[RT], head[RT], p_row[RT], lo_row[RT];
+  bf16x8 bq[RT][KT];  // Q^T as the B operand: lane holds Q[row][ks*32 + quad*8 .. +8]
+  f32x4 o[RT][DT];
+  float m[RT], l[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int rho = rho0 + rt * 16 + col;
+    row_ok[rt] = rho < q_len * G;
+    qi[rt] = row_ok[rt] ? rho / G : 0;
+    head[rt] = g * G + (row_ok[rt] ? rho % G : 0);
+    p_row[rt] = pos0 + qi[rt];  // the row's position: it sees keys <= p_row
+    lo_row[rt] = (window > 0 && p_row[rt] - window + 1 > 0) ? p_row[rt] - window + 1 : 0;
+    const bf16_t* qp = q + (size_t)(q_start + qi[rt]) * q_row_stride + (size_t)head[rt] * D;
 #pragma unroll
     for (int ks = 0; ks < KT; ++ks) {
       const int d0 = ks * 32 + quad * 8;
-      bq[ks] = (row_ok && d0 < D) ? ld16(qp + d0) : zero8();
+      bq[rt][ks] = (row_ok[rt] && d0 < D) ? ld16(qp + d0) : zero8();
     }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m[rt] = -INFINITY;
+    l[rt] = 0.f;
   }
 
-  f32x4 o[DT];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
-
   const int last_key = kv_len - 1;  // keys beyond it are not written yet
+  // page and slot of a key; pages of a power of two (page_shift >= 0) need no division
+  auto page_of = [&](int j) { return page_shift >= 0 ? j >> page_shift : j / page_size; };
+  auto slot_of = [&](int j) { return page_shift >= 0 ? j & (page_size - 1) : j % page_size; };
+  // per row tile, the positions of its first and last row (uniform over the wave): a
+  // block of keys wholly below the first row's position needs no mask
+  int p_first[RT], lo_last[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int r_first = rho0 + rt * 16;
+    int r_last = r_first + 15;
+    if (r_last > q_len * G - 1) r_last = q_len * G - 1;
+    p_first[rt] = pos0 + r_first / G;
+    const int p_last = pos0 + (r_last > r_first ? r_last : r_first) / G;
+    lo_last[rt] = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+  }
 
   // This lane's key of tile t in the block of 32 keys at j0: row `col` of tile t is
   // key j0 + (col/4)*8 + t*4 + col%4; its eight keys for the values are j0 + quad*8 .. +8.
@@ -118,7 +138,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int j = key_index(j0, t);
-      const bf16_t* kp = k_pages + (((size_t)pages[t] * K + g) * page_size + (j % page_size)) * D;
+      const bf16_t* kp = k_pages + (((size_t)pages[t] * K + g) * page_size + slot_of(j)) * D;
 #pragma unroll
       for (int ks = 0; ks < KT; ++ks) {
         const int d0 = ks * 32 + quad * 8;
@@ -131,12 +151,12 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   bf16x8 kcur[2][KT], knext[2][KT];
   int kpage[2], vpage;  // pages of the NEXT key block and of THIS value block
   if (j_first < kv_end) {
-    kpage[0] = bt[key_index(j_first, 0) / page_size];
-    kpage[1] = bt[key_index(j_first, 1) / page_size];
-    vpage = bt[value_index(j_first) / page_size];
+    kpage[0] = bt[page_of(key_index(j_first, 0))];
+    kpage[1] = bt[page_of(key_index(j_first, 1))];
+    vpage = bt[page_of(value_index(j_first))];
     load_keys(j_first, kpage, kcur);
-    kpage[0] = bt[key_index(j_first + 32, 0) / page_size];
-    kpage[1] = bt[key_index(j_first + 32, 1) / page_size];
+    kpage[0] = bt[page_of(key_index(j_first + 32, 0))];
+    kpage[1] = bt[page_of(key_index(j_first + 32, 1))];
   }
 
   for (int j0 = j_first; j0 < kv_end; j0 += 32) {
@@ -144,58 +164,74 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     // lane loads V^T[dim dt*16 + col][keys jv .. jv+8]
     const int jv = value_index(j0);
     const bool tail = j0 + 32 > kv_len;  // some of the 32 keys are not written yet
-    const bf16_t* vp = v_pages + ((size_t)vpage * K + g) * D * page_size + (jv % page_size);
+    const bf16_t* vp = v_pages + ((size_t)vpage * K + g) * D * page_size + slot_of(jv);
     bf16x8 vf[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) vf[dt] = ld16(vp + (size_t)(dt * 16 + col) * page_size);
     if (j0 + 32 < kv_end) {
       load_keys(j0 + 32, kpage, knext);
-      vpage = bt[value_index(j0 + 32) / page_size];
-      kpage[0] = bt[key_index(j0 + 64, 0) / page_size];
-      kpage[1] = bt[key_index(j0 + 64, 1) / page_size];
+      vpage = bt[page_of(value_index(j0 + 32))];
+      kpage[0] = bt[page_of(key_index(j0 + 64, 0))];
+      kpage[1] = bt[page_of(key_index(j0 + 64, 1))];
     }
 
-    // ---- S^T = K Q^T for 32 keys (two tiles of 16) ------------------------------
-    f32x4 s[2];
+    bf16x8 pb[RT];
+    float alpha[RT];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int rt = 0; rt < RT; ++rt) {
+      // ---- S^T = K Q^T for 32 keys (two tiles of 16) ----------------------------
+      f32x4 s[2];
 #pragma unroll
-      for (int ks = 0; ks < KT; ++ks)
-        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][ks], bq[ks], s[t], 0, 0, 0);
-    }
-    // ---- mask and online softmax: this lane has keys j0 + quad*8 + e, e = 0..7 ----
-    float sv[8];
-    float m_tile = -INFINITY;
+      for (int t = 0; t < 2; ++t) {
+        s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int j = j0 + quad * 8 + e;
-      const bool ok = row_ok && j >= kv_begin && j < kv_end && j >= lo_row && j <= p_row;
-      sv[e] = ok ? s[e / 4][e % 4] * scale_log2e : -INFINITY;
-      m_tile = fmaxf(m_tile, sv[e]);
-    }
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, HAL_WAVE));
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, HAL_WAVE));
-    const float m_new = fmaxf(m, m_tile);
-    float alpha = 1.f;
-    float pv[8];
-    if (m_new == -INFINITY) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) pv[e] = 0.f;
-    } else {
-      alpha = exp2f(m - m_new);  // m = -inf gives 0
-      float psum = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        pv[e] = exp2f(sv[e] - m_new);
-        psum += pv[e];
+        for (int ks = 0; ks < KT; ++ks)
+          s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][ks], bq[rt][ks], s[t], 0, 0, 0);
       }
-      l = l * alpha + psum;
-      m = m_new;
+      // ---- mask and online softmax: this lane has keys j0 + quad*8 + e, e = 0..7 --
+      float sv[8];
+      float m_tile = -INFINITY;
+      const bool full = j0 >= kv_begin && j0 + 32 <= kv_end && j0 + 31 <= p_first[rt] &&
+                        j0 >= lo_last[rt];
+      if (full) {  // every key of the block is visible to every row of the tile
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          sv[e] = s[e / 4][e % 4] * scale_log2e;
+          m_tile = fmaxf(m_tile, sv[e]);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int j = j0 + quad * 8 + e;
+          const bool ok =
+              row_ok[rt] && j >= kv_begin && j < kv_end && j >= lo_row[rt] && j <= p_row[rt];
+          sv[e] = ok ? s[e / 4][e % 4] * scale_log2e : -INFINITY;
+          m_tile = fmaxf(m_tile, sv[e]);
+        }
+      }
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, HAL_WAVE));
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, HAL_WAVE));
+      const float m_new = fmaxf(m[rt], m_tile);
+      alpha[rt] = 1.f;
+      float pv[8];
+      if (m_new == -INFINITY) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pv[e] = 0.f;
+      } else {
+        alpha[rt] = fast_exp2(m[rt] - m_new);  // m = -inf gives 0
+        float psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          pv[e] = fast_exp2(sv[e] - m_new);
+          psum += pv[e];
+        }
+        l[rt] = l[rt] * alpha[rt] + psum;
+        m[rt] = m_new;
+      }
+      u32x4 praw = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]),
+                    pack2(pv[6], pv[7])};
+      pb[rt] = __builtin_bit_cast(bf16x8, praw);
     }
-    u32x4 praw = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]),
-                  pack2(pv[6], pv[7])};
-    const bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
 
     // ---- O^T += V^T P^T ------------------------------------------------------------
     // unwritten slots may hold anything, NaN included, and 0 * NaN must not get in:
@@ -214,8 +250,11 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       for (int w = 0; w < 4; ++w) raw[w] &= keep[w];
       const bf16x8 va = __builtin_bit_cast(bf16x8, raw);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, o[dt], 0, 0, 0);
+      for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha[rt];
+        o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[rt], o[rt][dt], 0, 0, 0);
+      }
     }
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -223,35 +262,39 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       for (int ks = 0; ks < KT; ++ks) kcur[t][ks] = knext[t][ks];
   }
 
-  // the denominator is spread over the four lanes that share a row
-  l += __shfl_xor(l, 16, HAL_WAVE);
-  l += __shfl_xor(l, 32, HAL_WAVE);
-
-  if (!row_ok) return;
-  if (partial < 0) {
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      uint2 w;
-      w.x = pack2(o[dt][0] * inv, o[dt][1] * inv);
-      w.y = pack2(o[dt][2] * inv, o[dt][3] * inv);
-      *(uint2*)(op + dt * 16 + quad * 4) = w;
-    }
-  } else {
-    float* po = part_o + (((size_t)partial * K + g) * 16 + col) * D;
+  for (int rt = 0; rt < RT; ++rt) {
+    // the denominator is spread over the four lanes that share a row
+    float lt = l[rt];
+    lt += __shfl_xor(lt, 16, HAL_WAVE);
+    lt += __shfl_xor(lt, 32, HAL_WAVE);
+    if (!row_ok[rt]) continue;
+    if (partial < 0) {
+      const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+      bf16_t* op = out + (size_t)(q_start + qi[rt]) * out_row_stride + (size_t)head[rt] * D;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      *(f32x4*)(po + dt * 16 + quad * 4) = o[dt];
-    if (quad == 0) {
-      float* pm = part_ml + (((size_t)partial * K + g) * 16 + col) * 2;
-      pm[0] = m;
-      pm[1] = l;
+      for (int dt = 0; dt < DT; ++dt) {
+        uint2 w;
+        w.x = pack2(o[rt][dt][0] * inv, o[rt][dt][1] * inv);
+        w.y = pack2(o[rt][dt][2] * inv, o[rt][dt][3] * inv);
+        *(uint2*)(op + dt * 16 + quad * 4) = w;
+      }
+    } else {
+      const size_t slot = (size_t)(partial + rt) * K + g;
+      float* po = part_o + (slot * 16 + col) * D;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *(f32x4*)(po + dt * 16 + quad * 4) = o[rt][dt];
+      if (quad == 0) {
+        float* pm = part_ml + (slot * 16 + col) * 2;
+        pm[0] = m[rt];
+        pm[1] = lt;
+      }
     }
   }
 }
 
-// merge item: {segment, first row, first partial, number of partials}
+// merge item: {segment, first row (of 16), first partial slot, number of partials,
+// slots from one partial to the next, 0, 0, 0}
 // One block per (merge item, kv head); a wave owns a row at a time, a lane two
 // dimensions.  The weights exp2(m_i - max) of up to 64 partials are computed one per
 // lane and handed round with shuffles, so that the loads of the partial sums do not
@@ -266,8 +309,8 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
   if (mi >= *n_merges_ptr) return;
   const int g = blockIdx.y;
   const int G = H / K;
-  const int* mg = merges + (size_t)mi * 4;
-  const int seg = mg[0], rho0 = mg[1], first = mg[2], n = mg[3];
+  const int* mg = merges + (size_t)mi * ITEM_INTS;
+  const int seg = mg[0], rho0 = mg[1], first = mg[2], n = mg[3], stride = mg[4];
   const int q_start = seg_q_start[seg], q_len = seg_q_len[seg];
   const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
   const int n_waves = blockDim.x / HAL_WAVE;
@@ -277,7 +320,7 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
     // the largest running maximum of the row
     float m_all = -INFINITY;
     for (int i = lane; i < n; i += HAL_WAVE)
-      m_all = fmaxf(m_all, part_ml[(((size_t)(first + i) * K + g) * 16 + row) * 2]);
+      m_all = fmaxf(m_all, part_ml[(((size_t)(first + i * stride) * K + g) * 16 + row) * 2]);
     m_all = wave_max(m_all);
     float acc[D / 128 + 1][2];
 #pragma unroll
@@ -286,7 +329,7 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
     for (int i0 = 0; i0 < n; i0 += HAL_WAVE) {
       float w = 0.f;
       if (i0 + lane < n) {
-        const size_t base = ((size_t)(first + i0 + lane) * K + g) * 16 + row;
+        const size_t base = ((size_t)(first + (i0 + lane) * stride) * K + g) * 16 + row;
         const float mi_ = part_ml[base * 2], li = part_ml[base * 2 + 1];
         w = (mi_ == -INFINITY) ? 0.f : exp2f(mi_ - m_all);
         l_all += w * li;
@@ -295,7 +338,7 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
 #pragma unroll 8
       for (int i = 0; i < cnt; ++i) {
         const float wi = __shfl(w, i, HAL_WAVE);
-        const float* po = part_o + (((size_t)(first + i0 + i) * K + g) * 16 + row) * D;
+        const float* po = part_o + (((size_t)(first + (i0 + i) * stride) * K + g) * 16 + row) * D;
 #pragma unroll
         for (int c = 0; c < D / 128 + 1; ++c) {
           const int d = c * 128 + lane * 2;
@@ -321,16 +364,28 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
 
 extern "C" int hal_attention_mfma_head_dim() { return D; }
 
-// Host arrays are device pointers: items [max_items, 8], merges [max_merges, 4], the
-// live counts in n_items / n_merges (so a captured launch can serve a varying count).
+// How many 16-row tiles a wave takes in the kernel for long segments.
+#ifndef HAL_RT_BIG
+#define HAL_RT_BIG (D <= 64 ? 4 : (D <= 128 ? 2 : 1))
+#endif
+#define RT_BIG HAL_RT_BIG
+
+extern "C" int hal_attention_mfma_rows_per_big_item() { return 16 * RT_BIG; }
+
+// All arrays are device pointers.  `items` [max_items, 8] lists the work on segments of
+// at most 16 query rows (one tile per wave), `big_items` [max_big, 8] the work on longer
+// segments (hal_attention_mfma_rows_per_big_item() rows per wave), `merges`
+// [max_merges, 8] the row tiles whose key range was cut.  counts = {items, big items,
+// merges} holds the live numbers, so a captured launch can serve varying counts.
 extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_stride,
-                                  const int* items, const int* n_items, int max_items,
-                                  const int* merges, const int* n_merges, int max_merges,
-                                  const int* seg_q_start, const int* seg_q_len,
-                                  const int* seg_kv_len, const int* block_table, int bt_stride,
-                                  const void* k_pages, const void* v_pages, float* part_o,
-                                  float* part_ml, int H, int K, int head_dim, int page_size,
-                                  float scale, int window, hipStream_t stream) {
+                                  const int* items, int max_items, const int* big_items,
+                                  int max_big, const int* merges, int max_merges,
+                                  const int* counts, const int* seg_q_start,
+                                  const int* seg_q_len, const int* seg_kv_len,
+                                  const int* block_table, int bt_stride, const void* k_pages,
+                                  const void* v_pages, float* part_o, float* part_ml, int H, int K,
+                                  int head_dim, int page_size, float scale, int window,
+                                  hipStream_t stream) {
   HAL_REQUIRE(head_dim == D, "hal_attention_mfma: built for head size %d, called with %d", D,
               head_dim);
   HAL_REQUIRE(H > 0 && K > 0 && H % K == 0, "hal_attention_mfma: %d heads, %d kv heads", H, K);
@@ -340,21 +395,35 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   HAL_REQUIRE(q_row_stride % 8 == 0 && out_row_stride % 4 == 0 && ((uintptr_t)q % 16) == 0 &&
                   ((uintptr_t)out % 8) == 0,
               "hal_attention_mfma: q and out rows must be 16-byte aligned");
-  HAL_REQUIRE(window >= 0 && max_items >= 0 && max_merges >= 0, "hal_attention_mfma: bad counts");
+  HAL_REQUIRE(window >= 0 && max_items >= 0 && max_big >= 0 && max_merges >= 0,
+              "hal_attention_mfma: bad counts");
   HAL_REQUIRE(max_merges == 0 || (part_o && part_ml), "hal_attention_mfma: no partial buffers");
-  if (max_items == 0) return 0;
   const float scale_log2e = scale * 1.4426950408889634f;
+  int page_shift = -1;
+  if ((page_size & (page_size - 1)) == 0)
+    for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
   const int waves = 4;
-  dim3 grid((max_items + waves - 1) / waves, K);
-  hipLaunchKernelGGL(attention_mfma_kernel, grid, dim3(waves * HAL_WAVE), 0, stream,
-                     (const bf16_t*)q, q_row_stride, (bf16_t*)out, out_row_stride, items, n_items,
-                     seg_q_start, seg_q_len, seg_kv_len, block_table, bt_stride,
-                     (const bf16_t*)k_pages, (const bf16_t*)v_pages, part_o, part_ml, H, K,
-                     page_size, scale_log2e, window);
-  HAL_LAUNCH_CHECK();
+  if (max_items > 0) {
+    dim3 grid((max_items + waves - 1) / waves, K);
+    hipLaunchKernelGGL(attention_mfma_kernel<1>, grid, dim3(waves * HAL_WAVE), 0, stream,
+                       (const bf16_t*)q, q_row_stride, (bf16_t*)out, out_row_stride, items,
+                       counts, seg_q_start, seg_q_len, seg_kv_len, block_table, bt_stride,
+                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, part_o, part_ml, H, K,
+                       page_size, page_shift, scale_log2e, window);
+    HAL_LAUNCH_CHECK();
+  }
+  if (max_big > 0) {
+    dim3 grid((max_big + waves - 1) / waves, K);
+    hipLaunchKernelGGL(attention_mfma_kernel<RT_BIG>, grid, dim3(waves * HAL_WAVE), 0, stream,
+                       (const bf16_t*)q, q_row_stride, (bf16_t*)out, out_row_stride, big_items,
+                       counts + 1, seg_q_start, seg_q_len, seg_kv_len, block_table, bt_stride,
+                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, part_o, part_ml, H, K,
+                       page_size, page_shift, scale_log2e, window);
+    HAL_LAUNCH_CHECK();
+  }
   if (max_merges > 0) {
     hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K), dim3(256), 0, stream,
-                       (bf16_t*)out, out_row_stride, merges, n_merges, seg_q_start, seg_q_len,
+                       (bf16_t*)out, out_row_stride, merges, counts + 2, seg_q_start, seg_q_len,
                        part_o, part_ml, H, K);
     HAL_LAUNCH_CHECK();
   }

@@ -48,12 +48,13 @@ int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temp
 
 // ---- the head-size-specific library (attention_mfma.hip) ---------------------------------
 int hal_attention_mfma_head_dim();
+int hal_attention_mfma_rows_per_big_item();
 int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_stride,
-                       const int* items, const int* n_items, int max_items, const int* merges,
-                       const int* n_merges, int max_merges, const int* seg_q_start,
-                       const int* seg_q_len, const int* seg_kv_len, const int* block_table,
-                       int bt_stride, const void* k_pages, const void* v_pages, float* part_o,
-                       float* part_ml, int H, int K, int head_dim, int page_size, float scale,
-                       int window, hipStream_t stream);
+                       const int* items, int max_items, const int* big_items, int max_big,
+                       const int* merges, int max_merges, const int* counts,
+                       const int* seg_q_start, const int* seg_q_len, const int* seg_kv_len,
+                       const int* block_table, int bt_stride, const void* k_pages,
+                       const void* v_pages, float* part_o, float* part_ml, int H, int K,
+                       int head_dim, int page_size, float scale, int window, hipStream_t stream);
 
 }  // extern "C"

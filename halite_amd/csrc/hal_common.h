@@ -42,6 +42,15 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
   return __uint_as_float(((uint32_t)v.bits) << 16);
 }
 
+// two floats to two bf16 in one word (first in the low half), round to nearest even,
+// with the hardware's conversion
+typedef __attribute__((ext_vector_type(2))) __bf16 hal_bf16x2;
+typedef __attribute__((ext_vector_type(2))) float hal_f32x2;
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const hal_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, hal_bf16x2));
+}
+
 // round to nearest even; NaN stays NaN
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
   uint32_t u = __float_as_uint(f);
@@ -85,8 +94,8 @@ __device__ __forceinline__ void store4(float* p, const float (&v)[4]) {
 }
 __device__ __forceinline__ void store4(bf16_t* p, const float (&v)[4]) {
   uint2 t;
-  t.x = (uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16);
-  t.y = (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16);
+  t.x = pack_bf16x2(v[0], v[1]);
+  t.y = pack_bf16x2(v[2], v[3]);
   *(uint2*)p = t;
 }
 __device__ __forceinline__ void load4_any(const void* p, int dtype, size_t i, float (&v)[4]) {

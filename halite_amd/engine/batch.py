@@ -184,30 +184,31 @@ class StepContext:
 
     # The plans of the attention kernel are part of the same upload, so they are
     # declared before the first device access.
-    def plan_attention(self, group_id: int, n_heads: int, n_kv_heads: int, window: int, late=False) -> None:
+    def plan_attention(self, group_id: int, n_heads: int, n_kv_heads: int, window: int,
+                       head_dim: int = 128, late=False) -> None:
         key = (group_id, n_heads // n_kv_heads, window)
         if key in self._plan_host:
             return
         if self._dev is not None and not late:
             return
         plan = attention_kernels.plan_items(
-            self.seg_q_len_host, self.seg_kv_len_host, n_heads // n_kv_heads, n_kv_heads, window
+            self.seg_q_len_host, self.seg_kv_len_host, n_heads // n_kv_heads, n_kv_heads, window,
+            attention_kernels.rows_per_big_item(head_dim),
         )
         self._plan_host[key] = plan
         plan.name = f"plan{len(self._plan_host)}"
-        counts = np.array([plan.n_items, plan.n_merges], dtype=np.int32)
         if self._dev is None:
             cap = self.static.max_items if self.static is not None else None
-            if cap is not None:
-                plan.cap_items, plan.cap_merges = cap, min(cap, self.n_segs)
+            if cap is not None:  # decode only: no long segments
+                plan.cap_items, plan.cap_merges, plan.cap_partials = cap, min(cap, self.n_segs), cap
             self._packer.add(plan.name + "_items", plan.items, None if cap is None else cap * 8)
-            self._packer.add(plan.name + "_merges", plan.merges, None if cap is None else plan.cap_merges * 4)
-            self._packer.add(plan.name + "_counts", counts)
+            self._packer.add(plan.name + "_big", plan.big_items)
+            self._packer.add(plan.name + "_merges", plan.merges, None if cap is None else plan.cap_merges * 8)
+            self._packer.add(plan.name + "_counts", plan.counts())
         else:  # declared after the step's upload: a copy of its own
             if self.static is not None:
                 raise RuntimeError("a static step needs its attention plans before the upload")
-            dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(self.device)
-            self._plans[key] = (plan, dev(plan.items), dev(plan.merges), dev(counts))
+            self._plans[key] = attention_kernels.upload_plan(plan, self.device)
 
     def upload(self):
         if self._dev is not None:
@@ -254,15 +255,20 @@ class StepContext:
         if plan is None:
             return None
         if key not in self._plans:
-            off, _ = self._packer.offsets[plan.name + "_items"]
             self.upload()
-            items = self._dev[off : off + plan.cap_items * 8].view(-1, 8)
-            off, _ = self._packer.offsets[plan.name + "_merges"]
-            merges = self._dev[off : off + max(plan.cap_merges, 1) * 4].view(-1, 4)
+
+            def piece(name, rows):
+                off, _ = self._packer.offsets[plan.name + name]
+                return self._dev[off : off + rows * 8].view(rows, 8)
+
             counts = self._view(plan.name + "_counts")
-            self._plans[key] = (plan, items, merges, counts)
+            self._plans[key] = (plan, piece("_items", plan.cap_items), piece("_big", plan.cap_big),
+                                piece("_merges", plan.cap_merges), counts)
         return self._plans[key]
 
     def fits_static(self) -> bool:
         """Whether every plan of this step fits the static layout's capacities."""
-        return all(p.n_items <= p.cap_items and p.n_merges <= p.cap_merges for p in self._plan_host.values())
+        return all(
+            p.n_items <= p.cap_items and p.n_merges <= p.cap_merges and p.n_partials <= p.cap_partials and p.n_big == 0
+            for p in self._plan_host.values()
+        )

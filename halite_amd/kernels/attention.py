@@ -26,59 +26,89 @@ TARGET_WAVES = 2048
 
 @dataclass
 class AttentionPlan:
-    items: np.ndarray  # [n_items, 8] int32: segment, first row, first key, end key, partial, 0, 0, 0
-    merges: np.ndarray  # [n_merges, 4] int32: segment, first row, first partial, count
-    n_items: int
-    n_merges: int
-    n_partials: int
+    """Work lists of the matrix-core kernel for one step (rows are (token, head of the
+    group) pairs, token-major):
+    ``items`` [n, 8]: segment, first row, first key, end key, first partial slot or -1 —
+    tiles of 16 rows of segments with at most 16 rows (decode tokens);
+    ``big_items`` the same for longer segments, ``rows_big`` rows per tile;
+    ``merges`` [n, 8]: segment, first row of a 16-row tile, first partial slot, number of
+    partials, slots between partials."""
+
+    items: np.ndarray
+    big_items: np.ndarray
+    merges: np.ndarray
+    n_partials: int  # partial slots (one per 16 rows and piece)
+    rows_big: int = 64
     name: str = ""
     # room in the device arrays (larger than the live counts under a static layout)
     cap_items: int = 0
+    cap_big: int = 0
     cap_merges: int = 0
+    cap_partials: int = 0
 
     def __post_init__(self):
-        self.cap_items = max(self.cap_items, self.n_items)
-        self.cap_merges = max(self.cap_merges, self.n_merges)
+        self.cap_items = max(self.cap_items, len(self.items))
+        self.cap_big = max(self.cap_big, len(self.big_items))
+        self.cap_merges = max(self.cap_merges, len(self.merges))
+        self.cap_partials = max(self.cap_partials, self.n_partials)
+
+    @property
+    def n_items(self):
+        return len(self.items)
+
+    @property
+    def n_big(self):
+        return len(self.big_items)
+
+    @property
+    def n_merges(self):
+        return len(self.merges)
+
+    def counts(self) -> np.ndarray:
+        return np.array([self.n_items, self.n_big, self.n_merges], dtype=np.int32)
 
 
 def mfma_supported(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
     return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and page_size % 8 == 0
 
 
-def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: int) -> AttentionPlan:
-    """Cuts the step's query rows into tiles of 16 rows (a row is a token and a head
-    of the group, token-major) and, where there are too few tiles to fill the GPU,
-    cuts a tile's key range into pieces whose partial results are merged."""
+def rows_per_big_item(head_dim: int) -> int:
+    """Rows of a wave's tile for long segments; the kernel's HAL_RT_BIG times 16."""
+    return 64 if head_dim <= 64 else (32 if head_dim <= 128 else 16)
+
+
+def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick):
     seg_ids, rho0s, kv_b, kv_e = [], [], [], []
     for s, (ql, kl) in enumerate(zip(seg_q_len, seg_kv_len)):
         ql, kl = int(ql), int(kl)
         rows = ql * group_size
-        r0 = np.arange(0, rows, ROWS_PER_ITEM, dtype=np.int64)
+        if not pick(rows):
+            continue
+        r0 = np.arange(0, rows, rows_per_tile, dtype=np.int64)
         first_q = r0 // group_size
-        last_q = np.minimum(rows - 1, r0 + ROWS_PER_ITEM - 1) // group_size
+        last_q = np.minimum(rows - 1, r0 + rows_per_tile - 1) // group_size
         pos0 = kl - ql
         b = np.zeros_like(r0) if window <= 0 else np.maximum(0, pos0 + first_q - window + 1)
         e = pos0 + last_q + 1
         seg_ids.append(np.full(r0.shape, s, dtype=np.int64))
         rho0s.append(r0), kv_b.append(b), kv_e.append(e)
     if not seg_ids:
-        z = np.zeros((0, 8), dtype=np.int32)
-        return AttentionPlan(z, np.zeros((0, 4), dtype=np.int32), 0, 0, 0)
-    seg_ids, rho0s = np.concatenate(seg_ids), np.concatenate(rho0s)
-    kv_b, kv_e = np.concatenate(kv_b), np.concatenate(kv_e)
-    span = kv_e - kv_b
-    if len(span) * n_kv_heads * 2 >= TARGET_WAVES:
-        chunk = 1 << 30  # enough tiles to fill the GPU: nothing is cut
-    else:
-        total = int(span.sum()) * n_kv_heads
-        chunk = -(-total // TARGET_WAVES)
-        chunk = max(MIN_SPLIT_KEYS, -(-chunk // KEYS_PER_BLOCK) * KEYS_PER_BLOCK)
-    base = kv_b - kv_b % KEYS_PER_BLOCK  # pieces end on multiples of 32 keys
-    n_pieces = np.maximum(1, -(-(kv_e - base) // chunk))
+        z = np.zeros(0, dtype=np.int64)
+        return z, z, z, z
+    return np.concatenate(seg_ids), np.concatenate(rho0s), np.concatenate(kv_b), np.concatenate(kv_e)
 
+
+def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_seg):
+    """Items and merge entries of tiles whose key ranges are cut into pieces of
+    ``chunk`` keys (pieces end on multiples of 32 keys)."""
+    n_tiles = len(seg_ids)
+    if n_tiles == 0:
+        return np.zeros((0, 8), np.int32), np.zeros((0, 8), np.int32), first_slot
+    base = kv_b - kv_b % KEYS_PER_BLOCK
+    n_pieces = np.maximum(1, -(-(kv_e - base) // chunk))
     n_items = int(n_pieces.sum())
     items = np.zeros((n_items, 8), dtype=np.int32)
-    tile_of = np.repeat(np.arange(len(span)), n_pieces)
+    tile_of = np.repeat(np.arange(n_tiles), n_pieces)
     first_item = np.concatenate(([0], np.cumsum(n_pieces)[:-1]))
     piece = np.arange(n_items) - first_item[tile_of]
     items[:, 0] = seg_ids[tile_of]
@@ -87,33 +117,55 @@ def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: 
     items[:, 3] = np.minimum(kv_e[tile_of], base[tile_of] + (piece + 1) * chunk)
     split = n_pieces[tile_of] > 1
     items[:, 4] = -1
-    n_partials = int(split.sum())
-    items[split, 4] = np.arange(n_partials)
-    split_tiles = np.nonzero(n_pieces > 1)[0]
-    merges = np.zeros((len(split_tiles), 4), dtype=np.int32)
-    if len(split_tiles):
-        merges[:, 0] = seg_ids[split_tiles]
-        merges[:, 1] = rho0s[split_tiles]
-        merges[:, 2] = items[first_item[split_tiles], 4]
-        merges[:, 3] = n_pieces[split_tiles]
-    return AttentionPlan(items, merges, n_items, len(split_tiles), n_partials)
+    n_split = int(split.sum())
+    items[split, 4] = first_slot + np.arange(n_split) * slots_per_tile
+    merges = []
+    for t in np.nonzero(n_pieces > 1)[0]:
+        slot0 = int(items[first_item[t], 4])
+        rows_left = rows_of_seg[int(seg_ids[t])] - int(rho0s[t])
+        for sub in range(min(slots_per_tile, -(-rows_left // ROWS_PER_ITEM))):
+            merges.append([seg_ids[t], rho0s[t] + sub * ROWS_PER_ITEM, slot0 + sub, n_pieces[t], slots_per_tile, 0, 0, 0])
+    merges = np.array(merges, dtype=np.int32).reshape(-1, 8)
+    # the longest key ranges first: the waves that run longest start earliest
+    order = np.argsort(-(items[:, 3] - items[:, 2]), kind="stable")
+    return items[order], merges, first_slot + n_split * slots_per_tile
+
+
+def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: int,
+               rows_big: int = 64) -> AttentionPlan:
+    """Cuts the step's query rows into tiles: 16 rows for segments of at most 16 rows,
+    ``rows_big`` rows for longer ones; where there are too few tiles to fill the GPU, a
+    tile's key range is cut into pieces whose partial results are merged."""
+    rows_of_seg = [int(q) * group_size for q in seg_q_len]
+    small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: r <= ROWS_PER_ITEM or rows_big <= ROWS_PER_ITEM)
+    big = _tiles(seg_q_len, seg_kv_len, group_size, window, rows_big, lambda r: r > ROWS_PER_ITEM and rows_big > ROWS_PER_ITEM)
+    n_tiles = len(small[0]) + len(big[0])
+    if n_tiles * n_kv_heads * 2 >= TARGET_WAVES or n_tiles == 0:
+        chunk = 1 << 30  # enough tiles to fill the GPU: nothing is cut
+    else:
+        total = int((small[3] - small[2]).sum() + (big[3] - big[2]).sum()) * n_kv_heads
+        chunk = -(-total // TARGET_WAVES)
+        chunk = max(MIN_SPLIT_KEYS, -(-chunk // KEYS_PER_BLOCK) * KEYS_PER_BLOCK)
+    items, merges_s, slot = _cut(*small, chunk, 1, 0, rows_of_seg)
+    big_items, merges_b, slot = _cut(*big, chunk, rows_big // ROWS_PER_ITEM, slot, rows_of_seg)
+    merges = np.concatenate((merges_s, merges_b)) if len(merges_s) or len(merges_b) else np.zeros((0, 8), np.int32)
+    return AttentionPlan(items, big_items, merges, slot, rows_big)
 
 
 def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, window):
-    plan, items, merges, counts = plan_dev
+    plan, items, big_items, merges, counts = plan_dev
     n_pages, n_kv, page_size, head_dim = kv.k.shape
     lib = library.attention_library(head_dim)
     n = ctx.n_tokens
     out = torch.empty((n, n_heads * head_dim), dtype=torch.bfloat16, device=q.device)
     part_o = part_ml = None
-    n_part = plan.cap_items if plan.cap_items > plan.n_items else plan.n_partials
-    if n_part and plan.cap_merges:
-        part_o = torch.empty((n_part, n_kv, 16, head_dim), dtype=torch.float32, device=q.device)
-        part_ml = torch.empty((n_part, n_kv, 16, 2), dtype=torch.float32, device=q.device)
+    if plan.cap_partials and plan.cap_merges:
+        part_o = torch.empty((plan.cap_partials, n_kv, 16, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((plan.cap_partials, n_kv, 16, 2), dtype=torch.float32, device=q.device)
     P = ops._ptr
     rc = lib.hal_attention_mfma(
         P(q), q_row_stride, P(out), n_heads * head_dim,
-        P(items), P(counts[0:1]), plan.cap_items, P(merges), P(counts[1:2]), plan.cap_merges,
+        P(items), plan.cap_items, P(big_items), plan.cap_big, P(merges), plan.cap_merges, P(counts),
         P(ctx.seg_q_start), P(ctx.seg_q_len), P(ctx.seg_kv_len),
         P(group.block_table), group.block_table.shape[1], P(kv.k), P(kv.v), P(part_o), P(part_ml),
         n_heads, n_kv, head_dim, page_size, ctypes.c_float(scale), window, ops._stream(),
@@ -122,12 +174,18 @@ def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, wi
     return out
 
 
+def upload_plan(plan: AttentionPlan, device):
+    """A plan's arrays on the device, as ``attention_mfma`` takes them."""
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    return (plan, dev(plan.items), dev(plan.big_items), dev(plan.merges), dev(plan.counts()))
+
+
 def paged_attention(ctx, q, q_row_stride, kv, group, n_heads, scale, window):
     n_pages, n_kv, page_size, head_dim = kv.k.shape
     if mfma_supported(q.dtype, head_dim, page_size) and q_row_stride % 8 == 0:
         plan_dev = ctx.device_plan(group.group_id, n_heads // n_kv, window)
         if plan_dev is None:
-            ctx.plan_attention(group.group_id, n_heads, n_kv, window, late=True)
+            ctx.plan_attention(group.group_id, n_heads, n_kv, window, head_dim, late=True)
             plan_dev = ctx.device_plan(group.group_id, n_heads // n_kv, window)
         return attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, window)
     return ops.attention_simple(

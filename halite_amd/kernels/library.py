@@ -189,11 +189,18 @@ def attention_library(head_dim: int) -> ctypes.CDLL:
     return load_library(f"attn_d{head_dim}", ATTENTION_SOURCES, {"HAL_HEAD_DIM": head_dim})
 
 
-def build_all(head_dims=(16, 32, 64, 128), force=True) -> list[str]:
-    """Compile every library for the given head sizes (the build check)."""
+def build_all(head_dims=(16, 32, 64, 128), force=True, prune=True) -> list[str]:
+    """Compile every library for the given head sizes (the build check); with
+    ``prune`` builds of older sources are removed from the in-tree build folder."""
     paths = [build_library("core", CORE_SOURCES, {}, force=force)]
     for d in head_dims:
         paths.append(
             build_library(f"attn_d{d}", ATTENTION_SOURCES, {"HAL_HEAD_DIM": d}, force=force)
         )
+    if prune:
+        folder = _build_dirs()[0]
+        keep = {os.path.basename(p) for p in paths}
+        for name in os.listdir(folder) if os.path.isdir(folder) else []:
+            if name.startswith("libhalite_") and name.endswith(".so") and name not in keep:
+                os.remove(os.path.join(folder, name))
     return paths

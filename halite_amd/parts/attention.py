@@ -87,7 +87,7 @@ class Attention(Mixer):
     def prepare(self, ctx, run):
         group = ctx.cache.groups[run.kv.group_id]
         if attention_kernels.mfma_supported(self.build.dtype, self.p.head_dim, group.page_size):
-            ctx.plan_attention(group.group_id, self.p.n_heads, self.p.n_kv_heads, self.p.window or 0)
+            ctx.plan_attention(group.group_id, self.p.n_heads, self.p.n_kv_heads, self.p.window or 0, self.p.head_dim)
 
     def forward(self, x, ctx, run):
         p = self.p

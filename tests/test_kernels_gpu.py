@@ -183,7 +183,7 @@ def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use):
     else:
         q_len = np.array([n for _, n in segs], dtype=np.int32)
         kv_len = np.array([b + n for b, n in segs], dtype=np.int32)
-        plan = attn_kernels.plan_items(q_len, kv_len, H // K, K, window)
+        plan = attn_kernels.plan_items(q_len, kv_len, H // K, K, window, attn_kernels.rows_per_big_item(D))
         dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
 
         class Ctx:
@@ -198,8 +198,7 @@ def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use):
         class KV:
             k, v = k_pages, v_pages
 
-        counts = dev(np.array([plan.n_items, plan.n_merges], dtype=np.int32))
-        out = attn_kernels.attention_mfma(q, H * D, (plan, dev(plan.items), dev(plan.merges), counts), Ctx, Group, KV, H, scale, window)
+        out = attn_kernels.attention_mfma(q, H * D, attn_kernels.upload_plan(plan, gpu), Ctx, Group, KV, H, scale, window)
     close(out, torch.cat(want), 5e-6 if dtype == "float32" else 1.2e-2, f"attention {use}")
 
 
@@ -226,9 +225,12 @@ def test_attention_mfma_split_keys(gpu):
     # few rows and many keys: the key range is cut and merged
     segs = [(3000, 1), (1500, 2), (4000, 1)]
     plan = attn_kernels.plan_items(np.array([1, 2, 1]), np.array([3001, 1502, 4001]), 4, 2, 0)
-    assert plan.n_merges == 3
+    assert plan.n_merges == 3 and plan.n_big == 0
     attention_case(gpu, "bfloat16", 8, 2, 128, 64, segs, 0, seed=40, use="mfma")
     attention_case(gpu, "bfloat16", 8, 2, 128, 16, segs, 1000, seed=41, use="mfma")
+    # a short portion against a long context: tiles of 64 rows, cut and merged
+    attention_case(gpu, "bfloat16", 8, 2, 128, 64, [(5000, 40), (2500, 100)], 0, seed=42, use="mfma")
+    attention_case(gpu, "bfloat16", 6, 2, 48, 16, [(3000, 50)], 700, seed=43, use="mfma")
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 256, 64), (5, 331, 120), (64, 200, 352), (130, 96, 1000), (3, 4096, 4096)])
