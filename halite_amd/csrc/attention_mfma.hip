@@ -34,6 +34,7 @@ static_assert(HAL_HEAD_DIM % 16 == 0 && HAL_HEAD_DIM >= 16 && HAL_HEAD_DIM <= 25
 #define KT ((D + 31) / 32)  // 32-wide steps over the head dimension for Q K^T
 #define DT (D / 16)         // 16-wide tiles of the head dimension for P V
 #define ITEM_INTS 8
+#define RESCALE_SLACK 8.0f  // in powers of two
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -50,11 +51,14 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16
 // 2^x for x <= 0 (results below the normal range may flush to zero)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// item: {segment, first row, first key, end key, first partial slot or -1, 0, 0, 0}
-// A wave works on RT tiles of 16 rows (rows first row .. first row + 16*RT); the keys
-// and values it loads serve all of them.  Row tile rt of an item writes partial slot
-// `first partial slot + rt`.
-template <int RT>
+// item: {segment, first row of tile 0, first key, end key, first partial slot or -1,
+//        first row of tile 1, of tile 2, of tile 3 (or -1)}
+// A wave works on up to RT tiles of 16 rows of one segment; the keys and values it
+// loads serve all of them.  The tiles need not be neighbours: pairing an early tile of
+// a prompt with a late one gives every wave the same amount of causal work.  A tile
+// skips the blocks of keys that lie wholly outside its own range.  Row tile rt of an
+// item writes partial slot `first partial slot + rt`.
+template <int RT, bool POW2>
 __global__ void __launch_bounds__(256)
 attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
                       int out_row_stride, const int* __restrict__ items,
@@ -84,8 +88,9 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   float m[RT], l[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int rho = rho0 + rt * 16 + col;
-    row_ok[rt] = rho < q_len * G;
+    const int tile0 = rt == 0 ? rho0 : it[4 + rt];
+    const int rho = tile0 + col;
+    row_ok[rt] = tile0 >= 0 && rho < q_len * G;
     qi[rt] = row_ok[rt] ? rho / G : 0;
     head[rt] = g * G + (row_ok[rt] ? rho % G : 0);
     p_row[rt] = pos0 + qi[rt];  // the row's position: it sees keys <= p_row
@@ -94,7 +99,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 #pragma unroll
     for (int ks = 0; ks < KT; ++ks) {
       const int d0 = ks * 32 + quad * 8;
-      bq[rt][ks] = (row_ok[rt] && d0 < D) ? ld16(qp + d0) : zero8();
+      bq[rt][ks] = (row_ok[rt] && (D % 32 == 0 || d0 < D)) ? ld16(qp + d0) : zero8();
     }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -104,19 +109,21 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 
   const int last_key = kv_len - 1;  // keys beyond it are not written yet
   // page and slot of a key; pages of a power of two (page_shift >= 0) need no division
-  auto page_of = [&](int j) { return page_shift >= 0 ? j >> page_shift : j / page_size; };
-  auto slot_of = [&](int j) { return page_shift >= 0 ? j & (page_size - 1) : j % page_size; };
+  auto page_of = [&](int j) { return POW2 ? j >> page_shift : j / page_size; };
+  auto slot_of = [&](int j) { return POW2 ? j & (page_size - 1) : j % page_size; };
   // per row tile, the positions of its first and last row (uniform over the wave): a
   // block of keys wholly below the first row's position needs no mask
-  int p_first[RT], lo_last[RT];
+  int p_first[RT], p_last[RT], lo_first[RT], lo_last[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int r_first = rho0 + rt * 16;
+    const int r_first = rt == 0 ? rho0 : it[4 + rt];
     int r_last = r_first + 15;
     if (r_last > q_len * G - 1) r_last = q_len * G - 1;
+    if (r_last < r_first) r_last = r_first;
     p_first[rt] = pos0 + r_first / G;
-    const int p_last = pos0 + (r_last > r_first ? r_last : r_first) / G;
-    lo_last[rt] = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+    p_last[rt] = r_first >= 0 ? pos0 + r_last / G : -1;  // no tile: no key is in range
+    lo_first[rt] = (window > 0 && p_first[rt] - window + 1 > 0) ? p_first[rt] - window + 1 : 0;
+    lo_last[rt] = (window > 0 && p_last[rt] - window + 1 > 0) ? p_last[rt] - window + 1 : 0;
   }
 
   // This lane's key of tile t in the block of 32 keys at j0: row `col` of tile t is
@@ -142,7 +149,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 #pragma unroll
       for (int ks = 0; ks < KT; ++ks) {
         const int d0 = ks * 32 + quad * 8;
-        kf[t][ks] = d0 < D ? ld16(kp + d0) : zero8();
+        if constexpr (D % 32 == 0) kf[t][ks] = ld16(kp + d0);
+        else kf[t][ks] = d0 < D ? ld16(kp + d0) : zero8();
       }
     }
   };
@@ -177,8 +185,15 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 
     bf16x8 pb[RT];
     float alpha[RT];
+    bool active[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
+      // a block wholly after the tile's last row or before its first row's window
+      // does nothing for this tile
+      active[rt] = j0 <= p_last[rt] && j0 + 31 >= lo_first[rt];
+      alpha[rt] = 1.f;
+      pb[rt] = zero8();
+      if (!active[rt]) continue;
       // ---- S^T = K Q^T for 32 keys (two tiles of 16) ----------------------------
       f32x4 s[2];
 #pragma unroll
@@ -211,23 +226,24 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       }
       m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, HAL_WAVE));
       m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, HAL_WAVE));
-      const float m_new = fmaxf(m[rt], m_tile);
-      alpha[rt] = 1.f;
+      // The running maximum only has to keep exp2(s - m) in range, so it is raised
+      // only when the block's maximum exceeds it by more than 2^RESCALE_SLACK: then
+      // the accumulated sums are rarely rescaled (and a partial result's m, l and sums
+      // stay consistent with each other, which is all the merge needs).
+      const float m_new = m_tile > m[rt] + RESCALE_SLACK ? m_tile : m[rt];
+      // a row that has seen no key yet keeps m = -inf; subtracting 0 instead of -inf
+      // gives exp2(-inf) = 0 everywhere without a branch
+      const float m_sub = m_new == -INFINITY ? 0.f : m_new;
+      alpha[rt] = fast_exp2(m[rt] - m_sub);
       float pv[8];
-      if (m_new == -INFINITY) {
+      float psum = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) pv[e] = 0.f;
-      } else {
-        alpha[rt] = fast_exp2(m[rt] - m_new);  // m = -inf gives 0
-        float psum = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          pv[e] = fast_exp2(sv[e] - m_new);
-          psum += pv[e];
-        }
-        l[rt] = l[rt] * alpha[rt] + psum;
-        m[rt] = m_new;
+      for (int e = 0; e < 8; ++e) {
+        pv[e] = fast_exp2(sv[e] - m_sub);
+        psum += pv[e];
       }
+      l[rt] = l[rt] * alpha[rt] + psum;
+      m[rt] = m_new;
       u32x4 praw = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]),
                     pack2(pv[6], pv[7])};
       pb[rt] = __builtin_bit_cast(bf16x8, praw);
@@ -236,25 +252,36 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     // ---- O^T += V^T P^T ------------------------------------------------------------
     // unwritten slots may hold anything, NaN included, and 0 * NaN must not get in:
     // in the last block of the request the values of keys past the end are cleared
-    uint32_t keep[4];
+    if (tail) {
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const int ja = jv + 2 * w;
-      keep[w] = tail ? ((ja <= last_key ? 0x0000ffffu : 0u) | (ja + 1 <= last_key ? 0xffff0000u : 0u))
-                     : 0xffffffffu;
+      for (int w = 0; w < 4; ++w) {
+        const int ja = jv + 2 * w;
+        const uint32_t keep =
+            (ja <= last_key ? 0x0000ffffu : 0u) | (ja + 1 <= last_key ? 0xffff0000u : 0u);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          u32x4 raw = __builtin_bit_cast(u32x4, vf[dt]);
+          raw[w] &= keep;
+          vf[dt] = __builtin_bit_cast(bf16x8, raw);
+        }
+      }
     }
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      u32x4 raw = __builtin_bit_cast(u32x4, vf[dt]);
+    for (int rt = 0; rt < RT; ++rt) {
+      // rescale the sums only if some row of the tile raised its maximum
+      if (__builtin_amdgcn_ballot_w64(alpha[rt] != 1.f) != 0) {
 #pragma unroll
-      for (int w = 0; w < 4; ++w) raw[w] &= keep[w];
-      const bf16x8 va = __builtin_bit_cast(bf16x8, raw);
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha[rt];
-        o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[rt], o[rt][dt], 0, 0, 0);
+          for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha[rt];
       }
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      if (!active[rt]) continue;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb[rt], o[rt][dt], 0, 0, 0);
     }
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -405,7 +432,8 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   const int waves = 4;
   if (max_items > 0) {
     dim3 grid((max_items + waves - 1) / waves, K);
-    hipLaunchKernelGGL(attention_mfma_kernel<1>, grid, dim3(waves * HAL_WAVE), 0, stream,
+    hipLaunchKernelGGL((page_shift >= 0 ? attention_mfma_kernel<1, true> : attention_mfma_kernel<1, false>),
+                       grid, dim3(waves * HAL_WAVE), 0, stream,
                        (const bf16_t*)q, q_row_stride, (bf16_t*)out, out_row_stride, items,
                        counts, seg_q_start, seg_q_len, seg_kv_len, block_table, bt_stride,
                        (const bf16_t*)k_pages, (const bf16_t*)v_pages, part_o, part_ml, H, K,
@@ -414,7 +442,8 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   }
   if (max_big > 0) {
     dim3 grid((max_big + waves - 1) / waves, K);
-    hipLaunchKernelGGL(attention_mfma_kernel<RT_BIG>, grid, dim3(waves * HAL_WAVE), 0, stream,
+    hipLaunchKernelGGL((page_shift >= 0 ? attention_mfma_kernel<RT_BIG, true> : attention_mfma_kernel<RT_BIG, false>),
+                       grid, dim3(waves * HAL_WAVE), 0, stream,
                        (const bf16_t*)q, q_row_stride, (bf16_t*)out, out_row_stride, big_items,
                        counts + 1, seg_q_start, seg_q_len, seg_kv_len, block_table, bt_stride,
                        (const bf16_t*)k_pages, (const bf16_t*)v_pages, part_o, part_ml, H, K,

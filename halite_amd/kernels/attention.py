@@ -98,9 +98,10 @@ def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick):
     return np.concatenate(seg_ids), np.concatenate(rho0s), np.concatenate(kv_b), np.concatenate(kv_e)
 
 
-def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_seg):
+def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_seg, more_tiles=None):
     """Items and merge entries of tiles whose key ranges are cut into pieces of
-    ``chunk`` keys (pieces end on multiples of 32 keys)."""
+    ``chunk`` keys (pieces end on multiples of 32 keys).  ``more_tiles`` [n, k] holds
+    the first rows of an item's further 16-row tiles (-1: none)."""
     n_tiles = len(seg_ids)
     if n_tiles == 0:
         return np.zeros((0, 8), np.int32), np.zeros((0, 8), np.int32), first_slot
@@ -115,6 +116,9 @@ def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_
     items[:, 1] = rho0s[tile_of]
     items[:, 2] = np.maximum(kv_b[tile_of], base[tile_of] + piece * chunk)
     items[:, 3] = np.minimum(kv_e[tile_of], base[tile_of] + (piece + 1) * chunk)
+    items[:, 5:] = -1
+    if more_tiles is not None:
+        items[:, 5 : 5 + more_tiles.shape[1]] = more_tiles[tile_of]
     split = n_pieces[tile_of] > 1
     items[:, 4] = -1
     n_split = int(split.sum())
@@ -122,32 +126,61 @@ def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_
     merges = []
     for t in np.nonzero(n_pieces > 1)[0]:
         slot0 = int(items[first_item[t], 4])
-        rows_left = rows_of_seg[int(seg_ids[t])] - int(rho0s[t])
-        for sub in range(min(slots_per_tile, -(-rows_left // ROWS_PER_ITEM))):
-            merges.append([seg_ids[t], rho0s[t] + sub * ROWS_PER_ITEM, slot0 + sub, n_pieces[t], slots_per_tile, 0, 0, 0])
+        firsts = [int(rho0s[t])] + ([int(r) for r in more_tiles[t]] if more_tiles is not None else [])
+        for sub, r0 in enumerate(firsts):
+            if r0 >= 0:
+                merges.append([seg_ids[t], r0, slot0 + sub, n_pieces[t], slots_per_tile, 0, 0, 0])
     merges = np.array(merges, dtype=np.int32).reshape(-1, 8)
     # the longest key ranges first: the waves that run longest start earliest
     order = np.argsort(-(items[:, 3] - items[:, 2]), kind="stable")
     return items[order], merges, first_slot + n_split * slots_per_tile
 
 
+def _group_tiles(seg_ids, rho0s, kv_b, kv_e, per_item: int, zigzag: bool):
+    """Groups 16-row tiles of one segment into items of ``per_item`` tiles.  With
+    ``zigzag`` an early tile goes together with a late one (tile i with tile n-1-i), so
+    that every item has about the same number of (tile, key block) pairs under the
+    causal rule; otherwise neighbours go together."""
+    out_seg, out_rho, out_b, out_e, more = [], [], [], [], []
+    for s in np.unique(seg_ids):
+        idx = np.nonzero(seg_ids == s)[0]  # in row order
+        n = len(idx)
+        if zigzag and per_item == 2:
+            groups = [[idx[i], idx[n - 1 - i]] if i != n - 1 - i else [idx[i]] for i in range((n + 1) // 2)]
+        else:
+            groups = [list(idx[i : i + per_item]) for i in range(0, n, per_item)]
+        for grp in groups:
+            out_seg.append(s)
+            out_rho.append(rho0s[grp[0]])
+            out_b.append(min(kv_b[t] for t in grp))
+            out_e.append(max(kv_e[t] for t in grp))
+            more.append([rho0s[t] for t in grp[1:]] + [-1] * (per_item - len(grp)))
+    arr = lambda x: np.array(x, dtype=np.int64)
+    return arr(out_seg), arr(out_rho), arr(out_b), arr(out_e), arr(more).reshape(len(out_seg), per_item - 1)
+
+
 def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: int,
                rows_big: int = 64) -> AttentionPlan:
-    """Cuts the step's query rows into tiles: 16 rows for segments of at most 16 rows,
-    ``rows_big`` rows for longer ones; where there are too few tiles to fill the GPU, a
-    tile's key range is cut into pieces whose partial results are merged."""
+    """Cuts the step's query rows into tiles of 16 rows.  A segment of at most 16 rows
+    (decode tokens) gives one-tile items; a longer one gives items of ``rows_big / 16``
+    tiles that share the keys a wave loads.  Where there are too few items to fill the
+    GPU, an item's key range is cut into pieces whose partial results are merged."""
     rows_of_seg = [int(q) * group_size for q in seg_q_len]
-    small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: r <= ROWS_PER_ITEM or rows_big <= ROWS_PER_ITEM)
-    big = _tiles(seg_q_len, seg_kv_len, group_size, window, rows_big, lambda r: r > ROWS_PER_ITEM and rows_big > ROWS_PER_ITEM)
-    n_tiles = len(small[0]) + len(big[0])
-    if n_tiles * n_kv_heads * 2 >= TARGET_WAVES or n_tiles == 0:
-        chunk = 1 << 30  # enough tiles to fill the GPU: nothing is cut
+    per_item = max(1, rows_big // ROWS_PER_ITEM)
+    small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: r <= ROWS_PER_ITEM or per_item == 1)
+    big = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: r > ROWS_PER_ITEM and per_item > 1)
+    more = None
+    if len(big[0]):
+        *big, more = _group_tiles(*big, per_item, zigzag=window <= 0)
+    n_items = len(small[0]) + len(big[0])
+    if n_items * n_kv_heads * 2 >= TARGET_WAVES or n_items == 0:
+        chunk = 1 << 30  # enough items to fill the GPU: nothing is cut
     else:
         total = int((small[3] - small[2]).sum() + (big[3] - big[2]).sum()) * n_kv_heads
         chunk = -(-total // TARGET_WAVES)
         chunk = max(MIN_SPLIT_KEYS, -(-chunk // KEYS_PER_BLOCK) * KEYS_PER_BLOCK)
     items, merges_s, slot = _cut(*small, chunk, 1, 0, rows_of_seg)
-    big_items, merges_b, slot = _cut(*big, chunk, rows_big // ROWS_PER_ITEM, slot, rows_of_seg)
+    big_items, merges_b, slot = _cut(*big, chunk, per_item, slot, rows_of_seg, more)
     merges = np.concatenate((merges_s, merges_b)) if len(merges_s) or len(merges_b) else np.zeros((0, 8), np.int32)
     return AttentionPlan(items, big_items, merges, slot, rows_big)
 

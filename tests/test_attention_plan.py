@@ -5,28 +5,37 @@ from halite_amd.kernels.attention import plan_items
 
 
 def check_plan(plan, q_len, kv_len, group, window):
-    """Every (row tile, key) pair is covered exactly once; pieces meet on block edges;
-    a cut tile has one merge entry per 16 rows whose partial slots are its own."""
-    seen = {}
-    for rows_per_tile, arr in ((16, plan.items), (plan.rows_big, plan.big_items)):
-        for seg, rho0, b, e, partial, *_ in arr.tolist():
+    """Every 16-row tile belongs to exactly one item group; the pieces of a group are
+    contiguous, meet on block edges and cover every key that any of its tiles may see;
+    a cut group has one merge entry per tile whose partial slots are its own."""
+    per_item = max(1, plan.rows_big // 16)
+    groups = {}
+    for arr, is_big in ((plan.items, False), (plan.big_items, True)):
+        for seg, rho0, b, e, partial, *more in arr.tolist():
             rows = q_len[seg] * group
-            assert (rows <= 16 or plan.rows_big == 16) == (rows_per_tile == 16 and arr is plan.items)
-            assert 0 <= b < e <= kv_len[seg] and rho0 % rows_per_tile == 0 and rho0 < rows
-            seen.setdefault((seg, rho0, rows_per_tile), []).append((b, e, partial))
+            assert (rows > 16 and per_item > 1) == is_big
+            assert 0 <= b < e <= kv_len[seg]
+            tiles = tuple([rho0] + [m for m in more[: per_item - 1] if m >= 0]) if is_big else (rho0,)
+            if not is_big:
+                assert more == [-1, -1, -1]
+            assert all(t % 16 == 0 and 0 <= t < rows for t in tiles)
+            groups.setdefault((seg, tiles), []).append((b, e, partial))
     for s in range(len(q_len)):
         rows = q_len[s] * group
-        per = 16 if rows <= 16 or plan.rows_big == 16 else plan.rows_big
-        assert sorted(r for (seg, r, _) in seen if seg == s) == list(range(0, rows, per))
+        tiles = sorted(t for (seg, ts) in groups for t in ts if seg == s)
+        assert tiles == list(range(0, rows, 16))
     used_slots = set()
     n_merges = 0
-    for (seg, rho0, per), pieces in seen.items():
+    for (seg, tiles), pieces in groups.items():
         rows = q_len[seg] * group
         pos0 = kv_len[seg] - q_len[seg]
-        first_q = rho0 // group
-        last_q = min(rows - 1, rho0 + per - 1) // group
-        lo = max(0, pos0 + first_q - window + 1) if window else 0
-        hi = pos0 + last_q + 1
+        lo = hi = None
+        for t in tiles:
+            first_q, last_q = t // group, min(rows - 1, t + 15) // group
+            t_lo = max(0, pos0 + first_q - window + 1) if window else 0
+            t_hi = pos0 + last_q + 1
+            lo = t_lo if lo is None else min(lo, t_lo)
+            hi = t_hi if hi is None else max(hi, t_hi)
         pieces.sort()
         assert pieces[0][0] == lo and pieces[-1][1] == hi
         for (b0, e0, _), (b1, e1, _) in zip(pieces, pieces[1:]):
@@ -34,13 +43,12 @@ def check_plan(plan, q_len, kv_len, group, window):
         if len(pieces) == 1:
             assert pieces[0][2] == -1
             continue
-        stride = per // 16
+        stride = per_item if len(tiles) > 1 or rows > 16 and per_item > 1 else 1
         slots = [p for _, _, p in pieces]
         assert slots == list(range(slots[0], slots[0] + stride * len(slots), stride))
-        sub_tiles = min(stride, -(-(rows - rho0) // 16))
-        for sub in range(sub_tiles):
-            match = [m for m in plan.merges.tolist() if m[0] == seg and m[1] == rho0 + 16 * sub]
-            assert match == [[seg, rho0 + 16 * sub, slots[0] + sub, len(slots), stride, 0, 0, 0]]
+        for sub, t in enumerate(tiles):
+            match = [m for m in plan.merges.tolist() if m[0] == seg and m[1] == t]
+            assert match == [[seg, t, slots[0] + sub, len(slots), stride, 0, 0, 0]]
             n_merges += 1
         for s0 in slots:
             for sub in range(stride):
@@ -50,7 +58,7 @@ def check_plan(plan, q_len, kv_len, group, window):
     assert not used_slots or max(used_slots) < plan.n_partials
 
 
-@pytest.mark.parametrize("rows_big", [64, 16])
+@pytest.mark.parametrize("rows_big", [64, 32, 16])
 @pytest.mark.parametrize("window", [0, 7, 100])
 @pytest.mark.parametrize("group", [1, 3, 4, 20])
 def test_every_row_and_key_is_covered_once(group, window, rows_big):
@@ -65,6 +73,10 @@ def test_long_decode_is_split_and_prefill_is_not():
     assert plan.n_merges == 8 and plan.n_items > 8 * 4 and plan.n_big == 0
     plan = plan_items(np.array([2048]), np.array([2048]), 4, 8, 0)
     assert plan.n_merges == 0 and plan.n_big == 2048 * 4 // 64 and plan.n_items == 0
+    # zigzag: an early tile rides with a late one, every item reaches far
+    pair = plan_items(np.array([2048]), np.array([2048]), 4, 8, 0, 32)
+    assert pair.n_big == 256 and (pair.big_items[:, 3] > 1024).all()
+    assert sorted(pair.big_items[:, 1].tolist() + pair.big_items[:, 5].tolist()) == list(range(0, 8192, 16))
     # a short portion of a prompt against a long context: few big tiles, so they are cut
     q_len, kv_len = np.array([64]), np.array([20000])
     plan = plan_items(q_len, kv_len, 4, 8, 0)
