@@ -249,10 +249,43 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   }
 }
 
+// four elements per access; F is a multiple of 4
+template <typename T>
+__global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_tokens,
+                                    int F) {
+  const int f4 = F / 4;
+  const size_t n = (size_t)n_tokens * f4;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    const size_t t = i / f4, f = (i % f4) * 4;
+    float g[4], u[4], y[4];
+    load4(gu + t * 2 * F + f, g);
+    load4(gu + t * 2 * F + F + f, u);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) y[e] = u[e] * (g[e] / (1.0f + expf(-g[e])));
+    store4(out + t * F + f, y);
+  }
+}
+
 extern "C" int hal_silu_mul(const void* gu, void* out, int dtype, int n_tokens, int F,
                             hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && F > 0, "hal_silu_mul: bad sizes T=%d F=%d", n_tokens, F);
   if (n_tokens == 0) return 0;
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_silu_mul: unknown dtype %d", dtype);
+  if (F % 4 == 0) {
+    const size_t n4 = (size_t)n_tokens * (F / 4);
+    const size_t want4 = (n4 + 255) / 256;
+    const int blocks4 = (int)(want4 < 16384 ? want4 : 16384);
+    if (dtype == HAL_F32)
+      hipLaunchKernelGGL(silu_mul_vec_kernel<float>, dim3(blocks4), dim3(256), 0, stream,
+                         (const float*)gu, (float*)out, n_tokens, F);
+    else
+      hipLaunchKernelGGL(silu_mul_vec_kernel<bf16_t>, dim3(blocks4), dim3(256), 0, stream,
+                         (const bf16_t*)gu, (bf16_t*)out, n_tokens, F);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   const size_t n = (size_t)n_tokens * F;
   const int threads = 256;
   const size_t want = (n + threads - 1) / threads;

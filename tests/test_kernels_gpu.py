@@ -76,6 +76,9 @@ def test_silu_mul_and_residual_add(gpu, dtype):
     gu = rnd(11, 2 * 352, seed=6, scale=3.0).to(dt)
     g, u = gu[:, :352].float(), gu[:, 352:].float()
     close(ops.silu_mul(gu.to(gpu)), u * g * torch.sigmoid(g), 1e-6 if dtype == "float32" else 5e-3)
+    odd = rnd(7, 2 * 353, seed=16, scale=3.0).to(dt)  # a width that is no multiple of 4
+    g, u = odd[:, :353].float(), odd[:, 353:].float()
+    close(ops.silu_mul(odd.to(gpu)), u * g * torch.sigmoid(g), 1e-6 if dtype == "float32" else 5e-3)
     h, d = rnd(5, 77, seed=7), rnd(5, 77, seed=8).to(dt)
     close(ops.residual_add(h.to(gpu).clone(), d.to(gpu)), h + d.float(), 1e-7)
 
