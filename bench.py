@@ -79,6 +79,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
+    ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (for profiles)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -98,6 +99,8 @@ def main() -> int:
     context = args.context or full.max_position_embeddings
     elt = 2 if args.dtype == "bfloat16" else 4
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    if args.prefill_only:
+        batches, context = [1], 4096
     pool_tokens = max(batches) * (context + 64) + 4096
     runner = ModelRunner.from_random(
         cfg, seed=0,
@@ -148,6 +151,32 @@ def main() -> int:
         for s in slots:
             runner.free(s)
         return dt, kv_tokens
+
+    def prefill_run(T=2048):
+        ids = torch.randint(0, cfg.vocab_size, (T,), generator=gen).numpy().astype(np.int32)
+        times = []
+        for i in range(4):
+            s = runner.admit()
+            sync()
+            t0 = time.perf_counter()
+            logits = runner.step([Segment(s, 0, ids, [T - 1])])
+            tok, _ = sampler.forward(logits, [greedy], [0], [0])
+            tok.tolist()
+            sync()
+            times.append(time.perf_counter() - t0)
+            runner.free(s)
+        t = min(times[1:])
+        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+        return {
+            "value": round(T / t, 1),
+            "tokens": T,
+            "ms": round(t * 1e3, 3),
+            "frac": round(prefill_flops(cfg, n_layers, T) / t / peak, 4),
+        }
+
+    if args.prefill_only:
+        print(json.dumps({"metric": "prefill tokens per second", "layers": n_layers, "prefill": prefill_run()}), flush=True)
+        return 0
 
     # -- the headline: batch 8 -------------------------------------------------------
     results = {}
@@ -202,28 +231,7 @@ def main() -> int:
 
     if not args.no_points:
         record["points"] = {f"decode_b{b}": round(results[b][0], 2) for b in (1, 64) if b in results}
-        # -- prefill of one 2,048-token prompt ----------------------------------------
-        T = 2048
-        ids = torch.randint(0, cfg.vocab_size, (T,), generator=gen).numpy().astype(np.int32)
-        times = []
-        for i in range(4):
-            s = runner.admit()
-            sync()
-            t0 = time.perf_counter()
-            logits = runner.step([Segment(s, 0, ids, [T - 1])])
-            tok, _ = sampler.forward(logits, [greedy], [0], [0])
-            tok.tolist()
-            sync()
-            times.append(time.perf_counter() - t0)
-            runner.free(s)
-        t = min(times[1:])
-        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
-        record["prefill"] = {
-            "value": round(T / t, 1),
-            "tokens": T,
-            "ms": round(t * 1e3, 3),
-            "frac": round(prefill_flops(cfg, n_layers, T) / t / peak, 4),
-        }
+        record["prefill"] = prefill_run()
     print(json.dumps(record), flush=True)
     return 0
 

@@ -362,17 +362,28 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
         l_all += w * li;
       }
       const int cnt = n - i0 < HAL_WAVE ? n - i0 : HAL_WAVE;
-#pragma unroll 8
-      for (int i = 0; i < cnt; ++i) {
-        const float wi = __shfl(w, i, HAL_WAVE);
-        const float* po = part_o + (((size_t)(first + (i0 + i) * stride) * K + g) * 16 + row) * D;
+      // four partials at a time: their loads are issued together
+      for (int i = 0; i < cnt; i += 4) {
+        float wi[4];
+        const float* po[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int iu = i + u < cnt ? i + u : cnt - 1;
+          wi[u] = i + u < cnt ? __shfl(w, iu, HAL_WAVE) : 0.f;
+          po[u] = part_o + (((size_t)(first + (i0 + iu) * stride) * K + g) * 16 + row) * D;
+        }
 #pragma unroll
         for (int c = 0; c < D / 128 + 1; ++c) {
           const int d = c * 128 + lane * 2;
           if (d < D) {
-            const float2 v = *(const float2*)(po + d);
-            acc[c][0] += wi * v.x;
-            acc[c][1] += wi * v.y;
+            float2 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = *(const float2*)(po[u] + d);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              acc[c][0] += wi[u] * v[u].x;
+              acc[c][1] += wi[u] * v[u].y;
+            }
           }
         }
       }

@@ -20,7 +20,7 @@ from . import library, ops
 
 ROWS_PER_ITEM = 16
 KEYS_PER_BLOCK = 32
-MIN_SPLIT_KEYS = 256
+MIN_SPLIT_KEYS = 128
 TARGET_WAVES = 2048
 
 
