@@ -58,8 +58,9 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // a prompt with a late one gives every wave the same amount of causal work.  A tile
 // skips the blocks of keys that lie wholly outside its own range.  Row tile rt of an
 // item writes partial slot `first partial slot + rt`.
-template <int RT, bool POW2>
-__global__ void __launch_bounds__(256)
+#define N_XCD 8
+template <int RT, bool POW2, bool PAGE32>
+__global__ void __launch_bounds__(256, 2)
 attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
                       int out_row_stride, const int* __restrict__ items,
                       const int* __restrict__ n_items_ptr, const int* __restrict__ seg_q_start,
@@ -69,13 +70,30 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                       float* __restrict__ part_o, float* __restrict__ part_ml, int H, int K,
                       int page_size, int page_shift, float scale_log2e, int window) {
   const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
-  const int item = blockIdx.x * (blockDim.x / HAL_WAVE) + wave;
+  // Workgroups go to the eight XCDs in turn (linear id modulo 8) and each XCD has an L2 of
+  // its own: the ids are renumbered so that an XCD gets a contiguous run of (kv head, item
+  // block) pairs, i.e. the tiles that read one head's keys meet in one L2.
+  int bx = blockIdx.x, g = blockIdx.y;
+  {
+    const int nx = gridDim.x, n_blocks = nx * gridDim.y;
+    if (n_blocks % N_XCD == 0) {
+      const int linear = bx + nx * g;
+      const int v = (linear % N_XCD) * (n_blocks / N_XCD) + linear / N_XCD;
+      g = v / nx;
+      bx = v % nx;
+    }
+  }
+  const int item = bx * (blockDim.x / HAL_WAVE) + wave;
   if (item >= *n_items_ptr) return;
-  const int* it = items + (size_t)item * ITEM_INTS;
-  const int seg = it[0], rho0 = it[1], kv_begin = it[2], kv_end = it[3], partial = it[4];
-  const int g = blockIdx.y;
+  // everything that describes the item is the same for the whole wave: kept in scalar
+  // registers, so that loop control, block-level masks and page lookups cost no vector work
+  auto uniform = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
+  const int* it = items + (size_t)uniform(item) * ITEM_INTS;
+  const int seg = uniform(it[0]), rho0 = uniform(it[1]), kv_begin = uniform(it[2]),
+            kv_end = uniform(it[3]), partial = uniform(it[4]);
   const int G = H / K;
-  const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], kv_len = seg_kv_len[seg];
+  const int q_start = uniform(seg_q_start[seg]), q_len = uniform(seg_q_len[seg]),
+            kv_len = uniform(seg_kv_len[seg]);
   const int pos0 = kv_len - q_len;  // position of the segment's first token
   const int* bt = block_table + (size_t)seg * bt_stride;
 
@@ -88,7 +106,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   float m[RT], l[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int tile0 = rt == 0 ? rho0 : it[4 + rt];
+    const int tile0 = rt == 0 ? rho0 : uniform(it[4 + rt]);
     const int rho = tile0 + col;
     row_ok[rt] = tile0 >= 0 && rho < q_len * G;
     qi[rt] = row_ok[rt] ? rho / G : 0;
@@ -116,7 +134,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   int p_first[RT], p_last[RT], lo_first[RT], lo_last[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int r_first = rt == 0 ? rho0 : it[4 + rt];
+    const int r_first = rt == 0 ? rho0 : uniform(it[4 + rt]);
     int r_last = r_first + 15;
     if (r_last > q_len * G - 1) r_last = q_len * G - 1;
     if (r_last < r_first) r_last = r_first;
@@ -128,81 +146,122 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 
   // This lane's key of tile t in the block of 32 keys at j0: row `col` of tile t is
   // key j0 + (col/4)*8 + t*4 + col%4; its eight keys for the values are j0 + quad*8 .. +8.
-  // Keys outside [kv_begin, last_key] are clamped for the address only; their scores
-  // are masked and their values cleared.  Page numbers are looked up one block ahead
-  // of the loads that need them, so that no load waits for a table entry.
+  //
+  // PAGE32 (pages of a power of two, at least 32 tokens): a block of 32 keys lies in one
+  // page, so the page number and the block's base addresses are the same for the whole
+  // wave (scalar registers) and a lane adds constants of its own.  Keys of the page that
+  // are outside the item's range or not written yet are loaded like the others (the page
+  // is held), their scores are masked and their values cleared.
+  //
+  // Otherwise every lane looks its keys' pages up itself; keys outside
+  // [kv_begin, last_key] are clamped for the address only, and the page numbers are
+  // fetched one block ahead of the loads that need them.
+  const int koff0 = ((col / 4) * 8 + (col % 4)) * D + quad * 8;  // tile 1 is 4 keys on
+  const int voff = col * page_size + quad * 8;
   auto key_index = [&](int j0, int t) {
     const int j = j0 + (col / 4) * 8 + t * 4 + (col % 4);
     return j < kv_begin ? kv_begin : (j > last_key ? last_key : j);
   };
   auto value_index = [&](int j0) {
     int jv = j0 + quad * 8;
-    if (jv < (kv_begin & ~7)) jv = kv_begin & ~7;
-    if (jv > (last_key & ~7)) jv = last_key & ~7;
+    if constexpr (!PAGE32) {
+      if (jv < (kv_begin & ~7)) jv = kv_begin & ~7;
+      if (jv > (last_key & ~7)) jv = last_key & ~7;
+    }
     return jv;
   };
-  auto load_keys = [&](int j0, const int (&pages)[2], bf16x8 (&kf)[2][KT]) {
+  auto load_keys = [&](int j0, int page, bf16x8 (&kf)[2][KT]) {
+    if constexpr (PAGE32) {
+      const bf16_t* base =
+          k_pages + (((size_t)page * K + g) * page_size + (j0 & (page_size - 1))) * D;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int j = key_index(j0, t);
-      const bf16_t* kp = k_pages + (((size_t)pages[t] * K + g) * page_size + slot_of(j)) * D;
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int ks = 0; ks < KT; ++ks) {
-        const int d0 = ks * 32 + quad * 8;
-        if constexpr (D % 32 == 0) kf[t][ks] = ld16(kp + d0);
-        else kf[t][ks] = d0 < D ? ld16(kp + d0) : zero8();
+        for (int ks = 0; ks < KT; ++ks) {
+          const int d0 = ks * 32 + quad * 8;
+          if constexpr (D % 32 == 0) kf[t][ks] = ld16(base + koff0 + t * 4 * D + ks * 32);
+          else kf[t][ks] = d0 < D ? ld16(base + koff0 + t * 4 * D + ks * 32) : zero8();
+        }
+    } else {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int j = key_index(j0, t);
+        const long long page = bt[page_of(j)];
+        const bf16_t* kp = k_pages + (((size_t)page * K + g) * page_size + slot_of(j)) * D;
+#pragma unroll
+        for (int ks = 0; ks < KT; ++ks) {
+          const int d0 = ks * 32 + quad * 8;
+          if constexpr (D % 32 == 0) kf[t][ks] = ld16(kp + d0);
+          else kf[t][ks] = d0 < D ? ld16(kp + d0) : zero8();
+        }
       }
     }
   };
+  auto load_values = [&](int j0, int page, bf16x8 (&vf)[DT]) {
+    // lane loads V^T[dim dt*16 + col][keys jv .. jv+8]
+    if constexpr (PAGE32) {
+      const bf16_t* base =
+          v_pages + ((size_t)page * K + g) * D * page_size + (j0 & (page_size - 1));
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vf[dt] = ld16(base + voff + (size_t)dt * 16 * page_size);
+    } else {
+      const int jv = value_index(j0);
+      const long long page = bt[page_of(jv)];
+      const bf16_t* vp = v_pages + ((size_t)page * K + g) * D * page_size + slot_of(jv);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vf[dt] = ld16(vp + (size_t)(dt * 16 + col) * page_size);
+    }
+  };
 
+  // This block's values and the next block's keys (a second buffer) are asked for at
+  // the block's start; deeper or shallower schedules measured the same or worse.
   const int j_first = kv_begin & ~31;
-  bf16x8 kcur[2][KT], knext[2][KT];
-  int kpage[2], vpage;  // pages of the NEXT key block and of THIS value block
-  if (j_first < kv_end) {
-    kpage[0] = bt[page_of(key_index(j_first, 0))];
-    kpage[1] = bt[page_of(key_index(j_first, 1))];
-    vpage = bt[page_of(value_index(j_first))];
-    load_keys(j_first, kpage, kcur);
-    kpage[0] = bt[page_of(key_index(j_first + 32, 0))];
-    kpage[1] = bt[page_of(key_index(j_first + 32, 1))];
-  }
+  // PAGE32: the page numbers of this block, the next and the one after, looked up (scalar
+  // loads) two blocks before the loads that need them
+  auto page_at = [&](int j0) {
+    if constexpr (PAGE32) return uniform(bt[(j0 < kv_end ? j0 : j_first) >> page_shift]);
+    else return 0;
+  };
+  int page_cur = page_at(j_first), page_next = page_at(j_first + 32);
+  bf16x8 kcur[2][KT], vf[DT];
+  bf16x8 knext[2][KT];
+  if (j_first < kv_end) load_keys(j_first, page_cur, kcur);
 
   for (int j0 = j_first; j0 < kv_end; j0 += 32) {
-    // ---- issue this block's value loads and the next block's key loads first --------
-    // lane loads V^T[dim dt*16 + col][keys jv .. jv+8]
     const int jv = value_index(j0);
     const bool tail = j0 + 32 > kv_len;  // some of the 32 keys are not written yet
-    const bf16_t* vp = v_pages + ((size_t)vpage * K + g) * D * page_size + slot_of(jv);
-    bf16x8 vf[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) vf[dt] = ld16(vp + (size_t)(dt * 16 + col) * page_size);
-    if (j0 + 32 < kv_end) {
-      load_keys(j0 + 32, kpage, knext);
-      vpage = bt[page_of(value_index(j0 + 32))];
-      kpage[0] = bt[page_of(key_index(j0 + 64, 0))];
-      kpage[1] = bt[page_of(key_index(j0 + 64, 1))];
-    }
+    const bool more = j0 + 32 < kv_end;
+    const int page_after = page_at(j0 + 64);
+    load_values(j0, page_cur, vf);
+    if (more) load_keys(j0 + 32, page_next, knext);
 
-    bf16x8 pb[RT];
-    float alpha[RT];
+    // ---- S^T = K Q^T for 32 keys (two tiles of 16), all row tiles ------------------
+    f32x4 s[RT][2];
     bool active[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       // a block wholly after the tile's last row or before its first row's window
       // does nothing for this tile
       active[rt] = j0 <= p_last[rt] && j0 + 31 >= lo_first[rt];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        s[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (active[rt]) {
+#pragma unroll
+          for (int ks = 0; ks < KT; ++ks)
+            s[rt][t] =
+                __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][ks], bq[rt][ks], s[rt][t], 0, 0, 0);
+        }
+      }
+    }
+
+    bf16x8 pb[RT];
+    float alpha[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
       alpha[rt] = 1.f;
       pb[rt] = zero8();
       if (!active[rt]) continue;
-      // ---- S^T = K Q^T for 32 keys (two tiles of 16) ----------------------------
-      f32x4 s[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KT; ++ks)
-          s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][ks], bq[rt][ks], s[t], 0, 0, 0);
-      }
       // ---- mask and online softmax: this lane has keys j0 + quad*8 + e, e = 0..7 --
       float sv[8];
       float m_tile = -INFINITY;
@@ -211,7 +270,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       if (full) {  // every key of the block is visible to every row of the tile
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          sv[e] = s[e / 4][e % 4] * scale_log2e;
+          sv[e] = s[rt][e / 4][e % 4] * scale_log2e;
           m_tile = fmaxf(m_tile, sv[e]);
         }
       } else {
@@ -220,7 +279,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
           const int j = j0 + quad * 8 + e;
           const bool ok =
               row_ok[rt] && j >= kv_begin && j < kv_end && j >= lo_row[rt] && j <= p_row[rt];
-          sv[e] = ok ? s[e / 4][e % 4] * scale_log2e : -INFINITY;
+          sv[e] = ok ? s[rt][e / 4][e % 4] * scale_log2e : -INFINITY;
           m_tile = fmaxf(m_tile, sv[e]);
         }
       }
@@ -287,6 +346,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int ks = 0; ks < KT; ++ks) kcur[t][ks] = knext[t][ks];
+    page_cur = page_next;
+    page_next = page_after;
   }
 
 #pragma unroll
@@ -441,26 +502,22 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   if ((page_size & (page_size - 1)) == 0)
     for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
   const int waves = 4;
-  if (max_items > 0) {
-    dim3 grid((max_items + waves - 1) / waves, K);
-    hipLaunchKernelGGL((page_shift >= 0 ? attention_mfma_kernel<1, true> : attention_mfma_kernel<1, false>),
-                       grid, dim3(waves * HAL_WAVE), 0, stream,
-                       (const bf16_t*)q, q_row_stride, (bf16_t*)out, out_row_stride, items,
-                       counts, seg_q_start, seg_q_len, seg_kv_len, block_table, bt_stride,
-                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, part_o, part_ml, H, K,
-                       page_size, page_shift, scale_log2e, window);
-    HAL_LAUNCH_CHECK();
+#define LAUNCH_ATTENTION(RT_, LIST, MAX, COUNT)                                                   \
+  {                                                                                               \
+    dim3 grid(((MAX) + waves - 1) / waves, K);                                                    \
+    hipLaunchKernelGGL((page_shift >= 5   ? attention_mfma_kernel<RT_, true, true>                \
+                        : page_shift >= 0 ? attention_mfma_kernel<RT_, true, false>               \
+                                          : attention_mfma_kernel<RT_, false, false>),            \
+                       grid, dim3(waves * HAL_WAVE), 0, stream, (const bf16_t*)q, q_row_stride,   \
+                       (bf16_t*)out, out_row_stride, LIST, COUNT, seg_q_start, seg_q_len,         \
+                       seg_kv_len, block_table, bt_stride, (const bf16_t*)k_pages,                \
+                       (const bf16_t*)v_pages, part_o, part_ml, H, K, page_size, page_shift,      \
+                       scale_log2e, window);                                                      \
+    HAL_LAUNCH_CHECK();                                                                           \
   }
-  if (max_big > 0) {
-    dim3 grid((max_big + waves - 1) / waves, K);
-    hipLaunchKernelGGL((page_shift >= 0 ? attention_mfma_kernel<RT_BIG, true> : attention_mfma_kernel<RT_BIG, false>),
-                       grid, dim3(waves * HAL_WAVE), 0, stream,
-                       (const bf16_t*)q, q_row_stride, (bf16_t*)out, out_row_stride, big_items,
-                       counts + 1, seg_q_start, seg_q_len, seg_kv_len, block_table, bt_stride,
-                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, part_o, part_ml, H, K,
-                       page_size, page_shift, scale_log2e, window);
-    HAL_LAUNCH_CHECK();
-  }
+  if (max_items > 0) LAUNCH_ATTENTION(1, items, max_items, counts)
+  if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, big_items, max_big, counts + 1)
+#undef LAUNCH_ATTENTION
   if (max_merges > 0) {
     hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K), dim3(256), 0, stream,
                        (bf16_t*)out, out_row_stride, merges, counts + 2, seg_q_start, seg_q_len,
