@@ -15,7 +15,7 @@ import numpy as np
 import torch
 
 from ..parts.base import PagedKVNeed, StateNeed
-from .pages import CacheGroup, LayerPages, NoSpace, PagePool
+from .pages import CacheGroup, LayerPages, NoSpace, PagePool, tiled_layout
 from .slots import SlotAllocator, StateStore
 
 
@@ -69,7 +69,7 @@ class CacheManager:
                     vp = g.storage[i, 1].view(num_pages, k, d, page_size)
                 else:
                     kp = vp = None
-                self._pages[run] = LayerPages(g.group_id, kp, vp)
+                self._pages[run] = LayerPages(g.group_id, kp, vp, tiled_layout(dtype, d, page_size))
         for run, owner in self.borrowed.items():
             self._pages[run] = self._pages[owner]
         self.slots = SlotAllocator(n_slots)

@@ -62,14 +62,33 @@ class PagePool:
         return {p for p, h in enumerate(self._held) if h}
 
 
+def tiled_layout(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
+    """Whether pages of this shape are kept in the order in which the matrix-core
+    attention kernel loads them (contiguous KB per MFMA operand) instead of row by row:
+    bf16, heads of a multiple of 32 (up to 256), pages of a power of two of at least 32
+    tokens.  The kernel that appends and the kernel that reads are told by
+    ``LayerPages.tiled``."""
+    return (
+        dtype == torch.bfloat16
+        and head_dim % 32 == 0
+        and head_dim <= 256
+        and page_size >= 32
+        and page_size & (page_size - 1) == 0
+    )
+
+
 @dataclass
 class LayerPages:
     """The device pages of one run: keys ``[pages, K, page_size, D]`` and values,
-    transposed, ``[pages, K, D, page_size]``."""
+    transposed, ``[pages, K, D, page_size]``.  With ``tiled`` the bytes of one
+    (page, kv head) are the same in number but lie in blocks of 32 tokens, keys as
+    ``[block][16-key tile][32-dim step][dim quad][key][8 dims]`` and values as
+    ``[block][16-dim tile][8-key group][dim][8 keys]``."""
 
     group_id: int
     k: torch.Tensor | None
     v: torch.Tensor | None
+    tiled: bool = False
 
 
 @dataclass

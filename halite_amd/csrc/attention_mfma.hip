@@ -59,7 +59,8 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // skips the blocks of keys that lie wholly outside its own range.  Row tile rt of an
 // item writes partial slot `first partial slot + rt`.
 #define N_XCD 8
-template <int RT, bool POW2, bool PAGE32>
+#define WAVES 4  // per workgroup
+template <int RT, bool POW2, bool PAGE32, bool SHARED, bool TILED>
 __global__ void __launch_bounds__(256, 2)
 attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
                       int out_row_stride, const int* __restrict__ items,
@@ -83,14 +84,36 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       bx = v % nx;
     }
   }
-  const int item = bx * (blockDim.x / HAL_WAVE) + wave;
-  if (item >= *n_items_ptr) return;
   // everything that describes the item is the same for the whole wave: kept in scalar
   // registers, so that loop control, block-level masks and page lookups cost no vector work
   auto uniform = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
-  const int* it = items + (size_t)uniform(item) * ITEM_INTS;
-  const int seg = uniform(it[0]), rho0 = uniform(it[1]), kv_begin = uniform(it[2]),
-            kv_end = uniform(it[3]), partial = uniform(it[4]);
+  const int n_items = *n_items_ptr;
+  const int item = uniform(bx * WAVES + wave);
+  // SHARED: the four waves of a workgroup have items of one segment (the host lists them
+  // so) and walk the union of their key ranges together; the keys and values of a block
+  // are loaded once, by all four, into LDS.  A wave without an item of its own (the list
+  // ends, or the host padded the group) still loads and waits at the barriers.
+  if (SHARED ? bx * WAVES >= n_items : item >= n_items) return;
+  const bool have_item = item < n_items;
+  const int* it = items + (size_t)(have_item ? item : bx * WAVES) * ITEM_INTS;
+  const int seg = uniform(it[0]);
+  const int rho0 = have_item ? uniform(it[1]) : -1;
+  const int kv_begin = have_item ? uniform(it[2]) : 0, kv_end = have_item ? uniform(it[3]) : 0;
+  const int partial = have_item ? uniform(it[4]) : -1;
+  int walk_begin = kv_begin, walk_end = kv_end;  // the keys this wave walks through
+  if constexpr (SHARED) {
+    walk_begin = 0x7fffffff, walk_end = 0;
+    for (int w = 0; w < WAVES; ++w) {
+      if (bx * WAVES + w >= n_items) break;
+      const int* other = items + (size_t)(bx * WAVES + w) * ITEM_INTS;
+      const int b = uniform(other[2]), e = uniform(other[3]);
+      if (b < e) {
+        walk_begin = b < walk_begin ? b : walk_begin;
+        walk_end = e > walk_end ? e : walk_end;
+      }
+    }
+    if (walk_begin >= walk_end) return;  // the same for all four waves
+  }
   const int G = H / K;
   const int q_start = uniform(seg_q_start[seg]), q_len = uniform(seg_q_len[seg]),
             kv_len = uniform(seg_kv_len[seg]);
@@ -106,7 +129,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   float m[RT], l[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int tile0 = rt == 0 ? rho0 : uniform(it[4 + rt]);
+    const int tile0 = rt == 0 ? rho0 : (have_item ? uniform(it[4 + rt]) : -1);
     const int rho = tile0 + col;
     row_ok[rt] = tile0 >= 0 && rho < q_len * G;
     qi[rt] = row_ok[rt] ? rho / G : 0;
@@ -134,7 +157,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   int p_first[RT], p_last[RT], lo_first[RT], lo_last[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int r_first = rt == 0 ? rho0 : uniform(it[4 + rt]);
+    const int r_first = rt == 0 ? rho0 : (have_item ? uniform(it[4 + rt]) : -1);
     int r_last = r_first + 15;
     if (r_last > q_len * G - 1) r_last = q_len * G - 1;
     if (r_last < r_first) r_last = r_first;
@@ -160,80 +183,135 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   const int voff = col * page_size + quad * 8;
   auto key_index = [&](int j0, int t) {
     const int j = j0 + (col / 4) * 8 + t * 4 + (col % 4);
-    return j < kv_begin ? kv_begin : (j > last_key ? last_key : j);
+    return j < walk_begin ? walk_begin : (j > last_key ? last_key : j);
   };
   auto value_index = [&](int j0) {
     int jv = j0 + quad * 8;
     if constexpr (!PAGE32) {
-      if (jv < (kv_begin & ~7)) jv = kv_begin & ~7;
+      if (jv < (walk_begin & ~7)) jv = walk_begin & ~7;
       if (jv > (last_key & ~7)) jv = last_key & ~7;
     }
     return jv;
   };
-  auto load_keys = [&](int j0, int page, bf16x8 (&kf)[2][KT]) {
-    if constexpr (PAGE32) {
+  // One fragment is what one MFMA takes from the block of 32 keys, 16 bytes a lane:
+  // (t, ks) of the keys, dt of the values.
+  auto load_key_frag = [&](int j0, int page, int t, int ks) -> bf16x8 {
+    const int d0 = ks * 32 + quad * 8;
+    if (D % 32 != 0 && d0 >= D) return zero8();
+    if constexpr (TILED) {  // the fragment is one contiguous KB
       const bf16_t* base =
           k_pages + (((size_t)page * K + g) * page_size + (j0 & (page_size - 1))) * D;
+      return ld16(base + (t * KT + ks) * 512 + lane * 8);
+    } else if constexpr (PAGE32) {
+      const bf16_t* base =
+          k_pages + (((size_t)page * K + g) * page_size + (j0 & (page_size - 1))) * D;
+      return ld16(base + koff0 + t * 4 * D + ks * 32);
+    } else {
+      const int j = key_index(j0, t);
+      const long long pg = bt[page_of(j)];
+      return ld16(k_pages + (((size_t)pg * K + g) * page_size + slot_of(j)) * D + d0);
+    }
+  };
+  auto load_value_frag = [&](int j0, int page, int dt) -> bf16x8 {
+    // lane loads V^T[dim dt*16 + col][keys jv .. jv+8]
+    if constexpr (TILED) {
+      const bf16_t* base =
+          v_pages + (((size_t)page * K + g) * page_size + (j0 & (page_size - 1))) * D;
+      return ld16(base + dt * 512 + lane * 8);
+    } else if constexpr (PAGE32) {
+      const bf16_t* base =
+          v_pages + ((size_t)page * K + g) * D * page_size + (j0 & (page_size - 1));
+      return ld16(base + voff + (size_t)dt * 16 * page_size);
+    } else {
+      const int jv = value_index(j0);
+      const long long pg = bt[page_of(jv)];
+      return ld16(v_pages + ((size_t)pg * K + g) * D * page_size + slot_of(jv) +
+                  (size_t)(dt * 16 + col) * page_size);
+    }
+  };
+  // unwritten slots may hold anything, NaN included, and 0 * NaN must not get in: in the
+  // last block of the request the values of keys past the end are cleared
+  auto clear_unwritten = [&](int j0, bf16x8 v) -> bf16x8 {
+    const int jv = value_index(j0);
+    u32x4 raw = __builtin_bit_cast(u32x4, v);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int ja = jv + 2 * w;
+      raw[w] &= (ja <= last_key ? 0x0000ffffu : 0u) | (ja + 1 <= last_key ? 0xffff0000u : 0u);
+    }
+    return __builtin_bit_cast(bf16x8, raw);
+  };
+
+  const int j_first = walk_begin & ~31;
+  // PAGE32: the page numbers of this block and the next three, looked up (scalar loads)
+  // well before the loads that need them
+  auto page_at = [&](int j0) {
+    if constexpr (PAGE32) return uniform(bt[(j0 < walk_end ? j0 : j_first) >> page_shift]);
+    else return 0;
+  };
+  int page_0 = page_at(j_first), page_1 = page_at(j_first + 32), page_2 = page_at(j_first + 64);
+
+  // Without LDS: this block's values and the next block's keys (a second buffer) are asked
+  // for at the block's start; deeper or shallower schedules measured the same or worse.
+  bf16x8 kcur[2][KT], knext[SHARED ? 1 : 2][SHARED ? 1 : KT], vf[DT];
+  // With LDS: fragment f of a block (keys first, then values) is loaded by wave f % 4 into
+  // registers one block ahead, and written to the other half of the LDS buffer while this
+  // block is worked on; a fragment lies there in lane order, as the MFMA wants it back.
+  constexpr int NF = 2 * KT + DT, FPW = (NF + WAVES - 1) / WAVES;
+  __shared__ u32x4 frag_lds[SHARED ? 2 : 1][SHARED ? NF : 1][HAL_WAVE];
+  bf16x8 staged[SHARED ? FPW : 1];
+  auto fetch = [&](int j0, int page) {
+#pragma unroll
+    for (int i = 0; i < FPW; ++i) {
+      const int f = wave + WAVES * i;
+      if (f < 2 * KT) staged[i] = load_key_frag(j0, page, f / KT, f % KT);
+      else if (f < NF) staged[i] = load_value_frag(j0, page, f - 2 * KT);
+    }
+  };
+  auto stash = [&](int j0, int half) {
+#pragma unroll
+    for (int i = 0; i < FPW; ++i) {
+      const int f = wave + WAVES * i;
+      if (f >= NF) continue;
+      bf16x8 v = staged[i];
+      if (f >= 2 * KT && j0 + 32 > kv_len) v = clear_unwritten(j0, v);
+      frag_lds[half][f][lane] = __builtin_bit_cast(u32x4, v);
+    }
+  };
+  if constexpr (SHARED) {
+    fetch(j_first, page_0);
+    stash(j_first, 0);
+    if (j_first + 32 < walk_end) fetch(j_first + 32, page_1);
+    __syncthreads();
+  } else {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int ks = 0; ks < KT; ++ks) kcur[t][ks] = load_key_frag(j_first, page_0, t, ks);
+  }
+
+  int half = 0;
+  for (int j0 = j_first; j0 < walk_end; j0 += 32) {
+    const bool tail = j0 + 32 > kv_len;  // some of the 32 keys are not written yet
+    const bool more = j0 + 32 < walk_end;
+    const int page_3 = page_at(j0 + 96);
+    if constexpr (!SHARED) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vf[dt] = load_value_frag(j0, page_0, dt);
+      if (more) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int ks = 0; ks < KT; ++ks) knext[t][ks] = load_key_frag(j0 + 32, page_1, t, ks);
+      }
+    }
+    if constexpr (SHARED) {
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int ks = 0; ks < KT; ++ks) {
-          const int d0 = ks * 32 + quad * 8;
-          if constexpr (D % 32 == 0) kf[t][ks] = ld16(base + koff0 + t * 4 * D + ks * 32);
-          else kf[t][ks] = d0 < D ? ld16(base + koff0 + t * 4 * D + ks * 32) : zero8();
-        }
-    } else {
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const int j = key_index(j0, t);
-        const long long page = bt[page_of(j)];
-        const bf16_t* kp = k_pages + (((size_t)page * K + g) * page_size + slot_of(j)) * D;
-#pragma unroll
-        for (int ks = 0; ks < KT; ++ks) {
-          const int d0 = ks * 32 + quad * 8;
-          if constexpr (D % 32 == 0) kf[t][ks] = ld16(kp + d0);
-          else kf[t][ks] = d0 < D ? ld16(kp + d0) : zero8();
-        }
-      }
+        for (int ks = 0; ks < KT; ++ks)
+          kcur[t][ks] = __builtin_bit_cast(bf16x8, frag_lds[half][t * KT + ks][lane]);
     }
-  };
-  auto load_values = [&](int j0, int page, bf16x8 (&vf)[DT]) {
-    // lane loads V^T[dim dt*16 + col][keys jv .. jv+8]
-    if constexpr (PAGE32) {
-      const bf16_t* base =
-          v_pages + ((size_t)page * K + g) * D * page_size + (j0 & (page_size - 1));
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) vf[dt] = ld16(base + voff + (size_t)dt * 16 * page_size);
-    } else {
-      const int jv = value_index(j0);
-      const long long page = bt[page_of(jv)];
-      const bf16_t* vp = v_pages + ((size_t)page * K + g) * D * page_size + slot_of(jv);
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) vf[dt] = ld16(vp + (size_t)(dt * 16 + col) * page_size);
-    }
-  };
-
-  // This block's values and the next block's keys (a second buffer) are asked for at
-  // the block's start; deeper or shallower schedules measured the same or worse.
-  const int j_first = kv_begin & ~31;
-  // PAGE32: the page numbers of this block, the next and the one after, looked up (scalar
-  // loads) two blocks before the loads that need them
-  auto page_at = [&](int j0) {
-    if constexpr (PAGE32) return uniform(bt[(j0 < kv_end ? j0 : j_first) >> page_shift]);
-    else return 0;
-  };
-  int page_cur = page_at(j_first), page_next = page_at(j_first + 32);
-  bf16x8 kcur[2][KT], vf[DT];
-  bf16x8 knext[2][KT];
-  if (j_first < kv_end) load_keys(j_first, page_cur, kcur);
-
-  for (int j0 = j_first; j0 < kv_end; j0 += 32) {
-    const int jv = value_index(j0);
-    const bool tail = j0 + 32 > kv_len;  // some of the 32 keys are not written yet
-    const bool more = j0 + 32 < kv_end;
-    const int page_after = page_at(j0 + 64);
-    load_values(j0, page_cur, vf);
-    if (more) load_keys(j0 + 32, page_next, knext);
 
     // ---- S^T = K Q^T for 32 keys (two tiles of 16), all row tiles ------------------
     f32x4 s[RT][2];
@@ -242,7 +320,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     for (int rt = 0; rt < RT; ++rt) {
       // a block wholly after the tile's last row or before its first row's window
       // does nothing for this tile
-      active[rt] = j0 <= p_last[rt] && j0 + 31 >= lo_first[rt];
+      active[rt] = j0 <= p_last[rt] && j0 + 31 >= lo_first[rt] && j0 < kv_end && j0 + 32 > kv_begin;
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         s[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -309,22 +387,6 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     }
 
     // ---- O^T += V^T P^T ------------------------------------------------------------
-    // unwritten slots may hold anything, NaN included, and 0 * NaN must not get in:
-    // in the last block of the request the values of keys past the end are cleared
-    if (tail) {
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const int ja = jv + 2 * w;
-        const uint32_t keep =
-            (ja <= last_key ? 0x0000ffffu : 0u) | (ja + 1 <= last_key ? 0xffff0000u : 0u);
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          u32x4 raw = __builtin_bit_cast(u32x4, vf[dt]);
-          raw[w] &= keep;
-          vf[dt] = __builtin_bit_cast(bf16x8, raw);
-        }
-      }
-    }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       // rescale the sums only if some row of the tile raised its maximum
@@ -335,6 +397,14 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
           for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha[rt];
       }
     }
+    if constexpr (SHARED) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        vf[dt] = __builtin_bit_cast(bf16x8, frag_lds[half][2 * KT + dt][lane]);
+    } else if (tail) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vf[dt] = clear_unwritten(j0, vf[dt]);
+    }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       if (!active[rt]) continue;
@@ -342,12 +412,22 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       for (int dt = 0; dt < DT; ++dt)
         o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb[rt], o[rt][dt], 0, 0, 0);
     }
+    if constexpr (SHARED) {
+      // the other half was read in the block before this one, and every wave has passed
+      // the barrier since
+      if (more) stash(j0 + 32, half ^ 1);
+      if (j0 + 64 < walk_end) fetch(j0 + 64, page_2);
+      __syncthreads();
+      half ^= 1;
+    } else {
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int ks = 0; ks < KT; ++ks) kcur[t][ks] = knext[t][ks];
-    page_cur = page_next;
-    page_next = page_after;
+        for (int ks = 0; ks < KT; ++ks) kcur[t][ks] = knext[t][ks];
+    }
+    page_0 = page_1;
+    page_1 = page_2;
+    page_2 = page_3;
   }
 
 #pragma unroll
@@ -483,8 +563,8 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
                                   const int* seg_q_len, const int* seg_kv_len,
                                   const int* block_table, int bt_stride, const void* k_pages,
                                   const void* v_pages, float* part_o, float* part_ml, int H, int K,
-                                  int head_dim, int page_size, float scale, int window,
-                                  hipStream_t stream) {
+                                  int head_dim, int page_size, int tiled, float scale,
+                                  int window, hipStream_t stream) {
   HAL_REQUIRE(head_dim == D, "hal_attention_mfma: built for head size %d, called with %d", D,
               head_dim);
   HAL_REQUIRE(H > 0 && K > 0 && H % K == 0, "hal_attention_mfma: %d heads, %d kv heads", H, K);
@@ -497,26 +577,30 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   HAL_REQUIRE(window >= 0 && max_items >= 0 && max_big >= 0 && max_merges >= 0,
               "hal_attention_mfma: bad counts");
   HAL_REQUIRE(max_merges == 0 || (part_o && part_ml), "hal_attention_mfma: no partial buffers");
+  HAL_REQUIRE(!tiled || (D % 32 == 0 && page_size >= 32 && (page_size & (page_size - 1)) == 0),
+              "hal_attention_mfma: the tiled page layout needs a head size of a multiple of 32 "
+              "and pages of a power of two of at least 32 tokens (head %d, page %d)", D, page_size);
   const float scale_log2e = scale * 1.4426950408889634f;
   int page_shift = -1;
   if ((page_size & (page_size - 1)) == 0)
     for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
-  const int waves = 4;
-#define LAUNCH_ATTENTION(RT_, LIST, MAX, COUNT)                                                   \
+  const int waves = WAVES;
+#define LAUNCH_ATTENTION(RT_, SHARED_, LIST, MAX, COUNT)                                          \
   {                                                                                               \
     dim3 grid(((MAX) + waves - 1) / waves, K);                                                    \
-    hipLaunchKernelGGL((page_shift >= 5   ? attention_mfma_kernel<RT_, true, true>                \
-                        : page_shift >= 0 ? attention_mfma_kernel<RT_, true, false>               \
-                                          : attention_mfma_kernel<RT_, false, false>),            \
-                       grid, dim3(waves * HAL_WAVE), 0, stream, (const bf16_t*)q, q_row_stride,   \
-                       (bf16_t*)out, out_row_stride, LIST, COUNT, seg_q_start, seg_q_len,         \
-                       seg_kv_len, block_table, bt_stride, (const bf16_t*)k_pages,                \
+    auto kernel = attention_mfma_kernel<RT_, false, false, SHARED_, false>;                       \
+    if (tiled) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, D % 32 == 0>;             \
+    else if (page_shift >= 5) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, false>;    \
+    else if (page_shift >= 0) kernel = attention_mfma_kernel<RT_, true, false, SHARED_, false>;   \
+    hipLaunchKernelGGL(kernel, grid, dim3(waves * HAL_WAVE), 0, stream, (const bf16_t*)q,         \
+                       q_row_stride, (bf16_t*)out, out_row_stride, LIST, COUNT, seg_q_start,      \
+                       seg_q_len, seg_kv_len, block_table, bt_stride, (const bf16_t*)k_pages,     \
                        (const bf16_t*)v_pages, part_o, part_ml, H, K, page_size, page_shift,      \
                        scale_log2e, window);                                                      \
     HAL_LAUNCH_CHECK();                                                                           \
   }
-  if (max_items > 0) LAUNCH_ATTENTION(1, items, max_items, counts)
-  if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, big_items, max_big, counts + 1)
+  if (max_items > 0) LAUNCH_ATTENTION(1, false, items, max_items, counts)
+  if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, true, big_items, max_big, counts + 1)
 #undef LAUNCH_ATTENTION
   if (max_merges > 0) {
     hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K), dim3(256), 0, stream,

@@ -324,7 +324,7 @@ __global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
                                    const float* __restrict__ sin_t, int table_len,
                                    T* __restrict__ k_pages, T* __restrict__ v_pages, int H,
                                    int K, int D, int rot, int interleaved, int page_size,
-                                   int n_pages) {
+                                   int n_pages, bool tiled) {
   const int t = blockIdx.x;
   const int pos = positions[t];
   T* row = qkv + (size_t)t * row_stride;
@@ -354,9 +354,9 @@ __global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
     hp[i1] = y1;
     if (head >= H && page >= 0) {
       const int g = head - H;
-      T* kp = k_pages + (((size_t)page * K + g) * page_size + off) * D;
-      kp[i0] = y0;
-      kp[i1] = y1;
+      T* kp = k_pages + ((size_t)page * K + g) * page_size * D;
+      kp[kv_key_offset(tiled, page_size, D, off, i0)] = y0;
+      kp[kv_key_offset(tiled, page_size, D, off, i1)] = y1;
     }
   }
   if (page < 0) return;
@@ -364,11 +364,13 @@ __global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
   const int rest = D - rot;
   for (int idx = threadIdx.x; idx < K * rest; idx += blockDim.x) {
     const int g = idx / rest, i = rot + idx % rest;
-    k_pages[(((size_t)page * K + g) * page_size + off) * D + i] = row[(size_t)(H + g) * D + i];
+    k_pages[((size_t)page * K + g) * page_size * D + kv_key_offset(tiled, page_size, D, off, i)] =
+        row[(size_t)(H + g) * D + i];
   }
   for (int idx = threadIdx.x; idx < K * D; idx += blockDim.x) {
     const int g = idx / D, i = idx % D;
-    v_pages[(((size_t)page * K + g) * D + i) * page_size + off] = row[(size_t)(H + K + g) * D + i];
+    v_pages[((size_t)page * K + g) * D * page_size + kv_value_offset(tiled, page_size, D, off, i)] =
+        row[(size_t)(H + K + g) * D + i];
   }
 }
 
@@ -383,7 +385,7 @@ __global__ void rope_append_vec_kernel(T* __restrict__ qkv, int row_stride,
                                        const float* __restrict__ sin_t, int table_len,
                                        T* __restrict__ k_pages, T* __restrict__ v_pages, int H,
                                        int K, int D, int rot, int interleaved, int page_size,
-                                       int n_pages) {
+                                       int n_pages, bool tiled) {
   const int t = blockIdx.x;
   const int pos = positions[t];
   T* row = qkv + (size_t)t * row_stride;
@@ -419,16 +421,15 @@ __global__ void rope_append_vec_kernel(T* __restrict__ qkv, int row_stride,
           y0[u][i] = a[u][i] * c[u][i] - b[u][i] * sn[u][i];
           y1[u][i] = a[u][i] * sn[u][i] + b[u][i] * c[u][i];
         }
-      T* kp = (head >= H && page >= 0)
-                  ? k_pages + (((size_t)page * K + (head - H)) * page_size + off) * D
-                  : nullptr;
+      T* kp = (head >= H && page >= 0) ? k_pages + ((size_t)page * K + (head - H)) * page_size * D
+                                       : nullptr;
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         store4(hp + j + 4 * u, y0[u]);
         store4(hp + j + half + 4 * u, y1[u]);
         if (kp) {
-          store4(kp + j + 4 * u, y0[u]);
-          store4(kp + j + half + 4 * u, y1[u]);
+          store4(kp + kv_key_offset(tiled, page_size, D, off, j + 4 * u), y0[u]);
+          store4(kp + kv_key_offset(tiled, page_size, D, off, j + half + 4 * u), y1[u]);
         }
       }
     }
@@ -451,9 +452,9 @@ __global__ void rope_append_vec_kernel(T* __restrict__ qkv, int row_stride,
       store4(hp + e0, y[0]);
       store4(hp + e0 + 4, y[1]);
       if (head >= H && page >= 0) {
-        T* kp = k_pages + (((size_t)page * K + (head - H)) * page_size + off) * D;
-        store4(kp + e0, y[0]);
-        store4(kp + e0 + 4, y[1]);
+        T* kp = k_pages + ((size_t)page * K + (head - H)) * page_size * D;
+        store4(kp + kv_key_offset(tiled, page_size, D, off, e0), y[0]);
+        store4(kp + kv_key_offset(tiled, page_size, D, off, e0 + 4), y[1]);
       }
     }
   }
@@ -464,9 +465,9 @@ __global__ void rope_append_vec_kernel(T* __restrict__ qkv, int row_stride,
     float a[2][4];
     load4(row + (size_t)(H + g) * D + i, a[0]);
     load4(row + (size_t)(H + g) * D + i + 4, a[1]);
-    T* kp = k_pages + (((size_t)page * K + g) * page_size + off) * D + i;
-    store4(kp, a[0]);
-    store4(kp + 4, a[1]);
+    T* kp = k_pages + ((size_t)page * K + g) * page_size * D;
+    store4(kp + kv_key_offset(tiled, page_size, D, off, i), a[0]);
+    store4(kp + kv_key_offset(tiled, page_size, D, off, i + 4), a[1]);
   }
   const int d8 = D / 8;
   for (int idx = threadIdx.x; idx < K * d8; idx += blockDim.x) {
@@ -475,9 +476,9 @@ __global__ void rope_append_vec_kernel(T* __restrict__ qkv, int row_stride,
     T vals[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) vals[e] = vr[e];
-    T* vp = v_pages + (((size_t)page * K + g) * D + i) * page_size + off;
+    T* vp = v_pages + ((size_t)page * K + g) * D * page_size;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) vp[(size_t)e * page_size] = vals[e];
+    for (int e = 0; e < 8; ++e) vp[kv_value_offset(tiled, page_size, D, off, i + e)] = vals[e];
   }
 }
 
@@ -485,7 +486,7 @@ extern "C" int hal_rope_append(void* qkv, int dtype, int row_stride, const int* 
                                const int* token_seg, const int* block_table, int bt_stride,
                                const float* cos_t, const float* sin_t, int table_len,
                                void* k_pages, void* v_pages, int n_tokens, int H, int K, int D,
-                               int rot, int interleaved, int page_size, int n_pages,
+                               int rot, int interleaved, int page_size, int n_pages, int tiled,
                                hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && H >= 0 && K >= 0 && D > 0, "hal_rope_append: bad sizes");
   HAL_REQUIRE(rot >= 0 && rot <= D && rot % 2 == 0, "hal_rope_append: rotary dim %d of %d", rot, D);
@@ -495,6 +496,9 @@ extern "C" int hal_rope_append(void* qkv, int dtype, int row_stride, const int* 
               "hal_rope_append: cache arguments missing");
   if (n_tokens == 0) return 0;
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_rope_append: unknown dtype %d", dtype);
+  HAL_REQUIRE(!tiled || (page_size % 32 == 0 && D % 32 == 0),
+              "hal_rope_append: the tiled page layout needs pages and heads of a multiple of 32 "
+              "(page %d, head %d)", page_size, D);
   const bool vec = D % 8 == 0 && row_stride % 8 == 0 && (interleaved ? rot % 8 == 0 : rot % 16 == 0);
   if (vec) {
     int items = (H + K) * (rot / 8) / (interleaved ? 1 : 2);
@@ -505,12 +509,12 @@ extern "C" int hal_rope_append(void* qkv, int dtype, int row_stride, const int* 
       hipLaunchKernelGGL(rope_append_vec_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream,
                          (float*)qkv, row_stride, positions, token_seg, block_table, bt_stride,
                          cos_t, sin_t, table_len, (float*)k_pages, (float*)v_pages, H, K, D, rot,
-                         interleaved, page_size, n_pages);
+                         interleaved, page_size, n_pages, tiled != 0);
     else
       hipLaunchKernelGGL(rope_append_vec_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream,
                          (bf16_t*)qkv, row_stride, positions, token_seg, block_table, bt_stride,
                          cos_t, sin_t, table_len, (bf16_t*)k_pages, (bf16_t*)v_pages, H, K, D,
-                         rot, interleaved, page_size, n_pages);
+                         rot, interleaved, page_size, n_pages, tiled != 0);
     HAL_LAUNCH_CHECK();
     return 0;
   }
@@ -520,12 +524,12 @@ extern "C" int hal_rope_append(void* qkv, int dtype, int row_stride, const int* 
     hipLaunchKernelGGL(rope_append_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream,
                        (float*)qkv, row_stride, positions, token_seg, block_table, bt_stride,
                        cos_t, sin_t, table_len, (float*)k_pages, (float*)v_pages, H, K, D, rot,
-                       interleaved, page_size, n_pages);
+                       interleaved, page_size, n_pages, tiled != 0);
   else if (dtype == HAL_BF16)
     hipLaunchKernelGGL(rope_append_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream,
                        (bf16_t*)qkv, row_stride, positions, token_seg, block_table, bt_stride,
                        cos_t, sin_t, table_len, (bf16_t*)k_pages, (bf16_t*)v_pages, H, K, D, rot,
-                       interleaved, page_size, n_pages);
+                       interleaved, page_size, n_pages, tiled != 0);
   else
     return hal_fail("hal_rope_append: unknown dtype %d", dtype);
   HAL_LAUNCH_CHECK();

@@ -26,7 +26,7 @@ int hal_rope_append(void* qkv, int dtype, int row_stride, const int* positions,
                     const int* token_seg, const int* block_table, int bt_stride,
                     const float* cos_t, const float* sin_t, int table_len, void* k_pages,
                     void* v_pages, int n_tokens, int H, int K, int D, int rot, int interleaved,
-                    int page_size, int n_pages, hipStream_t stream);
+                    int page_size, int n_pages, int tiled, hipStream_t stream);
 
 int hal_attention_simple(const void* q, int q_row_stride, void* out, int out_row_stride,
                          int dtype, const int* positions, const int* token_seg,
@@ -55,6 +55,7 @@ int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_s
                        const int* seg_q_start, const int* seg_q_len, const int* seg_kv_len,
                        const int* block_table, int bt_stride, const void* k_pages,
                        const void* v_pages, float* part_o, float* part_ml, int H, int K,
-                       int head_dim, int page_size, float scale, int window, hipStream_t stream);
+                       int head_dim, int page_size, int tiled, float scale, int window,
+                       hipStream_t stream);
 
 }  // extern "C"

@@ -116,6 +116,28 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Where element (slot, d) of one kv head's part of a page lies, counted in elements from
+// that part's start.  Plain: keys [slot][D], values transposed [D][slot].  Tiled (pages of
+// a multiple of 32 tokens, head sizes of a multiple of 32): per block of 32 slots the keys
+// and the values lie in the order in which the matrix-core attention kernel's waves load
+// them, one contiguous KB per MFMA operand:
+//   keys   [block][tile t of 16 keys][32-dim step ks][dim quad][key c][8 dims],
+//          slot r of the block is key c = (r/8)*4 + r%4 of tile t = (r%8)/4;
+//   values [block][16-dim tile dt][8-key group][dim][8 keys].
+__host__ __device__ __forceinline__ size_t kv_key_offset(bool tiled, int page_size, int D, int slot,
+                                                         int d) {
+  if (!tiled) return (size_t)slot * D + d;
+  const int r = slot % 32, t = (r % 8) / 4, c = (r / 8) * 4 + r % 4;
+  const int ks = d / 32, quad = (d % 32) / 8;
+  return (size_t)(slot / 32) * 32 * D + (((t * (D / 32) + ks) * 64 + quad * 16 + c) * 8 + d % 8);
+}
+__host__ __device__ __forceinline__ size_t kv_value_offset(bool tiled, int page_size, int D,
+                                                           int slot, int d) {
+  if (!tiled) return (size_t)d * page_size + slot;
+  const int r = slot % 32;
+  return (size_t)(slot / 32) * 32 * D + (((d / 16) * 64 + (r / 8) * 16 + d % 16) * 8 + r % 8);
+}
+
 // Sum over a block of up to 1024 threads; every thread gets the result.
 // `scratch` is shared memory for 16 floats.  Safe to call repeatedly with the
 // same scratch.

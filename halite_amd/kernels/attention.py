@@ -22,6 +22,7 @@ ROWS_PER_ITEM = 16
 KEYS_PER_BLOCK = 32
 MIN_SPLIT_KEYS = 128
 TARGET_WAVES = 2048
+WAVES_PER_GROUP = 4  # waves of a workgroup of the kernel for long segments: they share keys through LDS
 
 
 @dataclass
@@ -73,8 +74,9 @@ def mfma_supported(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
 
 
 def rows_per_big_item(head_dim: int) -> int:
-    """Rows of a wave's tile for long segments; the kernel's HAL_RT_BIG times 16."""
-    return 64 if head_dim <= 64 else (32 if head_dim <= 128 else 16)
+    """Rows that one wave takes of a long segment: the kernel library for this head size
+    says how it was built."""
+    return int(library.attention_library(head_dim).hal_attention_mfma_rows_per_big_item())
 
 
 def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick):
@@ -98,7 +100,7 @@ def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick):
     return np.concatenate(seg_ids), np.concatenate(rho0s), np.concatenate(kv_b), np.concatenate(kv_e)
 
 
-def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_seg, more_tiles=None):
+def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_seg, more_tiles=None, group=1):
     """Items and merge entries of tiles whose key ranges are cut into pieces of
     ``chunk`` keys (pieces end on multiples of 32 keys).  ``more_tiles`` [n, k] holds
     the first rows of an item's further 16-row tiles (-1: none)."""
@@ -131,9 +133,41 @@ def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_
             if r0 >= 0:
                 merges.append([seg_ids[t], r0, slot0 + sub, n_pieces[t], slots_per_tile, 0, 0, 0])
     merges = np.array(merges, dtype=np.int32).reshape(-1, 8)
-    # the longest key ranges first: the waves that run longest start earliest
-    order = np.argsort(-(items[:, 3] - items[:, 2]), kind="stable")
-    return items[order], merges, first_slot + n_split * slots_per_tile
+    if group > 1:
+        items = _group_items(items, piece, group)
+    else:
+        # the longest key ranges first: the waves that run longest start earliest
+        items = items[np.argsort(-(items[:, 3] - items[:, 2]), kind="stable")]
+    return items, merges, first_slot + n_split * slots_per_tile
+
+
+def _group_items(items: np.ndarray, piece: np.ndarray, group: int) -> np.ndarray:
+    """Orders items so that every run of ``group`` items (a workgroup's waves) belongs to
+    one segment and to the same piece of neighbouring tiles, i.e. walks nearly the same
+    keys; a run that cannot be filled is padded with items that have no rows and no keys.
+    The runs with the longest walk come first."""
+    n = len(items)
+    order = np.lexsort((np.arange(n), piece, items[:, 0]))  # segment, then piece, then tile
+    runs = []
+    start = 0
+    keys = np.stack((items[order, 0], piece[order]), axis=1)
+    for i in range(1, n + 1):
+        if i == n or (keys[i] != keys[start]).any():
+            idx = order[start:i]
+            for c in range(0, len(idx), group):
+                run = items[idx[c : c + group]]
+                if len(run) < group:
+                    pad = np.full((group - len(run), 8), -1, dtype=np.int32)
+                    pad[:, 0] = run[0, 0]
+                    pad[:, 2:4] = 0
+                    run = np.concatenate((run, pad))
+                runs.append(run)
+            start = i
+    def walk(run):
+        live = run[run[:, 3] > run[:, 2]]
+        return int(live[:, 3].max() - live[:, 2].min()) if len(live) else 0
+    runs.sort(key=lambda r: -walk(r))
+    return np.concatenate(runs) if runs else np.zeros((0, 8), np.int32)
 
 
 def _group_tiles(seg_ids, rho0s, kv_b, kv_e, per_item: int, zigzag: bool):
@@ -180,7 +214,7 @@ def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: 
         chunk = -(-total // TARGET_WAVES)
         chunk = max(MIN_SPLIT_KEYS, -(-chunk // KEYS_PER_BLOCK) * KEYS_PER_BLOCK)
     items, merges_s, slot = _cut(*small, chunk, 1, 0, rows_of_seg)
-    big_items, merges_b, slot = _cut(*big, chunk, per_item, slot, rows_of_seg, more)
+    big_items, merges_b, slot = _cut(*big, chunk, per_item, slot, rows_of_seg, more, group=WAVES_PER_GROUP)
     merges = np.concatenate((merges_s, merges_b)) if len(merges_s) or len(merges_b) else np.zeros((0, 8), np.int32)
     return AttentionPlan(items, big_items, merges, slot, rows_big)
 
@@ -201,7 +235,8 @@ def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, wi
         P(items), plan.cap_items, P(big_items), plan.cap_big, P(merges), plan.cap_merges, P(counts),
         P(ctx.seg_q_start), P(ctx.seg_q_len), P(ctx.seg_kv_len),
         P(group.block_table), group.block_table.shape[1], P(kv.k), P(kv.v), P(part_o), P(part_ml),
-        n_heads, n_kv, head_dim, page_size, ctypes.c_float(scale), window, ops._stream(),
+        n_heads, n_kv, head_dim, page_size, 1 if getattr(kv, "tiled", False) else 0,
+        ctypes.c_float(scale), window, ops._stream(),
     )
     ops._check(lib, rc)
     return out
@@ -221,6 +256,11 @@ def paged_attention(ctx, q, q_row_stride, kv, group, n_heads, scale, window):
             ctx.plan_attention(group.group_id, n_heads, n_kv, window, head_dim, late=True)
             plan_dev = ctx.device_plan(group.group_id, n_heads // n_kv, window)
         return attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, window)
+    if getattr(kv, "tiled", False):
+        raise ops.KernelError(
+            f"pages are kept in the matrix-core kernel's order, which only that kernel reads "
+            f"(dtype {q.dtype}, head size {head_dim}, page size {page_size}, row stride {q_row_stride})"
+        )
     return ops.attention_simple(
         q, q_row_stride, ctx.positions, ctx.token_seg, group.block_table, kv.k, kv.v, n_heads, scale, window
     )

@@ -152,9 +152,11 @@ def rope_append(
     k_pages: torch.Tensor | None = None,
     v_pages: torch.Tensor | None = None,
     page_size: int = 0,
+    tiled: bool = False,
 ):
     """Rotate q and k in place in the packed rows ``[q | k | v]`` and append k and
-    v to the pages (``n_kv_heads == 0``: rows hold q only, nothing is appended)."""
+    v to the pages (``n_kv_heads == 0``: rows hold q only, nothing is appended);
+    ``tiled`` says that the pages are kept in the matrix-core kernel's own order."""
     lib = library.core_library()
     _dev(qkv, positions, cos, sin, token_seg, block_table, k_pages, v_pages)
     _i32(positions, "positions"), _i32(token_seg, "token_seg"), _i32(block_table, "block_table")
@@ -180,7 +182,7 @@ def rope_append(
             _ptr(block_table), 0 if block_table is None else block_table.shape[1],
             _ptr(cos), _ptr(sin), cos.shape[0], _ptr(k_pages), _ptr(v_pages),
             n, n_heads, n_kv_heads, head_dim, rotary_dim, 1 if interleaved else 0,
-            page_size, n_pages, _stream(),
+            page_size, n_pages, 1 if tiled else 0, _stream(),
         ),
     )
 

@@ -109,7 +109,7 @@ class Attention(Mixer):
         ops.rope_append(
             qkv, ctx.positions, cos, sin, p.n_heads, n_kv_append, p.head_dim, rot, interleaved,
             token_seg=ctx.token_seg, block_table=group.block_table,
-            k_pages=kv.k, v_pages=kv.v, page_size=group.page_size,
+            k_pages=kv.k, v_pages=kv.v, page_size=group.page_size, tiled=kv.tiled,
         )
         out = ctx.attention(qkv, qkv.shape[1], kv, group, p.n_heads, p.scale, p.window or 0)
         return ops.linear(out, self.w_out, tiled=self.t_out)

@@ -10,8 +10,17 @@ def check_plan(plan, q_len, kv_len, group, window):
     a cut group has one merge entry per tile whose partial slots are its own."""
     per_item = max(1, plan.rows_big // 16)
     groups = {}
+    # the long segments' items come in runs of four (a workgroup's waves): one segment per
+    # run, padded with items that have no rows and no keys
+    assert plan.n_big % 4 == 0
+    for r in range(0, plan.n_big, 4):
+        run = plan.big_items[r : r + 4]
+        assert len(set(run[:, 0].tolist())) == 1 and run[0, 1] >= 0
     for arr, is_big in ((plan.items, False), (plan.big_items, True)):
         for seg, rho0, b, e, partial, *more in arr.tolist():
+            if is_big and rho0 < 0:
+                assert (b, e, partial, more) == (0, 0, -1, [-1, -1, -1])
+                continue
             rows = q_len[seg] * group
             assert (rows > 16 and per_item > 1) == is_big
             assert 0 <= b < e <= kv_len[seg]

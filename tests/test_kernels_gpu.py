@@ -100,10 +100,46 @@ def paged_cache(k, v, page_size, seed, n_extra=3, dtype=torch.float32, poison=Tr
     return kp.to(dtype), vp.to(dtype), perm.to(torch.int32)
 
 
+def tiled_maps(page, D):
+    """Where element (slot, d) of one kv head's part of a page lies in the tiled page
+    layout: per block of 32 slots, keys as [16-key tile][32-dim step][dim quad][key][8 dims]
+    with slot r = key (r/8)*4 + r%4 of tile (r%8)/4, values as [16-dim tile][8-key group]
+    [dim][8 keys].  Both maps are permutations of the page's elements."""
+    slot, d = torch.arange(page).view(-1, 1), torch.arange(D).view(1, -1)
+    r = slot % 32
+    tile, key = (r % 8) // 4, (r // 8) * 4 + r % 4
+    kmap = (slot // 32) * 32 * D + ((tile * (D // 32) + d // 32) * 64 + ((d % 32) // 8) * 16 + key) * 8 + d % 8
+    vmap = (slot // 32) * 32 * D + ((d // 16) * 64 + (r // 8) * 16 + d % 16) * 8 + r % 8
+    for m in (kmap, vmap):
+        assert sorted(m.flatten().tolist()) == list(range(page * D))
+    return kmap.flatten(), vmap.flatten()
+
+
+def to_tiled(kp, vp):
+    """Plain pages (keys [P, K, page, D], values [P, K, D, page]) in the tiled layout
+    (same shapes, other order of the elements of a (page, kv head))."""
+    P_, K, page, D = kp.shape
+    kmap, vmap = tiled_maps(page, D)
+    kt, vt = torch.empty(P_, K, page * D, dtype=kp.dtype), torch.empty(P_, K, page * D, dtype=vp.dtype)
+    kt[:, :, kmap] = kp.reshape(P_, K, page * D)
+    vt[:, :, vmap] = vp.transpose(2, 3).reshape(P_, K, page * D)
+    return kt.view(P_, K, page, D), vt.view(P_, K, D, page)
+
+
+def from_tiled(kt, vt):
+    P_, K, page, D = kt.shape
+    kmap, vmap = tiled_maps(page, D)
+    kp = kt.reshape(P_, K, page * D)[:, :, kmap].view(P_, K, page, D)
+    vp = vt.reshape(P_, K, page * D)[:, :, vmap].view(P_, K, page, D).transpose(2, 3)
+    return kp, vp
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("interleaved", [False, True])
-@pytest.mark.parametrize("H,K,D,rot,page", [(4, 2, 16, 16, 4), (6, 2, 48, 48, 16), (3, 1, 32, 16, 8), (8, 8, 128, 128, 64)])
-def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page):
+@pytest.mark.parametrize("H,K,D,rot,page,tiled", [
+    (4, 2, 16, 16, 4, False), (6, 2, 48, 48, 16, False), (3, 1, 32, 16, 8, False), (8, 8, 128, 128, 64, False),
+    (8, 8, 128, 128, 64, True), (3, 1, 32, 16, 32, True), (4, 2, 64, 64, 32, True), (2, 1, 96, 40, 64, True)])
+def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page, tiled):
     dt = DT[dtype]
     n_seg, table_w = 3, -(-64 // page)
     lens, starts = [5, 1, 9], [3, 40, 0]
@@ -120,7 +156,7 @@ def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page):
     got = qkv.to(gpu).clone()
     ops.rope_append(got, positions.to(gpu), cos.to(gpu), sin.to(gpu), H, K, D, rot, interleaved,
                     token_seg=token_seg.to(gpu), block_table=bt.to(torch.int32).to(gpu),
-                    k_pages=kp, v_pages=vp, page_size=page)
+                    k_pages=kp, v_pages=vp, page_size=page, tiled=tiled)
     q = qkv[:, : H * D].float().view(T, H, D)
     k = qkv[:, H * D : (H + K) * D].float().view(T, K, D)
     v = qkv[:, (H + K) * D :].float().view(T, K, D)
@@ -132,6 +168,8 @@ def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page):
     close(got[:, : H * D].view(T, H, D), rq, tol, "rotated q")
     assert torch.equal(got[:, (H + K) * D :].cpu(), qkv[:, (H + K) * D :])  # v untouched
     kpc, vpc = kp.float().cpu(), vp.float().cpu()
+    if tiled:
+        kpc, vpc = from_tiled(kpc, vpc)
     written = torch.zeros(n_pages, page, dtype=torch.bool)
     for t in range(T):
         pos, seg = int(positions[t]), int(token_seg[t])
@@ -143,7 +181,7 @@ def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page):
     assert float(vpc.abs().sum(dim=(1, 2))[~written].sum()) == 0
 
 
-def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use):
+def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use, tiled=False):
     """``segs``: list of (cached before, new tokens).  Builds one dense sequence per
     segment, pages it, and compares the rows of the new tokens with plain attention
     over the whole sequence."""
@@ -177,7 +215,10 @@ def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use):
     bt = torch.full((len(segs), width), -1, dtype=torch.int32)
     for i, t in enumerate(tables):
         bt[i, : len(t)] = t
-    k_pages, v_pages = torch.cat(kps).to(gpu), torch.cat(vps).to(gpu)
+    k_pages, v_pages = torch.cat(kps), torch.cat(vps)
+    if tiled:
+        k_pages, v_pages = to_tiled(k_pages, v_pages)
+    k_pages, v_pages, is_tiled = k_pages.to(gpu), v_pages.to(gpu), tiled
     q = torch.cat(qs).to(dt).to(gpu)
     positions = torch.cat(pos).to(torch.int32).to(gpu)
     token_seg = torch.cat(seg_of).to(torch.int32).to(gpu)
@@ -199,7 +240,7 @@ def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use):
             block_table = bt.to(gpu)
 
         class KV:
-            k, v = k_pages, v_pages
+            k, v, tiled = k_pages, v_pages, is_tiled
 
         out = attn_kernels.attention_mfma(q, H * D, attn_kernels.upload_plan(plan, gpu), Ctx, Group, KV, H, scale, window)
     close(out, torch.cat(want), 5e-6 if dtype == "float32" else 1.2e-2, f"attention {use}")
@@ -222,6 +263,9 @@ def test_attention_simple(gpu, dtype, H, K, D, segs):
 def test_attention_mfma(gpu, H, K, D, segs):
     for page, window in ((8, 0), (16, 0), (64, 0), (24, 0), (16, 37), (8, 1), (64, 300)):
         attention_case(gpu, "bfloat16", H, K, D, page, segs, window, seed=30, use="mfma")
+    if D % 32 == 0:  # the pages in the kernel's own order
+        for page, window in ((32, 0), (64, 0), (128, 0), (64, 300), (32, 37)):
+            attention_case(gpu, "bfloat16", H, K, D, page, segs, window, seed=31, use="mfma", tiled=True)
 
 
 def test_attention_mfma_split_keys(gpu):
@@ -234,6 +278,9 @@ def test_attention_mfma_split_keys(gpu):
     # a short portion against a long context: tiles of 64 rows, cut and merged
     attention_case(gpu, "bfloat16", 8, 2, 128, 64, [(5000, 40), (2500, 100)], 0, seed=42, use="mfma")
     attention_case(gpu, "bfloat16", 6, 2, 48, 16, [(3000, 50)], 700, seed=43, use="mfma")
+    attention_case(gpu, "bfloat16", 8, 2, 128, 64, segs, 0, seed=44, use="mfma", tiled=True)
+    attention_case(gpu, "bfloat16", 8, 2, 128, 64, [(5000, 40), (2500, 100)], 0, seed=45, use="mfma", tiled=True)
+    attention_case(gpu, "bfloat16", 4, 1, 64, 32, [(3000, 50), (0, 600)], 700, seed=46, use="mfma", tiled=True)
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 256, 64), (5, 331, 120), (64, 200, 352), (130, 96, 1000), (3, 4096, 4096)])
