@@ -166,6 +166,12 @@ class CacheManager:
             for slot, table in g.tables.items():
                 if slot not in live:
                     raise AssertionError(f"group {g.group_id}: table of dead slot {slot}")
+                done = g.released.get(slot, 0)
+                if any(p >= 0 for p in table[:done]) or any(p < 0 for p in table[done:]):
+                    raise AssertionError(
+                        f"group {g.group_id}: slot {slot} has a hole behind its first held page "
+                        f"(released {done}, table {table})"
+                    )
                 for p in table:
                     if p < 0:
                         continue

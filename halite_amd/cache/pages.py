@@ -100,6 +100,7 @@ class CacheGroup:
     pool: PagePool
     # per live slot: page number for every logical page, -1 where none is held
     tables: dict[int, list[int]] = field(default_factory=dict)
+    released: dict[int, int] = field(default_factory=dict)
     storage: torch.Tensor | None = None  # [runs, 2, pages, K * page_size * D]
 
     def first_needed_page(self, next_position: int) -> int:
@@ -110,23 +111,25 @@ class CacheGroup:
         oldest_key = next_position - self.need.window + 1
         return max(0, oldest_key // self.page_size)
 
+    # A request's table has no holes behind its first held page: ``released[slot]``
+    # leading entries were given back (they are -1), every later entry holds a page.
     def pages_missing(self, slot: int, start: int, new_len: int) -> int:
         """Pages to allocate so that the tokens ``[start, new_len)`` can be run:
         their own positions, and nothing that the window has passed."""
-        table = self.tables.get(slot, [])
+        return len(self._wanted(slot, start, new_len))
+
+    def _wanted(self, slot: int, start: int, new_len: int) -> range | list[int]:
+        table = self.tables.get(slot, ())
         first = self.first_needed_page(start)
         last = (new_len - 1) // self.page_size
-        n = 0
-        for i in range(first, last + 1):
-            if i >= len(table) or table[i] < 0:
-                n += 1
-        return n
+        if first >= self.released.get(slot, 0):  # nothing that was given back is asked for again
+            return range(max(first, len(table)), last + 1)
+        return [i for i in range(first, last + 1) if i >= len(table) or table[i] < 0]
 
     def reserve(self, slot: int, start: int, new_len: int) -> None:
+        want = self._wanted(slot, start, new_len)
         table = self.tables.setdefault(slot, [])
-        first = self.first_needed_page(start)
         last = (new_len - 1) // self.page_size
-        want = [i for i in range(first, last + 1) if i >= len(table) or table[i] < 0]
         pages = self.pool.alloc(len(want))
         while len(table) <= last:
             table.append(-1)
@@ -141,14 +144,19 @@ class CacheGroup:
         if not table:
             return 0
         first = min(self.first_needed_page(next_position), len(table))
-        dead = [p for p in table[:first] if p >= 0]
-        for i in range(first):
+        done = self.released.get(slot, 0)
+        if first <= done:
+            return 0
+        dead = [p for p in table[done:first] if p >= 0]
+        for i in range(done, first):
             table[i] = -1
+        self.released[slot] = first
         self.pool.free(dead)
         return len(dead)
 
     def release_all(self, slot: int) -> int:
         table = self.tables.pop(slot, [])
+        self.released.pop(slot, None)
         held = [p for p in table if p >= 0]
         self.pool.free(held)
         return len(held)

@@ -80,24 +80,25 @@ def rows_per_big_item(head_dim: int) -> int:
 
 
 def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick):
-    seg_ids, rho0s, kv_b, kv_e = [], [], [], []
-    for s, (ql, kl) in enumerate(zip(seg_q_len, seg_kv_len)):
-        ql, kl = int(ql), int(kl)
-        rows = ql * group_size
-        if not pick(rows):
-            continue
-        r0 = np.arange(0, rows, rows_per_tile, dtype=np.int64)
-        first_q = r0 // group_size
-        last_q = np.minimum(rows - 1, r0 + rows_per_tile - 1) // group_size
-        pos0 = kl - ql
-        b = np.zeros_like(r0) if window <= 0 else np.maximum(0, pos0 + first_q - window + 1)
-        e = pos0 + last_q + 1
-        seg_ids.append(np.full(r0.shape, s, dtype=np.int64))
-        rho0s.append(r0), kv_b.append(b), kv_e.append(e)
-    if not seg_ids:
+    """The tiles of ``rows_per_tile`` rows of the segments whose row count ``pick``
+    accepts: segment, first row, first and end key of each (arrays)."""
+    ql = np.asarray(seg_q_len, dtype=np.int64)
+    kl = np.asarray(seg_kv_len, dtype=np.int64)
+    rows = ql * group_size
+    chosen = np.nonzero(pick(rows) & (rows > 0))[0] if len(ql) else np.zeros(0, dtype=np.int64)
+    if len(chosen) == 0:
         z = np.zeros(0, dtype=np.int64)
         return z, z, z, z
-    return np.concatenate(seg_ids), np.concatenate(rho0s), np.concatenate(kv_b), np.concatenate(kv_e)
+    n_tiles = -(-rows[chosen] // rows_per_tile)
+    seg_ids = np.repeat(chosen, n_tiles)
+    first_tile = np.concatenate(([0], np.cumsum(n_tiles)[:-1]))
+    r0 = (np.arange(int(n_tiles.sum())) - np.repeat(first_tile, n_tiles)) * rows_per_tile
+    first_q = r0 // group_size
+    last_q = np.minimum(rows[seg_ids] - 1, r0 + rows_per_tile - 1) // group_size
+    pos0 = (kl - ql)[seg_ids]
+    b = np.zeros_like(r0) if window <= 0 else np.maximum(0, pos0 + first_q - window + 1)
+    e = pos0 + last_q + 1
+    return seg_ids, r0, b, e
 
 
 def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_seg, more_tiles=None, group=1):
@@ -201,8 +202,8 @@ def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: 
     GPU, an item's key range is cut into pieces whose partial results are merged."""
     rows_of_seg = [int(q) * group_size for q in seg_q_len]
     per_item = max(1, rows_big // ROWS_PER_ITEM)
-    small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: r <= ROWS_PER_ITEM or per_item == 1)
-    big = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: r > ROWS_PER_ITEM and per_item > 1)
+    small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: (r <= ROWS_PER_ITEM) | (per_item == 1))
+    big = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: (r > ROWS_PER_ITEM) & (per_item > 1))
     more = None
     if len(big[0]):
         *big, more = _group_tiles(*big, per_item, zigzag=window <= 0)
