@@ -60,8 +60,11 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // item writes partial slot `first partial slot + rt`.
 #define N_XCD 8
 #define WAVES 4  // per workgroup
+// Two waves per SIMD leave 256 registers each, which keeps the accumulators in VGPRs (no
+// copies to and from AGPRs around every MFMA); the largest head sizes need more.
+#define MIN_WAVES_PER_SIMD (D > 160 ? 1 : 2)
 template <int RT, bool POW2, bool PAGE32, bool SHARED, bool TILED>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(256, MIN_WAVES_PER_SIMD)
 attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
                       int out_row_stride, const int* __restrict__ items,
                       const int* __restrict__ n_items_ptr, const int* __restrict__ seg_q_start,

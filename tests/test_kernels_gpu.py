@@ -246,7 +246,7 @@ def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use, tiled=Fal
     close(out, torch.cat(want), 5e-6 if dtype == "float32" else 1.2e-2, f"attention {use}")
 
 
-SHAPES = [(4, 2, 16), (6, 2, 48), (4, 1, 32), (8, 8, 64), (32, 8, 128), (5, 5, 80), (20, 1, 16)]
+SHAPES = [(4, 2, 16), (6, 2, 48), (4, 1, 32), (8, 8, 64), (32, 8, 128), (5, 5, 80), (20, 1, 16), (4, 2, 256), (6, 3, 112), (2, 1, 160)]
 SEGS = [[(0, 1)], [(0, 70)], [(63, 1), (0, 33), (64, 64), (129, 2), (200, 1)], [(700, 1), (5, 300)]]
 
 
