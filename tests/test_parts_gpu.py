@@ -1,6 +1,7 @@
 """The parts alone, and models put together from parts as data: a windowed layer, a
-layer that runs twice, a layer that reads another layer's cache, and a toy mixer with
-state of its own that is defined here and registered without touching the framework."""
+layer that runs twice, a layer that reads another layer's cache, and toy parts that are
+defined here and registered without touching the framework: a mixer with state of its
+own, a feed-forward that routes tokens to experts, and another position encoding."""
 
 import numpy as np
 import pytest
@@ -14,7 +15,7 @@ from halite_amd.config import LayerRun, LayerSpec, ModelConfig, ModelSpec, PartS
 from halite_amd.engine.batch import Segment
 from halite_amd.engine.runner import ModelRunner
 from halite_amd.parts import MIXERS, BuildContext, Decoder, Mixer, ParamDecl, StateNeed
-from halite_amd.parts.base import FEED_FORWARDS, NORMS, POSITIONS
+from halite_amd.parts.base import FEED_FORWARDS, NORMS, POSITIONS, FeedForward, PositionEncoding
 from halite_amd.weights import fill_random
 
 pytestmark = pytest.mark.gpu
@@ -79,16 +80,19 @@ def test_norm_and_feed_forward_parts(gpu, dtype):
 # -- models from hand-written specs ---------------------------------------------------
 
 
-def toy_spec(layers: dict, order: list, d=64, vocab=97, head_dim=16, rot=16, interleaved=False, max_pos=512):
+def toy_spec(layers: dict, order: list, d=64, vocab=97, head_dim=16, rot=16, interleaved=False, max_pos=512,
+             more_positions=None, ffs=None):
     norm = PartSpec(kind="rmsnorm", size=d, eps=1e-5)
+    gated = PartSpec(kind="gated", hidden_size=d, intermediate_size=2 * d + 8, activation="silu")
+    positions = {"rope": PartSpec(kind="rope", head_dim=head_dim, rotary_dim=rot, theta=10000.0,
+                                  interleaved=interleaved, max_positions=max_pos)}
+    positions.update(more_positions or {})
     return ModelSpec(
         architecture="toy", vocab_size=vocab, hidden_size=d, max_positions=max_pos,
         embedding=PartSpec(kind="embedding", vocab_size=vocab, size=d),
-        positions={"rope": PartSpec(kind="rope", head_dim=head_dim, rotary_dim=rot, theta=10000.0,
-                                    interleaved=interleaved, max_positions=max_pos)},
+        positions=positions,
         layers={
-            name: LayerSpec(mixer_norm=norm, mixer=mixer, ff_norm=norm,
-                            ff=PartSpec(kind="gated", hidden_size=d, intermediate_size=2 * d + 8, activation="silu"))
+            name: LayerSpec(mixer_norm=norm, mixer=mixer, ff_norm=norm, ff=(ffs or {}).get(name, gated))
             for name, mixer in layers.items()
         },
         order=order, final_norm=norm, head=PartSpec(kind="linear_head", vocab_size=vocab, size=d, tied=True),
@@ -131,9 +135,16 @@ def plain_attention_layer(att, x, positions, rope_p, cached_kv=None):
     return a.reshape(n, nq) @ att.w_out.float().cpu().T, (k, v)
 
 
-def plain_model(model, ids, mixers: dict):
+def plain_gated(ff, x):
+    f = ff.p.intermediate_size
+    wgu = ff.w_gate_up.float().cpu()
+    return P.gated_feed_forward(x, wgu[:f], wgu[f:], ff.w_out.float().cpu())
+
+
+def plain_model(model, ids, mixers: dict, ffs: dict | None = None):
     """The whole toy model from plain functions; ``mixers[layer name]`` is a function
-    ``(mixer part, x, positions, run index, memo) -> delta`` ."""
+    ``(mixer part, x, positions, run index, memo) -> delta``, ``ffs[layer name]`` a
+    function ``(feed-forward part, x) -> delta`` (the gated one if none is given)."""
     spec = model.spec
     ids = torch.as_tensor(ids)
     positions = torch.arange(len(ids))
@@ -144,9 +155,7 @@ def plain_model(model, ids, mixers: dict):
         x = P.rms_norm(h, blk.mixer_norm.weight.float().cpu(), blk.mixer_norm.p.eps)
         h = h + mixers[run.layer](blk.mixer, x, positions, i, run, memo)
         x = P.rms_norm(h, blk.ff_norm.weight.float().cpu(), blk.ff_norm.p.eps)
-        f = blk.ff.p.intermediate_size
-        wgu = blk.ff.w_gate_up.float().cpu()
-        h = h + P.gated_feed_forward(x, wgu[:f], wgu[f:], blk.ff.w_out.float().cpu())
+        h = h + (ffs or {}).get(run.layer, plain_gated)(blk.ff, x)
     h = P.rms_norm(h, model.final_norm.weight.float().cpu(), model.final_norm.p.eps)
     return P.output_head(h, model.embedding.weight.float().cpu())
 
@@ -269,3 +278,126 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(gpu, dtype):
     s = runner.admit()
     assert float(runner.cache.state.tensors[0]["sum"][s].abs().sum()) == 0
     runner.free(s)
+
+
+# -- a toy feed-forward that routes, and another position encoding ------------------------
+
+
+class RoutedParams(BaseModel):
+    hidden_size: int
+    n_experts: int
+    expert_size: int
+
+
+@FEED_FORWARDS.register("toy_routed")
+class ToyRouted(FeedForward):
+    """Each token goes to the expert with the largest router logit (float32 logits and
+    softmax); the expert is ``W2 silu(W1 x)`` and its output is weighted with the
+    router's probability."""
+
+    Params = RoutedParams
+
+    def param_decls(self):
+        p = self.p
+        return {
+            "router.weight": ParamDecl((p.n_experts, p.hidden_size)),
+            "w1.weight": ParamDecl((p.n_experts, p.expert_size, p.hidden_size)),
+            "w2.weight": ParamDecl((p.n_experts, p.hidden_size, p.expert_size)),
+        }
+
+    def forward(self, x, ctx):
+        probs = torch.softmax(x.float() @ self.router_weight.float().T, dim=-1)
+        weight, expert = probs.max(dim=-1)
+        out = torch.zeros_like(x, dtype=torch.float32)
+        for e in range(self.p.n_experts):
+            rows = torch.nonzero(expert == e)[:, 0]
+            if rows.numel():
+                hid = torch.nn.functional.silu(x[rows].float() @ self.w1_weight[e].float().T)
+                out[rows] = (hid @ self.w2_weight[e].float().T) * weight[rows, None]
+        return out.to(x.dtype)
+
+
+def plain_routed(ff, x):
+    router, w1, w2 = (t.float().cpu() for t in (ff.router_weight, ff.w1_weight, ff.w2_weight))
+    out = torch.zeros_like(x)
+    for t in range(x.shape[0]):
+        probs = torch.softmax(x[t] @ router.T, dim=-1)
+        e = int(probs.argmax())
+        out[t] = probs[e] * (w2[e] @ torch.nn.functional.silu(w1[e] @ x[t]))
+    return out
+
+
+class SinusoidParams(BaseModel):
+    size: int
+    base: float
+
+
+@POSITIONS.register("toy_sinusoid")
+class ToySinusoid(PositionEncoding):
+    """Absolute positions as a vector of sines and cosines that a mixer adds to its input."""
+
+    Params = SinusoidParams
+
+    def encode(self, positions):
+        half = self.p.size // 2
+        freq = self.p.base ** (-torch.arange(half, device=positions.device, dtype=torch.float32) / half)
+        ang = positions.float()[:, None] * freq[None, :]
+        return torch.cat((torch.sin(ang), torch.cos(ang)), dim=-1)
+
+
+class AddPositionParams(BaseModel):
+    hidden_size: int
+    position: str
+
+
+@MIXERS.register("toy_add_position")
+class ToyAddPosition(Mixer):
+    """``y = W (x + encode(position))`` with the position encoding that the model's
+    specification names: no cache and no state, only the step's positions."""
+
+    Params = AddPositionParams
+
+    def __init__(self, params, build):
+        super().__init__(params, build)
+        self.position = build.positions[params.position]
+
+    def param_decls(self):
+        return {"w.weight": ParamDecl((self.p.hidden_size, self.p.hidden_size))}
+
+    def forward(self, x, ctx, run):
+        y = x.float() + self.position.encode(ctx.positions)
+        return (y @ self.w_weight.float().T).to(x.dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routing_and_other_position_encodings(gpu, dtype):
+    """One model with: attention under a second rotary encoding (other base, adjacent
+    pairs, part of the head), a mixer that uses a position encoding defined here, a
+    feed-forward with routing in one layer and the gated one in the others."""
+    rope_a = dict(rotary_dim=16, theta=10000.0, interleaved=False)
+    rope_b = dict(rotary_dim=8, theta=300.0, interleaved=True)
+    spec = toy_spec(
+        {"a": attention_spec(), "b": attention_spec(kv=1, position="rope_b"),
+         "pos": PartSpec(kind="toy_add_position", hidden_size=64, position="sin")},
+        [LayerRun(layer="a"), LayerRun(layer="pos"), LayerRun(layer="b")],
+        more_positions={
+            "rope_b": PartSpec(kind="rope", head_dim=16, rotary_dim=8, theta=300.0, interleaved=True, max_positions=512),
+            "sin": PartSpec(kind="toy_sinusoid", size=64, base=50.0),
+        },
+        ffs={"b": PartSpec(kind="toy_routed", hidden_size=64, n_experts=3, expert_size=40)},
+    )
+    runner = make_runner(gpu, spec, dtype)
+    assert isinstance(runner.model.layers["b"].ff, ToyRouted) and not isinstance(runner.model.layers["a"].ff, ToyRouted)
+
+    def att_with(rope_p):
+        return lambda part, x, positions, i, run, memo: plain_attention_layer(part, x, positions, rope_p)[0]
+
+    def add_position(part, x, positions, i, run, memo):
+        half = 32
+        ang = positions.float()[:, None] * (50.0 ** (-torch.arange(half, dtype=torch.float32) / half))[None, :]
+        return (x + torch.cat((torch.sin(ang), torch.cos(ang)), -1)) @ part.w_weight.float().cpu().T
+
+    requests = {f"r{i}": [int(t) % 97 for t in tiny.random_tokens(tiny.TINY_A, n, 120 + i)] for i, n in enumerate([50, 4, 37])}
+    mixers = {"a": att_with(rope_a), "b": att_with(rope_b), "pos": add_position}
+    ref = {rid: plain_model(runner.model, toks, mixers, {"b": plain_routed}) for rid, toks in requests.items()}
+    replay_all(runner, requests, ref, TOL[dtype], 97)
