@@ -30,7 +30,7 @@ template <int NT, int MT, bool GATED, int U>
 __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
                                    const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
                                    int ldw, void* __restrict__ C, int ldc, int out_mode, int M,
-                                   int N, int K) {
+                                   int N, int K, int slots) {
   extern __shared__ float red[];  // [waves][sets][NT*MT][64][4]
   const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
   const int n_waves = blockDim.x / HAL_WAVE;
@@ -112,16 +112,44 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   }
 
   // every wave's partial sums -> LDS; then each output element is the sum over the
-  // waves in wave order (deterministic)
+  // waves in wave order (deterministic).  `slots` < n_waves (half of them) means that
+  // LDS holds only that many partial tiles: the upper half of the waves hands its
+  // sums to the lower half first (wave w + slots to wave w, same lanes).
   constexpr int TILE = SETS * NT * MT * 256;
-  float* mine = red + (size_t)wave * TILE;
+  if (slots < n_waves) {
+    if (wave >= slots) {
+      float* theirs = red + (size_t)(wave - slots) * TILE;
 #pragma unroll
-  for (int s = 0; s < SETS; ++s)
+      for (int s = 0; s < SETS; ++s)
 #pragma unroll
-    for (int f = 0; f < NT; ++f)
+        for (int f = 0; f < NT; ++f)
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-        *(f32x4*)(mine + ((s * NT + f) * MT + t) * 256 + lane * 4) = acc[s][f][t];
+          for (int t = 0; t < MT; ++t)
+            *(f32x4*)(theirs + ((s * NT + f) * MT + t) * 256 + lane * 4) = acc[s][f][t];
+    }
+    __syncthreads();
+    if (wave < slots) {
+      const float* from = red + (size_t)wave * TILE;
+#pragma unroll
+      for (int s = 0; s < SETS; ++s)
+#pragma unroll
+        for (int f = 0; f < NT; ++f)
+#pragma unroll
+          for (int t = 0; t < MT; ++t)
+            acc[s][f][t] += *(const f32x4*)(from + ((s * NT + f) * MT + t) * 256 + lane * 4);
+    }
+    __syncthreads();
+  }
+  if (wave < slots) {
+    float* mine = red + (size_t)wave * TILE;
+#pragma unroll
+    for (int s = 0; s < SETS; ++s)
+#pragma unroll
+      for (int f = 0; f < NT; ++f)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          *(f32x4*)(mine + ((s * NT + f) * MT + t) * 256 + lane * 4) = acc[s][f][t];
+  }
   __syncthreads();
 
   // element (f, t, lane, i) of the accumulator tile is row n_base + f*16 + (lane/16)*4 + i
@@ -133,7 +161,7 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
     const int m = t * 16 + ln % 16;
     if (n >= N || m >= M) continue;
     float v = 0.f, v2 = 0.f;
-    for (int w = 0; w < n_waves; ++w) {
+    for (int w = 0; w < slots; ++w) {
       v += red[(size_t)w * TILE + idx];
       if (GATED) v2 += red[(size_t)w * TILE + NT * MT * 256 + idx];
     }
@@ -153,11 +181,14 @@ static int launch_skinny(const bf16_t* X, int ldx, const bf16_t* W, const bf16_t
                          void* C, int ldc, int out_mode, int M, int N, int K, int waves,
                          hipStream_t stream) {
   constexpr int SETS = GATED ? 2 : 1;
-  const size_t smem = (size_t)waves * SETS * NT * MT * 256 * sizeof(float);
+  // LDS for the partial sums of all waves, or of half of them if that is too much
+  const size_t per_wave = (size_t)SETS * NT * MT * 256 * sizeof(float);
+  const int slots = (size_t)waves * per_wave > 64 * 1024 ? waves / 2 : waves;
+  const size_t smem = (size_t)slots * per_wave;
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
   hipLaunchKernelGGL((skinny_gemm_kernel<NT, MT, GATED, U>), dim3(blocks),
                      dim3(waves * HAL_WAVE), smem, stream, X, ldx, W, W2, ldw, C, ldc, out_mode,
-                     M, N, K);
+                     M, N, K, slots);
   HAL_LAUNCH_CHECK();
   return 0;
 }
@@ -184,21 +215,20 @@ extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const
   // Rows of W per wave (16 * nt): more of them mean that a fragment of X, which every
   // block reads again, serves more of W.  The waves of a block split K, more of them
   // when there are few blocks.  Tunable through the environment for measurements.
-  int nt = mt >= 3 ? 4 : mt;
+  int nt = mt >= 3 ? 2 : mt;
   int u = 0, waves = 0;
   if (const char* e = getenv("HAL_SKINNY_NT")) nt = atoi(e);
   if (const char* e = getenv("HAL_SKINNY_U")) u = atoi(e);
   if (const char* e = getenv("HAL_SKINNY_WAVES")) waves = atoi(e);
-  if (nt != 1 && nt != 2 && nt != 4) nt = 4;
-  if (mt >= 3 && nt < 4) nt = 4;
-  if (mt == 2 && nt < 2) nt = 2;
+  if (nt != 1 && nt != 2 && nt != 4) nt = 2;
+  if (mt >= 2 && nt < 2) nt = 2;
   const int blocks = (N + 16 * nt - 1) / (16 * nt);
   const int steps = (K + 31) / 32;
   if (waves <= 0) {
     waves = 4;
     while (waves < 16 && blocks * waves < 4096 && steps / (waves * 2) >= 4) waves *= 2;
   }
-  while (waves > 1 && (size_t)waves * sets * nt * mt * 1024 > 64 * 1024) waves /= 2;
+  while (waves > 1 && (size_t)waves * sets * nt * mt * 1024 > 2 * 64 * 1024) waves /= 2;
   // loads in flight per wave: about 16 fragments of 16 bytes
   if (u <= 0) u = 8 / (sets * nt);
   u = u >= 8 ? 8 : (u >= 4 ? 4 : (u >= 2 ? 2 : 1));
@@ -223,6 +253,8 @@ extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const
   SK_CASE(4, 1)
   SK_CASE(2, 2)
   SK_CASE(4, 2)
+  SK_CASE(2, 3)
+  SK_CASE(2, 4)
   SK_CASE(4, 3)
   SK_CASE(4, 4)
 #undef SK_LAUNCH
