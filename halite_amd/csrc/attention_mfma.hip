@@ -466,81 +466,93 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 
 // merge item: {segment, first row (of 16), first partial slot, number of partials,
 // slots from one partial to the next, 0, 0, 0}
-// One block per (merge item, kv head); a wave owns a row at a time, a lane two
-// dimensions.  The weights exp2(m_i - max) of up to 64 partials are computed one per
-// lane and handed round with shuffles, so that the loads of the partial sums do not
-// wait for one another.
+// One block per (merge item, kv head, row of the tile).  The four waves take every
+// fourth partial each, four loads in flight at a time, a lane two dimensions; their sums
+// are added in wave order through LDS (deterministic).
 __global__ void __launch_bounds__(256)
 attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
                        const int* __restrict__ merges, const int* __restrict__ n_merges_ptr,
                        const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                        const float* __restrict__ part_o, const float* __restrict__ part_ml, int H,
                        int K) {
+  constexpr int NC = (D + 127) / 128;  // a lane's pairs of dimensions
+  constexpr int MW = 4;                // waves
+  __shared__ float red_o[MW][NC * 128];
+  __shared__ float red_l[MW];
+  __shared__ float scratch[16];
   const int mi = blockIdx.x;
   if (mi >= *n_merges_ptr) return;
-  const int g = blockIdx.y;
+  const int g = blockIdx.y, row = blockIdx.z;
   const int G = H / K;
   const int* mg = merges + (size_t)mi * ITEM_INTS;
   const int seg = mg[0], rho0 = mg[1], first = mg[2], n = mg[3], stride = mg[4];
   const int q_start = seg_q_start[seg], q_len = seg_q_len[seg];
+  const int rho = rho0 + row;
+  if (rho >= q_len * G) return;  // the whole block
   const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
-  const int n_waves = blockDim.x / HAL_WAVE;
-  for (int row = wave; row < 16; row += n_waves) {
-    const int rho = rho0 + row;
-    if (rho >= q_len * G) break;  // rows are in order: the rest are invalid too
-    // the largest running maximum of the row
-    float m_all = -INFINITY;
-    for (int i = lane; i < n; i += HAL_WAVE)
-      m_all = fmaxf(m_all, part_ml[(((size_t)(first + i * stride) * K + g) * 16 + row) * 2]);
-    m_all = wave_max(m_all);
-    float acc[D / 128 + 1][2];
+  auto slot_row = [&](int i) { return ((size_t)(first + i * stride) * K + g) * 16 + row; };
+
+  // the largest running maximum of the row
+  float m_all = -INFINITY;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) m_all = fmaxf(m_all, part_ml[slot_row(i) * 2]);
+  m_all = block_max(m_all, scratch);
+
+  float acc[NC][2];
 #pragma unroll
-    for (int c = 0; c < D / 128 + 1; ++c) acc[c][0] = acc[c][1] = 0.f;
-    float l_all = 0.f;
-    for (int i0 = 0; i0 < n; i0 += HAL_WAVE) {
-      float w = 0.f;
-      if (i0 + lane < n) {
-        const size_t base = ((size_t)(first + (i0 + lane) * stride) * K + g) * 16 + row;
-        const float mi_ = part_ml[base * 2], li = part_ml[base * 2 + 1];
-        w = (mi_ == -INFINITY) ? 0.f : exp2f(mi_ - m_all);
-        l_all += w * li;
-      }
-      const int cnt = n - i0 < HAL_WAVE ? n - i0 : HAL_WAVE;
-      // four partials at a time: their loads are issued together
-      for (int i = 0; i < cnt; i += 4) {
-        float wi[4];
-        const float* po[4];
+  for (int c = 0; c < NC; ++c) acc[c][0] = acc[c][1] = 0.f;
+  float l_all = 0.f;
+  for (int i0 = wave; i0 < n; i0 += MW * 4) {
+    float w[4], li[4];
+    float2 v[4][NC];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int iu = i + u < cnt ? i + u : cnt - 1;
-          wi[u] = i + u < cnt ? __shfl(w, iu, HAL_WAVE) : 0.f;
-          po[u] = part_o + (((size_t)(first + (i0 + iu) * stride) * K + g) * 16 + row) * D;
-        }
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * MW;
+      const bool ok = i < n;
+      const size_t base = slot_row(ok ? i : i0);
+      const float2 ml = *(const float2*)(part_ml + base * 2);
+      w[u] = (!ok || ml.x == -INFINITY) ? 0.f : exp2f(ml.x - m_all);
+      li[u] = ml.y;
 #pragma unroll
-        for (int c = 0; c < D / 128 + 1; ++c) {
-          const int d = c * 128 + lane * 2;
-          if (d < D) {
-            float2 v[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = *(const float2*)(po[u] + d);
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-              acc[c][0] += wi[u] * v[u].x;
-              acc[c][1] += wi[u] * v[u].y;
-            }
-          }
-        }
+      for (int c = 0; c < NC; ++c) {
+        const int d = c * 128 + lane * 2;
+        v[u][c] = d < D ? *(const float2*)(part_o + base * D + d) : float2{0.f, 0.f};
       }
     }
-    l_all = wave_sum(l_all);
-    const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
-    const int qi = rho / G, head = g * G + rho % G;
-    bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
 #pragma unroll
-    for (int c = 0; c < D / 128 + 1; ++c) {
-      const int d = c * 128 + lane * 2;
-      if (d < D) *(uint32_t*)(op + d) = pack2(acc[c][0] * inv, acc[c][1] * inv);
+    for (int u = 0; u < 4; ++u) {
+      l_all += w[u] * li[u];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        acc[c][0] += w[u] * v[u][c].x;
+        acc[c][1] += w[u] * v[u][c].y;
+      }
     }
+  }
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    red_o[wave][c * 128 + lane * 2] = acc[c][0];
+    red_o[wave][c * 128 + lane * 2 + 1] = acc[c][1];
+  }
+  if (lane == 0) red_l[wave] = l_all;
+  __syncthreads();
+  if (wave != 0) return;
+  float l_sum = 0.f;
+#pragma unroll
+  for (int w = 0; w < MW; ++w) l_sum += red_l[w];
+  const float inv = l_sum > 0.f ? 1.0f / l_sum : 0.f;
+  const int qi = rho / G, head = g * G + rho % G;
+  bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int d = c * 128 + lane * 2;
+    if (d >= D) continue;
+    float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+    for (int w = 0; w < MW; ++w) {
+      o0 += red_o[w][d];
+      o1 += red_o[w][d + 1];
+    }
+    *(uint32_t*)(op + d) = pack2(o0 * inv, o1 * inv);
   }
 }
 
@@ -606,7 +618,7 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, true, big_items, max_big, counts + 1)
 #undef LAUNCH_ATTENTION
   if (max_merges > 0) {
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K), dim3(256), 0, stream,
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K, 16), dim3(256), 0, stream,
                        (bf16_t*)out, out_row_stride, merges, counts + 2, seg_q_start, seg_q_len,
                        part_o, part_ml, H, K);
     HAL_LAUNCH_CHECK();
