@@ -112,13 +112,13 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   }
 
   // every wave's partial sums -> LDS; then each output element is the sum over the
-  // waves in wave order (deterministic).  `slots` < n_waves (half of them) means that
-  // LDS holds only that many partial tiles: the upper half of the waves hands its
-  // sums to the lower half first (wave w + slots to wave w, same lanes).
+  // waves in wave order (deterministic).  `slots` < n_waves means that LDS holds only
+  // that many partial tiles: in rounds, the next `slots` waves hand their sums to the
+  // first `slots` waves (wave w + r*slots to wave w, same lanes) before those write.
   constexpr int TILE = SETS * NT * MT * 256;
-  if (slots < n_waves) {
-    if (wave >= slots) {
-      float* theirs = red + (size_t)(wave - slots) * TILE;
+  for (int base = slots; base < n_waves; base += slots) {
+    if (wave >= base && wave < base + slots) {
+      float* theirs = red + (size_t)(wave - base) * TILE;
 #pragma unroll
       for (int s = 0; s < SETS; ++s)
 #pragma unroll
@@ -128,7 +128,7 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
             *(f32x4*)(theirs + ((s * NT + f) * MT + t) * 256 + lane * 4) = acc[s][f][t];
     }
     __syncthreads();
-    if (wave < slots) {
+    if (wave < slots && wave + base < n_waves) {
       const float* from = red + (size_t)wave * TILE;
 #pragma unroll
       for (int s = 0; s < SETS; ++s)
@@ -181,9 +181,10 @@ static int launch_skinny(const bf16_t* X, int ldx, const bf16_t* W, const bf16_t
                          void* C, int ldc, int out_mode, int M, int N, int K, int waves,
                          hipStream_t stream) {
   constexpr int SETS = GATED ? 2 : 1;
-  // LDS for the partial sums of all waves, or of half of them if that is too much
+  // LDS for the partial sums of all waves, or of a half, a quarter ... if that is too much
   const size_t per_wave = (size_t)SETS * NT * MT * 256 * sizeof(float);
-  const int slots = (size_t)waves * per_wave > 64 * 1024 ? waves / 2 : waves;
+  int slots = waves;
+  while (slots > 1 && (size_t)slots * per_wave > 64 * 1024) slots /= 2;
   const size_t smem = (size_t)slots * per_wave;
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
   hipLaunchKernelGGL((skinny_gemm_kernel<NT, MT, GATED, U>), dim3(blocks),
@@ -228,7 +229,7 @@ extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const
     waves = 4;
     while (waves < 16 && blocks * waves < 4096 && steps / (waves * 2) >= 4) waves *= 2;
   }
-  while (waves > 1 && (size_t)waves * sets * nt * mt * 1024 > 2 * 64 * 1024) waves /= 2;
+  while (waves > 1 && (size_t)sets * nt * mt * 1024 > 64 * 1024) waves /= 2;  // one tile must fit
   // loads in flight per wave: about 16 fragments of 16 bytes
   if (u <= 0) u = 8 / (sets * nt);
   u = u >= 8 ? 8 : (u >= 4 ? 4 : (u >= 2 ? 2 : 1));

@@ -44,7 +44,8 @@ int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const void* W2, 
 
 int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temperature,
                const int* top_k, const float* top_p, const float* min_p, const uint64_t* seeds,
-               const int* draw_index, int* out_token, float* out_logprob, hipStream_t stream);
+               const int* draw_index, int* out_token, float* out_logprob, uint32_t* key_rows,
+               hipStream_t stream);
 
 // ---- the head-size-specific library (attention_mfma.hip) ---------------------------------
 int hal_attention_mfma_head_dim();

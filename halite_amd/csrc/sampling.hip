@@ -12,6 +12,7 @@
 #include "hal_api.h"
 
 #define SAMPLE_THREADS 1024
+#define SAMPLE_BINS 2048  // two per thread
 
 __device__ __forceinline__ float clean_logit(float x) { return x != x ? -1e5f : x; }
 
@@ -19,6 +20,11 @@ __device__ __forceinline__ float clean_logit(float x) { return x != x ? -1e5f : 
 __device__ __forceinline__ uint32_t sort_key(float x) {
   const uint32_t u = __float_as_uint(x);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// the float that a key stands for
+__device__ __forceinline__ float key_value(uint32_t key) {
+  return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
 }
 
 __device__ __forceinline__ float uniform_draw(uint64_t seed, uint32_t index) {
@@ -29,6 +35,27 @@ __device__ __forceinline__ float uniform_draw(uint64_t seed, uint32_t index) {
   x *= 0x94D049BB133111EBull;
   x ^= x >> 31;
   return (float)(x >> 40) * (1.0f / 16777216.0f);
+}
+
+// Sum of `v` over the threads after this one (exclusive), for a block of SAMPLE_THREADS
+// threads; `tmp` holds one entry per wave.  Ends with a barrier, so `tmp` can be used
+// again at once.
+__device__ __forceinline__ unsigned long long block_suffix_u64(unsigned long long v,
+                                                               unsigned long long* tmp) {
+  const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
+  unsigned long long inc = v;
+#pragma unroll
+  for (int off = 1; off < HAL_WAVE; off <<= 1) {
+    const uint32_t lo = __shfl_down((uint32_t)inc, off, HAL_WAVE);
+    const uint32_t hi = __shfl_down((uint32_t)(inc >> 32), off, HAL_WAVE);
+    if (lane + off < HAL_WAVE) inc += ((unsigned long long)hi << 32) | lo;
+  }
+  if (lane == 0) tmp[wave] = inc;
+  __syncthreads();
+  unsigned long long after = 0ull;
+  for (int w = wave + 1; w < SAMPLE_THREADS / HAL_WAVE; ++w) after += tmp[w];
+  __syncthreads();
+  return inc - v + after;
 }
 
 struct ArgMax {
@@ -46,13 +73,19 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
               const float* __restrict__ temperature, const int* __restrict__ top_k,
               const float* __restrict__ top_p, const float* __restrict__ min_p,
               const uint64_t* __restrict__ seeds, const int* __restrict__ draw_index,
-              int* __restrict__ out_token, float* __restrict__ out_logprob) {
+              int* __restrict__ out_token, float* __restrict__ out_logprob,
+              uint32_t* __restrict__ key_rows) {
   __shared__ float red[16];
   __shared__ float red2[16];
   __shared__ ArgMax amax_s[16];
-  __shared__ float chunk_sum[SAMPLE_THREADS];
   __shared__ int chosen_thread;
   __shared__ int last_thread;
+  __shared__ unsigned long long hist[2][SAMPLE_BINS];
+  __shared__ unsigned long long scan_tmp[SAMPLE_THREADS / HAL_WAVE];
+  __shared__ unsigned long long whole_mass;
+  __shared__ unsigned long long found_above[2];
+  __shared__ uint32_t found_bin[2];
+  __shared__ int found_any[2];
 
   const int row = blockIdx.x, tid = threadIdx.x;
   const int lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
@@ -67,6 +100,9 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
   // softmax's denominator); four logits per load where the row allows it.
   ArgMax am = {-INFINITY, 0x7fffffff};
   float part = 0.f;
+  // the keys of the row (order-preserving integers of z) are kept for the later passes
+  uint32_t* keys = (key_rows && !greedy) ? key_rows + (size_t)row * V : nullptr;
+  auto key_of = [&](float xv) { return sort_key(clean_logit(xv) / inv_scale); };
   auto take = [&](float xv, int i) {
     const float z = clean_logit(xv) / inv_scale;
     if (z > am.v) {
@@ -79,14 +115,26 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
   };
   if (ld % 4 == 0 && ((uintptr_t)logits % 16) == 0) {
     const int n4 = V / 4;
+    const bool keys4 = keys && V % 4 == 0;  // rows of keys start on 16 bytes then
 #pragma unroll 4
     for (int v = tid; v < n4; v += SAMPLE_THREADS) {
       const float4 q = *(const float4*)(x + 4 * v);
       take(q.x, 4 * v), take(q.y, 4 * v + 1), take(q.z, 4 * v + 2), take(q.w, 4 * v + 3);
+      if (keys4)
+        *(uint4*)(keys + 4 * v) = make_uint4(key_of(q.x), key_of(q.y), key_of(q.z), key_of(q.w));
+      else if (keys)
+        keys[4 * v] = key_of(q.x), keys[4 * v + 1] = key_of(q.y), keys[4 * v + 2] = key_of(q.z),
+                 keys[4 * v + 3] = key_of(q.w);
     }
-    for (int i = 4 * n4 + tid; i < V; i += SAMPLE_THREADS) take(x[i], i);
+    for (int i = 4 * n4 + tid; i < V; i += SAMPLE_THREADS) {
+      take(x[i], i);
+      if (keys) keys[i] = key_of(x[i]);
+    }
   } else {
-    for (int i = tid; i < V; i += SAMPLE_THREADS) take(x[i], i);
+    for (int i = tid; i < V; i += SAMPLE_THREADS) {
+      take(x[i], i);
+      if (keys) keys[i] = key_of(x[i]);
+    }
   }
   // combine the threads: the block's maximum, then the sums rescaled to it
   ArgMax mine_am = am;
@@ -114,127 +162,197 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
   }
 
   // ---- filters: the kept set is { key(z_i) >= key_min } and exp(z_i - m) >= min_p --
+  // Both thresholds are the key at which a sum over the tokens in descending order of
+  // their keys first reaches a target: the number of tokens reaches k (top-k), the mass
+  // reaches top_p of the reference mass (top-p).  That key is found digit by digit
+  // (11 + 11 + 10 bits) from histograms over the tokens that share the digits found so
+  // far: three passes over the row instead of one per bit.  Masses are summed as
+  // integers (2^-40 of the largest token's), so the sums do not depend on their order.
+  auto key_at = [&](int i) { return keys ? keys[i] : sort_key(clean_logit(x[i]) / inv_scale); };
   const float tp = top_p[row];
   const float mp = min_p[row];
+  const bool want_k = k > 0 && k < V, want_p = tp < 1.f;
   uint32_t key_min = 0;
-  float ref_mass = total;
-  if (k > 0 && k < V) {
-    // smallest key with fewer than k elements strictly above it
-    uint32_t lo = 0, hi = 0xffffffffu;  // predicate false below the answer, true at hi
-    while (lo < hi) {
-      const uint32_t mid = lo + (hi - lo) / 2;
-      float cnt = 0.f;
-      for (int i = tid; i < V; i += SAMPLE_THREADS) {
-        const float z = clean_logit(x[i]) / inv_scale;
-        if (sort_key(z) > mid) cnt += 1.f;
+  if (want_k || want_p) {
+    auto fixed = [&](uint32_t key) {
+      return (unsigned long long)(expf(key_value(key) - m) * 1099511627776.0f);
+    };
+    // one search: the digits found so far, the sum over all keys above them, the target
+    uint32_t prefix[2] = {0u, 0u};
+    unsigned long long above[2] = {0ull, 0ull}, target[2] = {(unsigned long long)(k > 0 ? k : 0), 0ull};
+    auto descend = [&](bool on_k, bool on_p) {
+      const bool on[2] = {on_k, on_p};
+      prefix[0] = on_k ? 0u : prefix[0], prefix[1] = on_p ? 0u : prefix[1];
+      above[0] = on_k ? 0ull : above[0], above[1] = on_p ? 0ull : above[1];
+#pragma unroll 1
+      for (int level = 0; level < 3; ++level) {
+        const int shift = level == 0 ? 21 : (level == 1 ? 10 : 0);
+        const int up = level == 0 ? 32 : (level == 1 ? 21 : 10);  // bits below `up` are open
+        for (int b = tid; b < 2 * SAMPLE_BINS; b += SAMPLE_THREADS) (&hist[0][0])[b] = 0ull;
+        __syncthreads();
+        for (int i = tid; i < V; i += SAMPLE_THREADS) {
+          const uint32_t key = key_at(i);
+          const uint32_t high = level == 0 ? 0u : key >> up;
+          const uint32_t bin = (key >> shift) & (SAMPLE_BINS - 1) & ((1u << (up - shift)) - 1u);
+          if (on[0] && high == prefix[0]) atomicAdd(&hist[0][bin], 1ull);
+          if (on[1] && high == prefix[1]) atomicAdd(&hist[1][bin], fixed(key));
+        }
+        __syncthreads();
+        if (level == 0 && on[1]) {
+          // the whole mass, as the histogram has it: the reference of top-p unless the
+          // caller has set another
+          unsigned long long all = hist[1][2 * tid] + hist[1][2 * tid + 1];
+          all += block_suffix_u64(all, scan_tmp);
+          if (tid == 0) whole_mass = all;
+          __syncthreads();
+          if (target[1] == ~0ull) {
+            const double t = (double)tp * (double)whole_mass;
+            target[1] = (unsigned long long)t;
+          }
+        }
+#pragma unroll
+        for (int sidx = 0; sidx < 2; ++sidx) {
+          if (!on[sidx]) continue;
+          // bins in descending order: thread t has bins 2t+1 and 2t
+          const unsigned long long h1 = hist[sidx][2 * tid + 1], h0 = hist[sidx][2 * tid];
+          const unsigned long long higher = above[sidx] + block_suffix_u64(h1 + h0, scan_tmp);
+          if (tid == 0) found_bin[sidx] = 0u, found_above[sidx] = above[sidx] + 0ull, found_any[sidx] = 0;
+          __syncthreads();
+          if (higher < target[sidx] && higher + h1 >= target[sidx]) {
+            found_bin[sidx] = 2 * tid + 1, found_above[sidx] = higher, found_any[sidx] = 1;
+          } else if (higher + h1 < target[sidx] && higher + h1 + h0 >= target[sidx]) {
+            found_bin[sidx] = 2 * tid, found_above[sidx] = higher + h1, found_any[sidx] = 1;
+          }
+          __syncthreads();
+          // a target of zero, or one beyond the whole sum, is met by no bin: the first
+          // keeps the largest key only, the second every key
+          if (!found_any[sidx]) {
+            if (target[sidx] == 0ull) {
+              int top = -1;
+              if (h1 != 0ull) top = 2 * tid + 1; else if (h0 != 0ull) top = 2 * tid;
+              if (top >= 0) atomicMax(&found_bin[sidx], (uint32_t)top);
+            }
+            __syncthreads();
+          }
+          prefix[sidx] = (prefix[sidx] << (up - shift)) | found_bin[sidx];
+          above[sidx] = found_above[sidx];
+          __syncthreads();
+        }
       }
-      cnt = block_sum(cnt, red);
-      if (cnt < (float)k) hi = mid; else lo = mid + 1;
-    }
-    key_min = lo;
-    if (mp > 0.f) {
-      // with min_p the reference renormalises after top-k, so top-p refers to
-      // the mass that top-k kept
-      float kept = 0.f;
+    };
+    const bool p_after_k = want_k && want_p && mp > 0.f;  // top-p refers to what top-k kept
+    target[1] = ~0ull;                                    // top_p of the whole mass
+    if (!p_after_k) {
+      descend(want_k, want_p);
+      if (want_k) key_min = prefix[0];
+      if (want_p && prefix[1] > key_min) key_min = prefix[1];
+    } else {
+      descend(true, false);
+      key_min = prefix[0];
+      // with min_p the reference renormalises after top-k, so top-p refers to the
+      // mass that top-k kept
+      unsigned long long kept = 0ull;
       for (int i = tid; i < V; i += SAMPLE_THREADS) {
-        const float z = clean_logit(x[i]) / inv_scale;
-        if (sort_key(z) >= key_min) kept += expf(z - m);
+        const uint32_t key = key_at(i);
+        if (key >= key_min) kept += fixed(key);
       }
-      ref_mass = block_sum(kept, red);
+      kept += block_suffix_u64(kept, scan_tmp);
+      if (tid == 0) whole_mass = kept;
+      __syncthreads();
+      target[1] = (unsigned long long)((double)tp * (double)whole_mass);
+      __syncthreads();
+      descend(false, true);
+      if (prefix[1] > key_min) key_min = prefix[1];
     }
-  }
-  if (tp < 1.f) {
-    // smallest key such that the elements strictly above it hold < top_p of the mass
-    const float thr = tp * ref_mass;
-    uint32_t lo = 0, hi = 0xffffffffu;
-    while (lo < hi) {
-      const uint32_t mid = lo + (hi - lo) / 2;
-      float mass = 0.f;
-      for (int i = tid; i < V; i += SAMPLE_THREADS) {
-        const float z = clean_logit(x[i]) / inv_scale;
-        if (sort_key(z) > mid) mass += expf(z - m);
-      }
-      mass = block_sum(mass, red2);
-      if (mass < thr) hi = mid; else lo = mid + 1;
-    }
-    if (lo > key_min) key_min = lo;
   }
 
   // ---- inverse CDF over the kept tokens in index order -----------------------------
-  // A thread owns a contiguous run of tokens; a block-wide prefix sum of the runs'
-  // kept mass finds the run that holds the target, and its thread walks it.
-  const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-  const int begin = tid * chunk;
-  const int end = begin + chunk < V ? begin + chunk : V;
-  float mine = 0.f;
-#pragma unroll 4
-  for (int i = begin; i < end; ++i) {
-    const float z = clean_logit(x[i]) / inv_scale;
+  // A wave owns a contiguous run of tokens and reads it 64 tokens at a time; a prefix
+  // sum over the waves' kept masses finds the wave that holds the target, and that wave
+  // walks its run again with a prefix sum over each 64 tokens.
+  const int n_waves = SAMPLE_THREADS / HAL_WAVE;
+  const int run_len = ((V + n_waves - 1) / n_waves + HAL_WAVE - 1) / HAL_WAVE * HAL_WAVE;
+  const int begin = wave * run_len;
+  const int end = begin + run_len < V ? begin + run_len : V;
+  auto kept_mass_of = [&](int i, float& z) {
+    if (i >= end) return 0.f;
+    const uint32_t key = key_at(i);
+    if (key < key_min) return 0.f;
+    z = key_value(key);
     const float e = expf(z - m);
-    if (sort_key(z) >= key_min && e >= mp) mine += e;
-  }
-  float incl = mine;
-#pragma unroll
-  for (int off = 1; off < HAL_WAVE; off <<= 1) {
-    const float up = __shfl_up(incl, off, HAL_WAVE);
-    if (lane >= off) incl += up;
-  }
+    return e >= mp ? e : 0.f;
+  };
+  float mine = 0.f, zz;
+  for (int i = begin + lane; i < end; i += HAL_WAVE) mine += kept_mass_of(i, zz);
+  const float wave_mass = wave_sum(mine);
   if (tid == 0) {
     chosen_thread = 0x7fffffff;
     last_thread = -1;
   }
-  if (lane == HAL_WAVE - 1) red2[wave] = incl;
+  if (lane == 0) red2[wave] = wave_mass;
   __syncthreads();
-  float before = incl - mine, kept_mass = 0.f;
-  for (int w = 0; w < SAMPLE_THREADS / HAL_WAVE; ++w) {
+  float before = 0.f, kept_mass = 0.f;
+  for (int w = 0; w < n_waves; ++w) {
     if (w < wave) before += red2[w];
     kept_mass += red2[w];
   }
   const float target = uniform_draw(seeds[row], (uint32_t)draw_index[row]) * kept_mass;
-  if (mine > 0.f) {
-    atomicMax(&last_thread, tid);
-    if (before + mine > target) atomicMin(&chosen_thread, tid);
+  if (lane == 0 && wave_mass > 0.f) {
+    atomicMax(&last_thread, wave);
+    if (before + wave_mass > target) atomicMin(&chosen_thread, wave);
   }
   __syncthreads();
   int pick = chosen_thread;
   if (pick == 0x7fffffff) pick = last_thread;  // rounding left the target at the very end
-  const float chosen_before = before;
-  if (tid == pick) {
-    float run = chosen_before;
-    int tok = -1, last_kept = -1;
-    float z_tok = 0.f, z_last = 0.f;
-    for (int i = begin; i < end; ++i) {
-      const float z = clean_logit(x[i]) / inv_scale;
-      const float e = expf(z - m);
-      if (sort_key(z) >= key_min && e >= mp) {
-        run += e;
-        last_kept = i;
-        z_last = z;
-        if (run > target) {
-          tok = i;
-          z_tok = z;
-          break;
-        }
-      }
+  if (wave != pick) return;
+  float run = before;
+  int tok = -1, last_kept = -1;
+  float z_tok = 0.f, z_last = 0.f;
+  for (int i0 = begin; i0 < end && tok < 0; i0 += HAL_WAVE) {
+    float z = 0.f;
+    const float e = kept_mass_of(i0 + lane, z);
+    float incl = e;
+#pragma unroll
+    for (int off = 1; off < HAL_WAVE; off <<= 1) {
+      const float up = __shfl_up(incl, off, HAL_WAVE);
+      if (lane >= off) incl += up;
     }
-    if (tok < 0) {
-      tok = last_kept;
-      z_tok = z_last;
+    const unsigned long long kept_lanes = __builtin_amdgcn_ballot_w64(e > 0.f);
+    const unsigned long long hit = __builtin_amdgcn_ballot_w64(e > 0.f && run + incl > target);
+    if (kept_lanes) {
+      const int hi = 63 - __builtin_clzll(kept_lanes);
+      last_kept = i0 + hi;
+      z_last = __shfl(z, hi, HAL_WAVE);
     }
+    if (hit) {
+      const int lo = __builtin_ctzll(hit);
+      tok = i0 + lo;
+      z_tok = __shfl(z, lo, HAL_WAVE);
+    }
+    run += __shfl(incl, HAL_WAVE - 1, HAL_WAVE);
+  }
+  if (tok < 0) {
+    tok = last_kept;
+    z_tok = z_last;
+  }
+  if (lane == 0) {
     out_token[row] = tok;
     out_logprob[row] = z_tok - m - logf(total);
   }
 }
 
+// `key_rows`: room for n_rows * V 32-bit words that the kernel may use between its
+// passes, or null (every pass then derives the keys from the logits again).
 extern "C" int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temperature,
                           const int* top_k, const float* top_p, const float* min_p,
                           const uint64_t* seeds, const int* draw_index, int* out_token,
-                          float* out_logprob, hipStream_t stream) {
+                          float* out_logprob, uint32_t* key_rows, hipStream_t stream) {
   HAL_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "hal_sample: bad sizes rows=%d V=%d ld=%d", n_rows,
               V, ld);
   if (n_rows == 0) return 0;
   hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, ld, V,
-                     temperature, top_k, top_p, min_p, seeds, draw_index, out_token, out_logprob);
+                     temperature, top_k, top_p, min_p, seeds, draw_index, out_token, out_logprob,
+                     key_rows);
   HAL_LAUNCH_CHECK();
   return 0;
 }

@@ -243,8 +243,11 @@ def sample(
     min_p: torch.Tensor,
     seeds: torch.Tensor,
     draw_index: torch.Tensor,
+    all_greedy: bool = False,
 ):
-    """Next token and log-probability of every row of float32 ``logits``."""
+    """Next token and log-probability of every row of float32 ``logits``.  Unless
+    ``all_greedy`` says that no row samples, the kernel gets room for one 32-bit key per
+    logit, which its passes over a row then read instead of deriving it again."""
     lib = library.core_library()
     _dev(logits, temperature, top_k, top_p, min_p, seeds, draw_index)
     n, vocab = logits.shape
@@ -256,11 +259,12 @@ def sample(
         _need(t.numel() == n, "sample: one parameter per row")
     tokens = torch.empty(n, dtype=torch.int32, device=logits.device)
     logprobs = torch.empty(n, dtype=torch.float32, device=logits.device)
+    keys = None if all_greedy else torch.empty((n, vocab), dtype=torch.int32, device=logits.device)
     _check(
         lib,
         lib.hal_sample(
             _ptr(logits), vocab, n, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(min_p),
-            _ptr(seeds), _ptr(draw_index), _ptr(tokens), _ptr(logprobs), _stream(),
+            _ptr(seeds), _ptr(draw_index), _ptr(tokens), _ptr(logprobs), _ptr(keys), _stream(),
         ),
     )
     return tokens, logprobs

@@ -29,8 +29,27 @@ class Sampler:
     sampled before); it returns int32 tokens and float32 log-probabilities on the
     device.  NaN logits count as -1e5 (sampler.py:21-26)."""
 
+    RING = 4  # pinned staging buffers in turn; one is reused only after its copy is done
+
     def __init__(self, device):
         self.device = torch.device(device)
+        self._staging: list[tuple[torch.Tensor, torch.cuda.Event | None]] = []
+        self._turn = 0
+
+    def _stage(self, words: int) -> torch.Tensor:
+        """A pinned int32 buffer of at least ``words`` entries whose last copy has finished."""
+        if len(self._staging) < self.RING:
+            self._staging.append((torch.empty(max(words, 1024), dtype=torch.int32, pin_memory=True), None))
+            self._turn = len(self._staging) - 1
+        else:
+            self._turn = (self._turn + 1) % self.RING
+        buf, event = self._staging[self._turn]
+        if event is not None:
+            event.synchronize()
+        if buf.numel() < words:
+            buf = torch.empty(2 * words, dtype=torch.int32, pin_memory=True)
+        self._staging[self._turn] = (buf, None)
+        return buf
 
     def forward(self, logits: torch.Tensor, params: list[SamplingParams], seeds: list[int], draw_index: list[int]):
         n = logits.shape[0]
@@ -39,15 +58,27 @@ class Sampler:
         if n == 0:
             e = torch.empty(0, device=self.device)
             return e.to(torch.int32), e.to(torch.float32)
-        f = np.empty((3, n), dtype=np.float32)
-        i = np.empty((2, n), dtype=np.int32)
+        # all per-row parameters in one buffer, one copy: seeds (int64), then three float32
+        # rows and two int32 rows
+        host = self._stage(7 * n)
+        words = host.numpy()
+        words[: 2 * n].view(np.int64)[:] = seeds
+        f = words[2 * n : 5 * n].view(np.float32).reshape(3, n)
+        i = words[5 * n : 7 * n].reshape(2, n)
         for r, p in enumerate(params):
             f[0, r] = 0.0 if p.greedy else p.temperature
             f[1, r] = p.top_p
             f[2, r] = p.min_p
             i[0, r] = 1 if p.greedy else min(p.top_k, 2**31 - 1)
             i[1, r] = draw_index[r]
-        fd = torch.from_numpy(f).to(self.device)
-        idv = torch.from_numpy(i).to(self.device)
-        sd = torch.tensor(seeds, dtype=torch.int64).to(self.device)
-        return ops.sample(logits.contiguous(), fd[0], idv[0], fd[1], fd[2], sd, idv[1])
+        dev = torch.empty(7 * n, dtype=torch.int32, device=self.device)
+        dev.copy_(host[: 7 * n], non_blocking=True)
+        if self.device.type == "cuda":
+            event = torch.cuda.Event()
+            event.record()
+            self._staging[self._turn] = (self._staging[self._turn][0], event)
+        fd = dev[2 * n : 5 * n].view(torch.float32).view(3, n)
+        idv = dev[5 * n : 7 * n].view(2, n)
+        sd = dev[: 2 * n].view(torch.int64)
+        return ops.sample(logits.contiguous(), fd[0], idv[0], fd[1], fd[2], sd, idv[1],
+                          all_greedy=all(p.greedy for p in params))

@@ -377,6 +377,37 @@ def test_sample_matches_the_plain_sampler(gpu, kw):
     assert agree > 0.85 * n
 
 
+@pytest.mark.parametrize("vocab", [50257, 128256])
+def test_sample_large_vocabulary(gpu, vocab):
+    """Many tokens per thread: the filters' thresholds and the drawn tokens against the
+    plain sampler, with and without the room for keys between the passes."""
+    base = rnd(1, vocab, seed=83, scale=3.0)[0]
+    base[vocab // 3] = float("nan")
+    n = 24
+    logits = base[None].repeat(n, 1)
+    for kw in ({"top_p": 0.9, "temperature": 0.8}, {"top_k": 50}, {"top_k": 200, "top_p": 0.6, "min_p": 0.02}, {}):
+        params = {"temperature": 1.0, "seed": 5, **kw}
+        clean = torch.where(torch.isnan(base), torch.full_like(base, -1e5), base)
+        probs = P.filtered_probabilities(clean, params["temperature"], params.get("top_k", -1), params.get("top_p", 1.0), params.get("min_p", 0.0))
+        tok, lp = _sample(gpu, logits, seed=5, **kw)
+        f = lambda v, dt: torch.full((n,), v, dtype=dt, device=gpu)
+        tok_again, _ = ops.sample(
+            logits.to(gpu), f(params["temperature"], torch.float32), f(kw.get("top_k", -1), torch.int32),
+            f(kw.get("top_p", 1.0), torch.float32), f(kw.get("min_p", 0.0), torch.float32), f(5, torch.int64),
+            torch.arange(n, dtype=torch.int32, device=gpu), all_greedy=True,  # no room for keys: they are derived again
+        )
+        assert torch.equal(tok, tok_again)
+        agree = 0
+        for i in range(n):
+            t, logprob, margin = P.sample_token(clean, params, i)
+            assert probs[int(tok[i])] > 0, f"{kw}: a filtered token was sampled"
+            if margin > 2e-5:
+                assert int(tok[i]) == t, f"{kw} draw {i}: kernel {int(tok[i])}, plain {t}"
+                assert abs(float(lp[i]) - logprob) < 2e-4
+                agree += 1
+        assert agree > 0.8 * n
+
+
 def test_sample_rows_are_independent(gpu):
     logits = rnd(8, 331, seed=82, scale=2.0)
     temp = torch.tensor([0.0, 1.0, 0.5, 2.0, 1.0, 0.0, 1.0, 0.7])
