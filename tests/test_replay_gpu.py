@@ -79,6 +79,18 @@ def test_schedules(folders, name, page, schedule, dtype):
     assert runner.cache.idle()
 
 
+def test_bfloat16_run_of_a_folder_stored_in_float32(folders):
+    """Tensors stored in 32-bit stay so: the products then run on the float32 kernels
+    with bfloat16 activations, cache and attention."""
+    folder, requests, ref = folders[("B", "float32")]
+    trace = replay.mixed(requests, seed=2)
+    runner = make_runner(folder, "bfloat16", replay.peak_tokens(trace))
+    assert runner.model.embedding.weight.dtype == torch.float32
+    assert runner.cache.groups[0].storage.dtype == torch.bfloat16
+    rows = replay.collect(trace, replay.run_trace(runner, trace), 512)
+    replay.compare(rows, ref, TOL["bfloat16"])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_cuts_agree_with_each_other(folders, dtype):
     """The logits at a position do not depend on how the tokens were cut, beyond
