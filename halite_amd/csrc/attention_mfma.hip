@@ -17,7 +17,18 @@
 // (A = 16 dims x 32 keys straight from the transposed value page, B = the lane's own
 // eight probabilities).  The keys of the two 16-key MFMA tiles are interleaved so that
 // a lane's eight probabilities are eight consecutive keys, which is one 16-byte load of
-// the transposed values.  Nothing goes through LDS.
+// the transposed values.
+//
+// Two kernels come from one body.  Decode tokens (segments of at most 16 rows) run one
+// item per wave, nothing goes through LDS, and the key range of a long request is cut
+// into many items.  Prompt portions run four items per workgroup (up to RT_BIG tiles
+// each): the waves walk the union of their key ranges together and load each block of
+// keys and values once, into LDS, one block ahead.
+//
+// The pages are read in one of three ways: pages in the kernel's fragment order (TILED:
+// one contiguous KB per MFMA operand, see kv_key_offset in hal_common.h), row-major pages
+// of a power of two of at least 32 tokens (PAGE32: the page number of a block is the
+// same for the whole wave), and any other page size (a lane looks its own keys up).
 //
 // scores, causal rule and grouped heads as in src/halite/transformers/attention.py:
 // 647-714 and src/halite/transformers/infer/engine/flashinfer_backend.py:217-261.
@@ -180,8 +191,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   // is held), their scores are masked and their values cleared.
   //
   // Otherwise every lane looks its keys' pages up itself; keys outside
-  // [kv_begin, last_key] are clamped for the address only, and the page numbers are
-  // fetched one block ahead of the loads that need them.
+  // [walk_begin, last_key] are clamped for the address only.
   const int koff0 = ((col / 4) * 8 + (col % 4)) * D + quad * 8;  // tile 1 is 4 keys on
   const int voff = col * page_size + quad * 8;
   auto key_index = [&](int j0, int t) {
