@@ -43,6 +43,26 @@ LLAMA_3_1_8B = dict(
 )
 
 
+LLAMA_3_2_3B = dict(
+    LLAMA_3_1_8B,
+    hidden_size=3072,
+    num_hidden_layers=28,
+    num_attention_heads=24,
+    intermediate_size=8192,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    tie_word_embeddings=True,
+)
+
+LLAMA_3_1_70B = dict(
+    LLAMA_3_1_8B,
+    hidden_size=8192,
+    num_hidden_layers=80,
+    num_attention_heads=64,
+    intermediate_size=28672,
+)
+
+
 def layer_params(c) -> int:
     d, f = c.hidden_size, c.intermediate_size
     qkv = (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim * d
@@ -68,6 +88,104 @@ def prefill_flops(c, n_layers, t) -> float:
     return linear + attention + head
 
 
+def engine_workload(args) -> int:
+    """The two further workloads: requests through the scheduler (entry point, prompt
+    portions, decoding, sampling), one JSON line.
+
+    ``mixed3b``: Llama-3.2-3B shape, 32 requests with prompt lengths uniform in 64..4096,
+    prompts cut into portions of 512 tokens, 256 new tokens each.
+    ``llama70b``: Llama-3.1-70B shape on the one GPU (141 GB of weights), 16 requests
+    with 2,048-token prompts and 128 new tokens each.
+    """
+    import torch
+
+    from halite_amd.config import LlamaConfig, ModelConfig, ServerConfig
+    from halite_amd.engine.engine import InferenceEngine
+    from halite_amd.engine.runner import ModelRunner
+    from halite_amd.sampling import SamplingParams
+
+    gen = torch.Generator().manual_seed(0)
+    if args.workload == "mixed3b":
+        raw, name = LLAMA_3_2_3B, "Llama-3.2-3B shape"
+        lengths = torch.randint(64, 4097, (32,), generator=gen).tolist()
+        new_tokens, chunk = 256, 512
+    else:
+        raw, name = LLAMA_3_1_70B, "Llama-3.1-70B shape"
+        lengths, new_tokens, chunk = [2048] * 16, 128, 8192
+    full = LlamaConfig(**raw)
+    n_layers = args.layers or full.num_hidden_layers
+    cfg = full.model_copy(update={"num_hidden_layers": n_layers})
+    pool = sum(-(-(n + new_tokens) // 64) * 64 for n in lengths) + 1024
+    server = ServerConfig(
+        kv_cache_num_tokens=pool, max_seqs_per_forward=len(lengths), max_tokens_per_forward=8192,
+        chunked_prefill_size=chunk, max_prefill_tokens=8192, use_cudagraph=not args.no_graph,
+        cudagraph_max_batch_size=len(lengths),
+    )
+    t0 = time.perf_counter()
+    runner = ModelRunner.from_random(cfg, seed=0, server_config=server, model_config=ModelConfig(dtype=args.dtype, context_len=8192))
+    torch.cuda.synchronize()
+    print(f"[bench] {name}: {n_layers} layers built in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
+    engine = InferenceEngine(runner, None, seed=0)
+    params = SamplingParams(max_new_tokens=new_tokens, temperature=0.0, ignore_eos=True)
+
+    def requests():
+        return [(torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist(), params) for n in lengths]
+
+    # an untimed pass over a few short requests: libraries, graphs of the small batches
+    engine.infer_batch([(torch.randint(0, cfg.vocab_size, (64,), generator=gen).tolist(),
+                         SamplingParams(max_new_tokens=4, temperature=0.0, ignore_eos=True)) for _ in range(2)])
+    before = engine.stats.steps, engine.stats.retractions, len(engine.stats.tokens_per_step)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    results = engine.infer_batch(requests())
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    generated = sum(len(o) for r in results for o in r.output_ids)
+    assert generated == len(lengths) * new_tokens, generated
+    steps = engine.stats.steps - before[0]
+    per_step = engine.stats.tokens_per_step[before[2]:]
+    record = {
+        "metric": f"generated tokens per second through the scheduler ({name}, {len(lengths)} requests)",
+        "value": round(generated / dt, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": 0,
+        "ms_per_step": round(dt / steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: seeded uniform-random token ids, random weights N(0, 0.02)",
+        "config": {
+            "model": name,
+            "layers": n_layers,
+            "layers_of_model": full.num_hidden_layers,
+            "hidden_size": cfg.hidden_size,
+            "heads": cfg.num_attention_heads,
+            "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim,
+            "intermediate_size": cfg.intermediate_size,
+            "vocab_size": cfg.vocab_size,
+            "global_batch": len(lengths),
+            "seq_len": max(lengths) + new_tokens,
+            "prompt_tokens": sum(lengths),
+            "new_tokens_each": new_tokens,
+            "prefill_portion": chunk,
+            "page_size": runner.cache.page_size,
+            "hip_graph": not args.no_graph,
+            "parallelism": "single GPU",
+        },
+        "seconds": round(dt, 3),
+        "total_tokens_per_second": round((generated + sum(lengths)) / dt, 1),
+        "mean_tokens_per_step": round(sum(per_step) / max(1, len(per_step)), 1),
+        "retractions": engine.stats.retractions - before[1],
+        "weights_gb": round(runner.model.param_bytes() / 1e9, 2),
+    }
+    print(json.dumps(record), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -80,10 +198,14 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (for profiles)")
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b"],
+                    help="decode8b: the headline line; the others run requests through the scheduler")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.workload != "decode8b":
+        return engine_workload(args)
 
     import numpy as np
     import torch
