@@ -148,27 +148,28 @@ def _group_items(items: np.ndarray, piece: np.ndarray, group: int) -> np.ndarray
     keys; a run that cannot be filled is padded with items that have no rows and no keys.
     The runs with the longest walk come first."""
     n = len(items)
+    if n == 0:
+        return np.zeros((0, 8), np.int32)
     order = np.lexsort((np.arange(n), piece, items[:, 0]))  # segment, then piece, then tile
-    runs = []
-    start = 0
-    keys = np.stack((items[order, 0], piece[order]), axis=1)
-    for i in range(1, n + 1):
-        if i == n or (keys[i] != keys[start]).any():
-            idx = order[start:i]
-            for c in range(0, len(idx), group):
-                run = items[idx[c : c + group]]
-                if len(run) < group:
-                    pad = np.full((group - len(run), 8), -1, dtype=np.int32)
-                    pad[:, 0] = run[0, 0]
-                    pad[:, 2:4] = 0
-                    run = np.concatenate((run, pad))
-                runs.append(run)
-            start = i
-    def walk(run):
-        live = run[run[:, 3] > run[:, 2]]
-        return int(live[:, 3].max() - live[:, 2].min()) if len(live) else 0
-    runs.sort(key=lambda r: -walk(r))
-    return np.concatenate(runs) if runs else np.zeros((0, 8), np.int32)
+    seg, pc = items[order, 0], piece[order]
+    new_class = np.concatenate(([True], (seg[1:] != seg[:-1]) | (pc[1:] != pc[:-1])))
+    class_start = np.nonzero(new_class)[0]
+    class_len = np.diff(np.concatenate((class_start, [n])))
+    padded_len = -(-class_len // group) * group
+    padded_start = np.concatenate(([0], np.cumsum(padded_len)[:-1]))
+    class_of = np.cumsum(new_class) - 1
+    dest = padded_start[class_of] + (np.arange(n) - class_start[class_of])
+    total = int(padded_len.sum())
+    out = np.full((total, 8), -1, dtype=np.int32)
+    out[:, 2:4] = 0
+    out[:, 0] = np.repeat(seg[class_start], padded_len)  # the padding carries its run's segment
+    out[dest] = items[order]
+    runs = out.reshape(total // group, group, 8)
+    live = runs[:, :, 3] > runs[:, :, 2]
+    first_key = np.where(live, runs[:, :, 2], np.iinfo(np.int32).max).min(axis=1)
+    end_key = np.where(live, runs[:, :, 3], 0).max(axis=1)
+    walk = np.where(live.any(axis=1), end_key - first_key, 0)
+    return runs[np.argsort(-walk, kind="stable")].reshape(total, 8)
 
 
 def _group_tiles(seg_ids, rho0s, kv_b, kv_e, per_item: int, zigzag: bool):
@@ -177,21 +178,28 @@ def _group_tiles(seg_ids, rho0s, kv_b, kv_e, per_item: int, zigzag: bool):
     that every item has about the same number of (tile, key block) pairs under the
     causal rule; otherwise neighbours go together."""
     out_seg, out_rho, out_b, out_e, more = [], [], [], [], []
-    for s in np.unique(seg_ids):
-        idx = np.nonzero(seg_ids == s)[0]  # in row order
-        n = len(idx)
+    starts = np.nonzero(np.concatenate(([True], seg_ids[1:] != seg_ids[:-1])))[0]  # tiles are in segment order
+    ends = np.concatenate((starts[1:], [len(seg_ids)]))
+    for lo, hi in zip(starts.tolist(), ends.tolist()):
+        n = hi - lo
         if zigzag and per_item == 2:
-            groups = [[idx[i], idx[n - 1 - i]] if i != n - 1 - i else [idx[i]] for i in range((n + 1) // 2)]
+            n_items = (n + 1) // 2
+            members = np.stack((lo + np.arange(n_items), hi - 1 - np.arange(n_items)), axis=1)
+            valid = np.ones_like(members, dtype=bool)
+            if n % 2:
+                valid[-1, 1] = False  # the middle tile rides alone
         else:
-            groups = [list(idx[i : i + per_item]) for i in range(0, n, per_item)]
-        for grp in groups:
-            out_seg.append(s)
-            out_rho.append(rho0s[grp[0]])
-            out_b.append(min(kv_b[t] for t in grp))
-            out_e.append(max(kv_e[t] for t in grp))
-            more.append([rho0s[t] for t in grp[1:]] + [-1] * (per_item - len(grp)))
-    arr = lambda x: np.array(x, dtype=np.int64)
-    return arr(out_seg), arr(out_rho), arr(out_b), arr(out_e), arr(more).reshape(len(out_seg), per_item - 1)
+            n_items = -(-n // per_item)
+            members = lo + np.arange(n_items * per_item).reshape(n_items, per_item)
+            valid = members < hi
+            members = np.minimum(members, hi - 1)
+        out_seg.append(seg_ids[members[:, 0]])
+        out_rho.append(rho0s[members[:, 0]])
+        out_b.append(np.where(valid, kv_b[members], np.iinfo(np.int64).max).min(axis=1))
+        out_e.append(np.where(valid, kv_e[members], 0).max(axis=1))
+        more.append(np.where(valid[:, 1:], rho0s[members[:, 1:]], -1))
+    cat = lambda x: np.concatenate(x).astype(np.int64)
+    return cat(out_seg), cat(out_rho), cat(out_b), cat(out_e), np.concatenate(more).astype(np.int64).reshape(-1, per_item - 1)
 
 
 def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: int,
