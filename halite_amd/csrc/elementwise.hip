@@ -469,6 +469,37 @@ __global__ void rope_append_vec_kernel(T* __restrict__ qkv, int row_stride,
     store4(kp + kv_key_offset(tiled, page_size, D, off, i), a[0]);
     store4(kp + kv_key_offset(tiled, page_size, D, off, i + 4), a[1]);
   }
+  // Values: eight consecutive slots of one dimension lie side by side in a page (both
+  // layouts).  Where this token and the seven after it are one request's positions
+  // 8j .. 8j+7, the block of the first writes the values of all eight, eight at a time;
+  // the other seven leave theirs to it.
+  if (page_size % 8 == 0) {
+    const int t0 = t - off % 8;  // where the group's first token would be
+    const int seg = token_seg[t];
+    const bool whole = t0 >= 0 && t0 + 7 < (int)gridDim.x && token_seg[t0] == seg &&
+                       token_seg[t0 + 7] == seg && positions[t0] == pos - off % 8 &&
+                       positions[t0 + 7] == pos - off % 8 + 7;
+    if (whole) {
+      if (t != t0) return;
+      for (int idx = threadIdx.x; idx < K * D; idx += blockDim.x) {
+        const int g = idx / D, d = idx % D;
+        __attribute__((aligned(16))) T vals[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          vals[e] = qkv[(size_t)(t + e) * row_stride + (size_t)(H + K + g) * D + d];
+        T* vp = v_pages + ((size_t)page * K + g) * D * page_size +
+                kv_value_offset(tiled, page_size, D, off, d);
+        // eight elements in one or two 16-byte stores (the offset is a multiple of 8)
+        if constexpr (sizeof(T) == 2) {
+          *(uint4*)vp = *(const uint4*)vals;
+        } else {
+          *(uint4*)vp = *(const uint4*)vals;
+          *(uint4*)(vp + 4) = *(const uint4*)(vals + 4);
+        }
+      }
+      return;
+    }
+  }
   const int d8 = D / 8;
   for (int idx = threadIdx.x; idx < K * d8; idx += blockDim.x) {
     const int g = idx / d8, i = (idx % d8) * 8;

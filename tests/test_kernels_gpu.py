@@ -141,8 +141,8 @@ def from_tiled(kt, vt):
     (8, 8, 128, 128, 64, True), (3, 1, 32, 16, 32, True), (4, 2, 64, 64, 32, True), (2, 1, 96, 40, 64, True)])
 def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page, tiled):
     dt = DT[dtype]
-    n_seg, table_w = 3, -(-64 // page)
-    lens, starts = [5, 1, 9], [3, 40, 0]
+    n_seg, table_w = 4, -(-64 // page)
+    lens, starts = [5, 1, 9, 20], [3, 40, 0, 6]  # runs of eight aligned positions and ragged ends
     T = sum(lens)
     qkv = rnd(T, (H + 2 * K) * D, seed=9).to(dt)
     positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).to(torch.int32)
