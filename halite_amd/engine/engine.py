@@ -149,6 +149,11 @@ class InferenceEngine:
     def initialize(self):
         self.initialized = True
 
+    def load_state_dict(self, state_dict: dict, assign: bool = True):
+        """New weights for the running engine (engine.py:48-52 of the reference; tensors
+        are named as in a model folder and are always copied into the engine's own)."""
+        self.model_runner.load_state_dict(state_dict)
+
     def cleanup(self):
         self.scheduler.initialize()
         self.initialized = False

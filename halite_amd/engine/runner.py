@@ -145,6 +145,15 @@ class ModelRunner:
         runner.arch, runner.config = arch, cfg
         return runner
 
+    def load_state_dict(self, tensors: dict) -> None:
+        """New weights from tensors in memory, named as in a model folder.  The requests
+        that are live keep their cache; captured graphs hold the old tensors and are
+        dropped."""
+        from ..weights import load_state_dict
+
+        load_state_dict(self.model, self.arch.weight_map(self.config), tensors)
+        self._graphs.clear()
+
     # -- requests -------------------------------------------------------------------
     def admit(self) -> int:
         return self.cache.admit()

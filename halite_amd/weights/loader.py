@@ -20,7 +20,7 @@ import re
 import torch
 
 from ..parts.decoder import Decoder
-from .safetensors_io import ModelFiles, SafetensorsError
+from .safetensors_io import _NAMES, ModelFiles, SafetensorsError
 
 _FLOATS = {"F32", "BF16", "F16", "F64"}
 _INTS = {"I64", "I32", "I16", "I8", "U8"}
@@ -71,11 +71,44 @@ def stored_to_target_dtype(stored: str, engine_dtype: torch.dtype, integer: bool
     return torch.bfloat16
 
 
+class _TensorDict:
+    """Tensors in memory behind the interface of ``ModelFiles``."""
+
+    def __init__(self, tensors: dict[str, torch.Tensor]):
+        self.tensors = tensors
+
+    def names(self):
+        return list(self.tensors)
+
+    def dtype_of(self, name):
+        return _NAMES.get(self.tensors[name].dtype, str(self.tensors[name].dtype))
+
+    def shape_of(self, name):
+        return tuple(self.tensors[name].shape)
+
+    def tensor(self, name):
+        return self.tensors[name]
+
+    def close(self):
+        pass
+
+
+def load_state_dict(model: Decoder, weight_table: dict[str, str], tensors: dict[str, torch.Tensor]) -> None:
+    """The same as ``load_weights`` from tensors in memory, named as in a folder (the
+    reference's engine takes new weights this way,
+    src/halite/transformers/infer/engine/engine.py:48-52)."""
+    _fill(model, weight_table, _TensorDict(tensors), "the given tensors")
+
+
 def load_weights(model: Decoder, weight_table: dict[str, str], folder: str) -> None:
     try:
         files = ModelFiles(folder)
     except SafetensorsError as e:
         raise WeightError(folder, other=[str(e)]) from e
+    _fill(model, weight_table, files, folder)
+
+
+def _fill(model: Decoder, weight_table: dict[str, str], files, folder: str) -> None:
     try:
         name_to_path = expand_weight_map(weight_table, list(model.spec.layers))
         path_to_name = {v: k for k, v in name_to_path.items()}

@@ -131,6 +131,33 @@ def test_portions_retraction_and_page_reuse_keep_the_tokens(models):
     assert tight.model_runner.cache.idle()
 
 
+def test_new_weights_for_a_running_engine(models, tmp_path):
+    """``load_state_dict`` takes tensors named as in a model folder: afterwards the
+    engine generates what an engine built from those weights generates (graphs that were
+    captured with the old tensors included), and a bad dict is refused with the list."""
+    from halite_amd.weights import WeightError
+
+    folder, pc, pw = models[("A", "float32")]
+    server = ServerConfig(kv_cache_num_tokens=1024, use_cudagraph=True)
+    engine = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="float32"))
+    prompt = tiny.random_tokens(tiny.TINY_A, 20, 7)
+    params = {"max_new_tokens": 12, "temperature": 0.0}
+    before = engine.infer_batch([(prompt, params)])[0].output_ids[0]
+    other = tiny.random_weights(tiny.TINY_A, seed=99, std=0.08)
+    engine.load_state_dict(other)
+    after = engine.infer_batch([(prompt, params)])[0].output_ids[0]
+    new_folder = str(tmp_path / "other")
+    tiny.write_model_folder(new_folder, tiny.TINY_A, other, torch.float32)
+    fresh = InferenceEngine.from_pretrained(new_folder, server, ModelConfig(dtype="float32"))
+    assert after == fresh.infer_batch([(prompt, params)])[0].output_ids[0] and after != before
+    broken = dict(other)
+    broken.pop("model.norm.weight")
+    broken["extra.weight"] = torch.zeros(3)
+    with pytest.raises(WeightError, match="model.norm.weight") as err:
+        engine.load_state_dict(broken)
+    assert "extra.weight" in str(err.value)
+
+
 def test_command_line(models, tmp_path):
     folder, pc, pw = models[("B", "float32")]
     cmd = [sys.executable, "-m", "halite_amd.cli.generate", "--model", folder, "--prompt-ids", "5,17,3,250,9",
