@@ -6,6 +6,7 @@ import time
 from collections.abc import Sequence
 
 import numpy as np
+import torch
 
 from ..config.engine import ModelConfig, ServerConfig
 from ..sampling import Sampler, SamplingParams, request_seed
@@ -65,6 +66,11 @@ class InferenceEngine:
             [r.seed for r in rows],
             [len(r.output_ids) for r in rows],
         )
+        # the two results are the halves of one buffer: one copy, one wait
+        n = tokens.numel()
+        if tokens.data_ptr() + 4 * n == logprobs.data_ptr():
+            host = torch.as_strided(tokens, (2 * n,), (1,)).cpu()
+            return host[:n].tolist(), host[n:].view(torch.float32).tolist()
         return tokens.tolist(), logprobs.tolist()
 
     # -- requests ----------------------------------------------------------------------

@@ -257,8 +257,9 @@ def sample(
     _need(seeds.dtype == torch.int64, "sample: seeds are int64")
     for t in (temperature, top_k, top_p, min_p, seeds, draw_index):
         _need(t.numel() == n, "sample: one parameter per row")
-    tokens = torch.empty(n, dtype=torch.int32, device=logits.device)
-    logprobs = torch.empty(n, dtype=torch.float32, device=logits.device)
+    # one buffer for both results, so that the host can fetch them with one copy
+    both = torch.empty(2 * n, dtype=torch.int32, device=logits.device)
+    tokens, logprobs = both[:n], both[n:].view(torch.float32)
     keys = None if all_greedy else torch.empty((n, vocab), dtype=torch.int32, device=logits.device)
     _check(
         lib,
