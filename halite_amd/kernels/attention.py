@@ -126,14 +126,20 @@ def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_
     items[:, 4] = -1
     n_split = int(split.sum())
     items[split, 4] = first_slot + np.arange(n_split) * slots_per_tile
-    merges = []
-    for t in np.nonzero(n_pieces > 1)[0]:
-        slot0 = int(items[first_item[t], 4])
-        firsts = [int(rho0s[t])] + ([int(r) for r in more_tiles[t]] if more_tiles is not None else [])
-        for sub, r0 in enumerate(firsts):
-            if r0 >= 0:
-                merges.append([seg_ids[t], r0, slot0 + sub, n_pieces[t], slots_per_tile, 0, 0, 0])
-    merges = np.array(merges, dtype=np.int32).reshape(-1, 8)
+    # one merge entry per 16-row tile of every item that was cut
+    cut = np.nonzero(n_pieces > 1)[0]
+    firsts = rho0s[cut][:, None]
+    if more_tiles is not None:
+        firsts = np.concatenate((firsts, more_tiles[cut]), axis=1)
+    sub = np.broadcast_to(np.arange(firsts.shape[1]), firsts.shape)
+    keep = firsts >= 0
+    rows_of = np.broadcast_to(cut[:, None], firsts.shape)[keep]
+    merges = np.zeros((int(keep.sum()), 8), dtype=np.int32)
+    merges[:, 0] = seg_ids[rows_of]
+    merges[:, 1] = firsts[keep]
+    merges[:, 2] = items[first_item[rows_of], 4] + sub[keep]
+    merges[:, 3] = n_pieces[rows_of]
+    merges[:, 4] = slots_per_tile
     if group > 1:
         items = _group_items(items, piece, group)
     else:
