@@ -75,6 +75,7 @@ class CacheManager:
         self.slots = SlotAllocator(n_slots)
         self.state = StateStore(n_slots, state_needs or {}, self.device if allocate else "cpu")
         self.lengths: dict[int, int] = {}
+        self.version = 0  # counts every change of slots, lengths and pages
 
     # -- sizes ------------------------------------------------------------------
     @staticmethod
@@ -98,6 +99,7 @@ class CacheManager:
 
     # -- requests -----------------------------------------------------------------
     def admit(self) -> int:
+        self.version += 1
         slot = self.slots.alloc()
         self.lengths[slot] = 0
         self.state.reset(slot)
@@ -126,17 +128,20 @@ class CacheManager:
         for m, g in zip(missing, self.groups):
             if m > g.pool.available:
                 raise NoSpace(f"group {g.group_id}: {m} pages wanted, {g.pool.available} free")
+        self.version += 1
         for g in self.groups:
             for slot, new_len in spans:
                 g.reserve(slot, self.lengths[slot], new_len)
 
     def advance(self, slot: int, new_len: int) -> None:
         """The tokens up to ``new_len`` are in the cache now."""
+        self.version += 1
         self.lengths[slot] = new_len
         for g in self.groups:
             g.release_passed(slot, new_len)
 
     def free(self, slot: int) -> None:
+        self.version += 1
         for g in self.groups:
             g.release_all(slot)
         del self.lengths[slot]

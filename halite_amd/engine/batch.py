@@ -210,6 +210,13 @@ class StepContext:
                 raise RuntimeError("a static step needs its attention plans before the upload")
             self._plans[key] = attention_kernels.upload_plan(plan, self.device)
 
+    def replace_tokens(self, tokens: np.ndarray) -> None:
+        """Other token ids for a context that was put together before they were known
+        (and has not been copied to the device yet)."""
+        if self._dev is not None or tokens.size != self.n_tokens:
+            raise RuntimeError("token ids can only be replaced, one for one, before the upload")
+        self._packer.parts[0] = np.ascontiguousarray(tokens, dtype=np.int32).reshape(-1)
+
     def upload(self):
         if self._dev is not None:
             return

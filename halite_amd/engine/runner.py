@@ -14,7 +14,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from ..cache import CacheManager
+from ..cache import CacheManager, NoSpace
 from ..config.engine import ModelConfig, ServerConfig
 from ..config.registry import read_config
 from ..parts.decoder import Decoder
@@ -85,6 +85,8 @@ class ModelRunner:
             if hasattr(pos, "tables"):
                 pos.tables(self.context_len)
         self._graphs: dict[int, dict] = {}
+        self._ahead = None  # (requests and positions, cache version, context) of a step put together ahead
+        self.steps_taken_ahead = 0
         kv_heads = [n.n_kv_heads for n in needs.values()] or [1]
         self._min_kv_heads = min(kv_heads)
         self.graph_replays = 0
@@ -153,6 +155,7 @@ class ModelRunner:
 
         load_state_dict(self.model, self.arch.weight_map(self.config), tensors)
         self._graphs.clear()
+        self._ahead = None
 
     # -- requests -------------------------------------------------------------------
     def admit(self) -> int:
@@ -189,14 +192,17 @@ class ModelRunner:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         self.check_segments(segments)
         spans = [(s.slot, s.start + s.tokens.size) for s in segments]
-        self.cache.reserve(spans)
-        logits = None
-        if (
+        graph_step = (
             self.server_config.use_cudagraph
             and len(segments) <= self.server_config.cudagraph_max_batch_size
             and all(s.tokens.size == 1 and s.want == [0] for s in segments)
-        ):
-            logits = self._step_graph(segments)
+        )
+        ahead = self._take_step_ahead(segments) if graph_step else None
+        if ahead is None:  # a step that was put together ahead has its pages already
+            self.cache.reserve(spans)
+        logits = None
+        if graph_step:
+            logits = self._step_graph(segments, ahead)
         if logits is None:
             ctx = StepContext(segments, self.cache, self.device, self._staging)
             for run in self.model.runs:
@@ -204,9 +210,43 @@ class ModelRunner:
             logits = self.model.forward(ctx)
         for slot, new_len in spans:
             self.cache.advance(slot, new_len)
+        if graph_step:
+            self._put_step_ahead(segments)
         return logits
 
-    def _step_graph(self, segments: list[Segment]):
+    # While the GPU works on a decode step, the host puts the next one together as far as
+    # it can without the tokens: the same requests, one position on.  If that is what
+    # the next call brings (and nothing else touched the cache meanwhile), only the token
+    # ids are filled in.
+    def _put_step_ahead(self, segments: list[Segment]) -> None:
+        self._ahead = None
+        entry = self._graphs.get(len(segments))
+        if entry is None or entry["graph"] is None:
+            return
+        nxt = [Segment(s.slot, s.start + 1, [0], [0]) for s in segments]
+        if any(s.start + 1 > self.context_len for s in nxt):
+            return
+        try:
+            self.cache.reserve([(s.slot, s.start + 1) for s in nxt])
+        except NoSpace:
+            return
+        ctx = StepContext(nxt, self.cache, self.device, self._staging, static=entry["layout"])
+        for run in self.model.runs:
+            self.model.mixer_of_run(run.index).prepare(ctx, run)
+        self._ahead = (tuple((s.slot, s.start) for s in nxt), self.cache.version, ctx)
+
+    def _take_step_ahead(self, segments: list[Segment]):
+        ahead, self._ahead = self._ahead, None
+        if ahead is None:
+            return None
+        key, version, ctx = ahead
+        if version != self.cache.version or key != tuple((s.slot, s.start) for s in segments):
+            return None
+        ctx.replace_tokens(np.concatenate([s.tokens for s in segments]))
+        self.steps_taken_ahead += 1
+        return ctx
+
+    def _step_graph(self, segments: list[Segment], ahead=None):
         """A decode-only step through a captured HIP graph, one graph per batch size
         (the reference captures its decode pass per padded batch size,
         src/halite/transformers/infer/engine/model_runner.py:159-239).  The step's
@@ -220,9 +260,11 @@ class ModelRunner:
             width = {g.group_id: -(-self.context_len // g.page_size) for g in self.cache.groups}
             cap = attention_kernels.TARGET_WAVES // self._min_kv_heads + 2 * B + 8
             entry = self._graphs[B] = {"layout": StaticLayout(B, width, cap, self.device), "graph": None}
-        ctx = StepContext(segments, self.cache, self.device, self._staging, static=entry["layout"])
-        for run in self.model.runs:
-            self.model.mixer_of_run(run.index).prepare(ctx, run)
+        ctx = ahead
+        if ctx is None:
+            ctx = StepContext(segments, self.cache, self.device, self._staging, static=entry["layout"])
+            for run in self.model.runs:
+                self.model.mixer_of_run(run.index).prepare(ctx, run)
         if not ctx.fits_static():
             return None
         ctx.upload()
