@@ -48,6 +48,9 @@ int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temp
                hipStream_t stream);
 
 // ---- the head-size-specific library (attention_mfma.hip) ---------------------------------
+int hal_sample_greedy(const float* logits, int ld, int n_rows, int V, float* parts,
+                      int* out_token, float* out_logprob, hipStream_t stream);
+
 int hal_attention_mfma_head_dim();
 int hal_attention_mfma_rows_per_big_item();
 int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_stride,

@@ -356,3 +356,91 @@ extern "C" int hal_sample(const float* logits, int ld, int n_rows, int V, const 
   HAL_LAUNCH_CHECK();
   return 0;
 }
+
+// ---- all rows greedy: the row is spread over GREEDY_PARTS blocks --------------------------
+// Stage one: a block takes a contiguous share of a row and leaves its maximum, the first
+// index of that maximum and the sum of exp(x - maximum); stage two joins a row's shares in
+// order (ties go to the lower index, as everywhere).
+#define GREEDY_PARTS 32
+#define GREEDY_THREADS 256
+
+__global__ void __launch_bounds__(GREEDY_THREADS)
+greedy_part_kernel(const float* __restrict__ logits, int ld, int V, float* __restrict__ parts) {
+  __shared__ ArgMax amax_s[GREEDY_THREADS / HAL_WAVE];
+  __shared__ float red[16];
+  const int row = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
+  const int share = ((V + GREEDY_PARTS - 1) / GREEDY_PARTS + 3) / 4 * 4;
+  const int begin = part * share;
+  const int end = begin + share < V ? begin + share : V;
+  const float* x = logits + (size_t)row * ld;
+  ArgMax am = {-INFINITY, 0x7fffffff};
+  for (int i = begin + tid; i < end; i += GREEDY_THREADS) {
+    const float z = clean_logit(x[i]);
+    if (z > am.v) am.v = z, am.i = i;  // a thread's indices rise: the first maximum stays
+  }
+#pragma unroll
+  for (int off = HAL_WAVE / 2; off > 0; off >>= 1) {
+    ArgMax o;
+    o.v = __shfl_xor(am.v, off, HAL_WAVE);
+    o.i = __shfl_xor(am.i, off, HAL_WAVE);
+    am = argmax_merge(am, o);
+  }
+  if (lane == 0) amax_s[wave] = am;
+  __syncthreads();
+  am = amax_s[0];
+  for (int w = 1; w < GREEDY_THREADS / HAL_WAVE; ++w) am = argmax_merge(am, amax_s[w]);
+  float sum = 0.f;
+  for (int i = begin + tid; i < end; i += GREEDY_THREADS) sum += expf(clean_logit(x[i]) - am.v);
+  sum = block_sum(sum, red);
+  if (tid == 0) {
+    float* p = parts + ((size_t)row * GREEDY_PARTS + part) * 4;
+    p[0] = am.v;
+    p[1] = __int_as_float(am.i);
+    p[2] = begin < end ? sum : 0.f;
+  }
+}
+
+__global__ void __launch_bounds__(HAL_WAVE)
+greedy_join_kernel(const float* __restrict__ parts, int* __restrict__ out_token,
+                   float* __restrict__ out_logprob) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  ArgMax am = {-INFINITY, 0x7fffffff};
+  float sum = 0.f;
+  if (lane < GREEDY_PARTS) {
+    const float* p = parts + ((size_t)row * GREEDY_PARTS + lane) * 4;
+    am.v = p[0], am.i = __float_as_int(p[1]), sum = p[2];
+  }
+  ArgMax best = am;
+#pragma unroll
+  for (int off = HAL_WAVE / 2; off > 0; off >>= 1) {
+    ArgMax o;
+    o.v = __shfl_xor(best.v, off, HAL_WAVE);
+    o.i = __shfl_xor(best.i, off, HAL_WAVE);
+    best = argmax_merge(best, o);
+  }
+  const float scaled = (am.v == -INFINITY) ? 0.f : sum * expf(am.v - best.v);
+  const float total = wave_sum(scaled);
+  if (lane == 0) {
+    out_token[row] = best.i;
+    out_logprob[row] = -logf(total);
+  }
+}
+
+// Greedy decoding of every row: first index of the maximum and its log-probability under
+// softmax(logits).  `parts` has room for n_rows * 32 * 4 floats.
+extern "C" int hal_sample_greedy(const float* logits, int ld, int n_rows, int V, float* parts,
+                                 int* out_token, float* out_logprob, hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "hal_sample_greedy: bad sizes rows=%d V=%d ld=%d",
+              n_rows, V, ld);
+  HAL_REQUIRE(n_rows <= 65535, "hal_sample_greedy: %d rows exceed the grid limit", n_rows);
+  if (n_rows == 0) return 0;
+  HAL_REQUIRE(parts != nullptr, "hal_sample_greedy: no room for the partial results");
+  hipLaunchKernelGGL(greedy_part_kernel, dim3(GREEDY_PARTS, n_rows), dim3(GREEDY_THREADS), 0, stream,
+                     logits, ld, V, parts);
+  HAL_LAUNCH_CHECK();
+  hipLaunchKernelGGL(greedy_join_kernel, dim3(n_rows), dim3(HAL_WAVE), 0, stream, parts, out_token,
+                     out_logprob);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}

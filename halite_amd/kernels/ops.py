@@ -244,10 +244,13 @@ def sample(
     seeds: torch.Tensor,
     draw_index: torch.Tensor,
     all_greedy: bool = False,
+    key_scratch: bool = True,
 ):
-    """Next token and log-probability of every row of float32 ``logits``.  Unless
-    ``all_greedy`` says that no row samples, the kernel gets room for one 32-bit key per
-    logit, which its passes over a row then read instead of deriving it again."""
+    """Next token and log-probability of every row of float32 ``logits``.
+    ``all_greedy`` promises that no row samples (``temperature`` 0 or ``top_k`` 1 in
+    every row): the rows are then spread over many blocks.  Otherwise, with
+    ``key_scratch``, the kernel gets room for one 32-bit key per logit, which its passes
+    over a row read instead of deriving it again."""
     lib = library.core_library()
     _dev(logits, temperature, top_k, top_p, min_p, seeds, draw_index)
     n, vocab = logits.shape
@@ -260,7 +263,11 @@ def sample(
     # one buffer for both results, so that the host can fetch them with one copy
     both = torch.empty(2 * n, dtype=torch.int32, device=logits.device)
     tokens, logprobs = both[:n], both[n:].view(torch.float32)
-    keys = None if all_greedy else torch.empty((n, vocab), dtype=torch.int32, device=logits.device)
+    if all_greedy and logits.is_contiguous():  # every row spread over many blocks
+        parts = torch.empty((n, 32, 4), dtype=torch.float32, device=logits.device)
+        _check(lib, lib.hal_sample_greedy(_ptr(logits), vocab, n, vocab, _ptr(parts), _ptr(tokens), _ptr(logprobs), _stream()))
+        return tokens, logprobs
+    keys = torch.empty((n, vocab), dtype=torch.int32, device=logits.device) if key_scratch and not all_greedy else None
     _check(
         lib,
         lib.hal_sample(

@@ -355,6 +355,13 @@ def test_sample_greedy(gpu, vocab):
     close(lp, want.float(), 1e-5, "greedy logprob")
     tok2, _ = _sample(gpu, logits, temperature=0.9, top_k=1)
     assert torch.equal(tok, tok2)
+    # the rows spread over many blocks (what the engine uses when no row samples)
+    n = logits.shape[0]
+    f = lambda v, dt: torch.full((n,), v, dtype=dt, device=gpu)
+    tok3, lp3 = ops.sample(logits.to(gpu), f(0.0, torch.float32), f(-1, torch.int32), f(1.0, torch.float32),
+                           f(0.0, torch.float32), f(7, torch.int64), f(0, torch.int32), all_greedy=True)
+    assert torch.equal(tok, tok3)
+    close(lp3, want.float(), 1e-5, "greedy logprob, many blocks")
 
 
 @pytest.mark.parametrize("kw", [{}, {"top_k": 5}, {"top_p": 0.7}, {"top_k": 40, "top_p": 0.9}, {"min_p": 0.1},
@@ -394,7 +401,7 @@ def test_sample_large_vocabulary(gpu, vocab):
         tok_again, _ = ops.sample(
             logits.to(gpu), f(params["temperature"], torch.float32), f(kw.get("top_k", -1), torch.int32),
             f(kw.get("top_p", 1.0), torch.float32), f(kw.get("min_p", 0.0), torch.float32), f(5, torch.int64),
-            torch.arange(n, dtype=torch.int32, device=gpu), all_greedy=True,  # no room for keys: they are derived again
+            torch.arange(n, dtype=torch.int32, device=gpu), key_scratch=False,  # the keys are derived again in every pass
         )
         assert torch.equal(tok, tok_again)
         agree = 0
