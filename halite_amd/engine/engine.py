@@ -52,7 +52,7 @@ class InferenceEngine:
     def _run_step(self, plan: StepPlan):
         segments, rows = [], []
         for i, (r, k) in enumerate(plan.entries):
-            ids = r.all_ids[r.n_cached : r.n_cached + k]
+            ids = r.ids_between(r.n_cached, r.n_cached + k)
             wants = plan.wants_logits(i)
             segments.append(Segment(r.slot, r.n_cached, np.asarray(ids, dtype=np.int32), [k - 1] if wants else []))
             if wants:

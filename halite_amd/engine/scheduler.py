@@ -62,6 +62,15 @@ class Request:
     def all_ids(self) -> list[int]:
         return self.input_ids + self.output_ids
 
+    def ids_between(self, start: int, end: int) -> list[int]:
+        """``all_ids[start:end]`` without putting the two lists together."""
+        n_in = len(self.input_ids)
+        if end <= n_in:
+            return self.input_ids[start:end]
+        if start >= n_in:
+            return self.output_ids[start - n_in : end - n_in]
+        return self.input_ids[start:] + self.output_ids[: end - n_in]
+
     @property
     def n_total(self) -> int:
         return len(self.input_ids) + len(self.output_ids)
@@ -234,10 +243,11 @@ class Scheduler:
         n_prefill = 0
 
         # 2. portions of the prompts that are under way, earlier requests first
+        in_step = {id(r) for r in decoding}
         for r in self.running:
             if budget <= 0:
                 break
-            if r.decoding or r in decoding:
+            if id(r) in in_step or r.decoding:
                 continue
             k = self._max_portion(r, spans, min(r.remaining, conf.chunked_prefill_size, budget))
             if k > 0:
@@ -247,7 +257,7 @@ class Scheduler:
                 n_prefill += k
 
         # 3. admission, first come first served (scheduler.py:211-265)
-        if not retracted_any:
+        if not retracted_any and self.waiting and budget > 0:
             free_tokens = self.cache.free_pages() * self.cache.page_size
             remaining_total = free_tokens - sum(
                 min(r.sampling_params.max_new_tokens - len(r.output_ids), CLIP_MAX_NEW_TOKENS)
