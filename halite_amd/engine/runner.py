@@ -179,9 +179,12 @@ class ModelRunner:
                 raise StepError(f"slot {s.slot}: tokens start at {s.start} but {have} are cached")
             if s.start + n > self.context_len:
                 raise StepError(f"slot {s.slot}: {s.start + n} tokens exceed the context length {self.context_len}")
-            lo, hi = int(s.tokens.min()), int(s.tokens.max())
-            if lo < 0 or hi >= self.vocab_size:
-                raise StepError(f"slot {s.slot}: token id {lo if lo < 0 else hi} outside the vocabulary of {self.vocab_size}")
+        every = np.concatenate([s.tokens for s in segments]) if len(segments) > 1 else segments[0].tokens
+        if int(every.min()) < 0 or int(every.max()) >= self.vocab_size:
+            for s in segments:
+                lo, hi = int(s.tokens.min()), int(s.tokens.max())
+                if lo < 0 or hi >= self.vocab_size:
+                    raise StepError(f"slot {s.slot}: token id {lo if lo < 0 else hi} outside the vocabulary of {self.vocab_size}")
 
     @torch.no_grad()
     def step(self, segments: list[Segment]) -> torch.Tensor:
