@@ -38,7 +38,7 @@ LLAMA_3_1_8B = dict(
     rope_theta=500000.0,
     rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
                       original_max_position_embeddings=8192),
-    max_position_embeddings=8192,
+    max_position_embeddings=131072,
     tie_word_embeddings=False,
 )
 
@@ -218,7 +218,7 @@ def main() -> int:
     full = LlamaConfig(**LLAMA_3_1_8B)
     n_layers = args.layers or full.num_hidden_layers
     cfg = full.model_copy(update={"num_hidden_layers": n_layers})
-    context = args.context or full.max_position_embeddings
+    context = args.context or 8192  # the benchmark's context; the model itself goes to 131,072
     elt = 2 if args.dtype == "bfloat16" else 4
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     if args.prefill_only:
@@ -312,7 +312,7 @@ def main() -> int:
     achieved = need / step_s
 
     record = {
-        "metric": "decode tokens per second (Llama-3.1-8B shape, batch 8, context 8192)",
+        "metric": f"decode tokens per second (Llama-3.1-8B shape, batch {args.batch}, context {context})",
         "value": round(value, 2),
         "unit": "tok/s",
         "n_gpus": 1,
