@@ -197,7 +197,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
-    ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (for profiles)")
+    ap.add_argument("--prefill-only", action="store_true", help="measure only the prefill (for profiles)")
+    ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill measurement")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b"],
                     help="decode8b: the headline line; the others run requests through the scheduler")
     args = ap.parse_args()
@@ -222,7 +223,7 @@ def main() -> int:
     elt = 2 if args.dtype == "bfloat16" else 4
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     if args.prefill_only:
-        batches, context = [1], 4096
+        batches, context = [1], max(4096, args.prefill_tokens + 64)
     pool_tokens = max(batches) * (context + 64) + 4096
     runner = ModelRunner.from_random(
         cfg, seed=0,
@@ -274,7 +275,7 @@ def main() -> int:
             runner.free(s)
         return dt, kv_tokens
 
-    def prefill_run(T=2048):
+    def prefill_run(T=args.prefill_tokens):
         ids = torch.randint(0, cfg.vocab_size, (T,), generator=gen).numpy().astype(np.int32)
         times = []
         for i in range(4):
@@ -337,7 +338,7 @@ def main() -> int:
             "global_batch": args.batch,
             "seq_len": context,
             "context_len": context,
-            "prefill_tokens": 2048,
+            "prefill_tokens": args.prefill_tokens,
             "page_size": runner.cache.page_size,
             "hip_graph": not args.no_graph,
             "parallelism": "single GPU",

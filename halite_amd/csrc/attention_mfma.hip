@@ -74,7 +74,7 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // Two waves per SIMD leave 256 registers each, which keeps the accumulators in VGPRs (no
 // copies to and from AGPRs around every MFMA); the largest head sizes need more.
 #define MIN_WAVES_PER_SIMD (D > 160 ? 1 : 2)
-template <int RT, bool POW2, bool PAGE32, bool SHARED, bool TILED>
+template <int RT, bool POW2, bool PAGE32, bool SHARED, bool TILED, int KB>
 __global__ void __launch_bounds__(256, MIN_WAVES_PER_SIMD)
 attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
                       int out_row_stride, const int* __restrict__ items,
@@ -255,48 +255,67 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     return __builtin_bit_cast(bf16x8, raw);
   };
 
+  // A step of the walk takes KB keys: 32 without LDS, 32 or 64 with it (SUBS blocks of 32).
+  static_assert(KB == 32 || (SHARED && KB == 64), "keys per step");
+  constexpr int SUBS = KB / 32;
   const int j_first = walk_begin & ~31;
-  // PAGE32: the page numbers of this block and the next three, looked up (scalar loads)
-  // well before the loads that need them
+  // PAGE32: page numbers are looked up (scalar loads) well before the loads that need them
   auto page_at = [&](int j0) {
     if constexpr (PAGE32) return uniform(bt[(j0 < walk_end ? j0 : j_first) >> page_shift]);
     else return 0;
   };
-  int page_0 = page_at(j_first), page_1 = page_at(j_first + 32), page_2 = page_at(j_first + 64);
 
   // Without LDS: this block's values and the next block's keys (a second buffer) are asked
   // for at the block's start; deeper or shallower schedules measured the same or worse.
+  int page_0 = 0, page_1 = 0, page_2 = 0;
   bf16x8 kcur[2][KT], knext[SHARED ? 1 : 2][SHARED ? 1 : KT], vf[DT];
-  // With LDS: fragment f of a block (keys first, then values) is loaded by wave f % 4 into
-  // registers one block ahead, and written to the other half of the LDS buffer while this
-  // block is worked on; a fragment lies there in lane order, as the MFMA wants it back.
+  // With LDS: fragment f of a block of 32 keys (keys first, then values) is loaded by wave
+  // f % 4 into registers one step ahead, and written to the other half of the LDS buffer
+  // while this step is worked on; a fragment lies there in lane order, as the MFMA wants
+  // it back.
   constexpr int NF = 2 * KT + DT, FPW = (NF + WAVES - 1) / WAVES;
-  __shared__ u32x4 frag_lds[SHARED ? 2 : 1][SHARED ? NF : 1][HAL_WAVE];
-  bf16x8 staged[SHARED ? FPW : 1];
-  auto fetch = [&](int j0, int page) {
+  __shared__ u32x4 frag_lds[SHARED ? 2 : 1][SHARED ? SUBS * NF : 1][HAL_WAVE];
+  bf16x8 staged[SHARED ? SUBS * FPW : 1];
+  int pages_ahead[SUBS];  // of the step after the next
+  auto fetch = [&](int j0, const int (&pages)[SUBS]) {
 #pragma unroll
-    for (int i = 0; i < FPW; ++i) {
-      const int f = wave + WAVES * i;
-      if (f < 2 * KT) staged[i] = load_key_frag(j0, page, f / KT, f % KT);
-      else if (f < NF) staged[i] = load_value_frag(j0, page, f - 2 * KT);
-    }
+    for (int u = 0; u < SUBS; ++u)
+#pragma unroll
+      for (int i = 0; i < FPW; ++i) {
+        const int f = wave + WAVES * i;
+        if (f < 2 * KT) staged[u * FPW + i] = load_key_frag(j0 + 32 * u, pages[u], f / KT, f % KT);
+        else if (f < NF) staged[u * FPW + i] = load_value_frag(j0 + 32 * u, pages[u], f - 2 * KT);
+      }
   };
   auto stash = [&](int j0, int half) {
 #pragma unroll
-    for (int i = 0; i < FPW; ++i) {
-      const int f = wave + WAVES * i;
-      if (f >= NF) continue;
-      bf16x8 v = staged[i];
-      if (f >= 2 * KT && j0 + 32 > kv_len) v = clear_unwritten(j0, v);
-      frag_lds[half][f][lane] = __builtin_bit_cast(u32x4, v);
-    }
+    for (int u = 0; u < SUBS; ++u)
+#pragma unroll
+      for (int i = 0; i < FPW; ++i) {
+        const int f = wave + WAVES * i;
+        if (f >= NF) continue;
+        bf16x8 v = staged[u * FPW + i];
+        if (f >= 2 * KT && j0 + 32 * u + 32 > kv_len) v = clear_unwritten(j0 + 32 * u, v);
+        frag_lds[half][u * NF + f][lane] = __builtin_bit_cast(u32x4, v);
+      }
+  };
+  auto pages_of = [&](int j0, int (&pages)[SUBS]) {
+#pragma unroll
+    for (int u = 0; u < SUBS; ++u) pages[u] = page_at(j0 + 32 * u);
   };
   if constexpr (SHARED) {
-    fetch(j_first, page_0);
+    int pages[SUBS];
+    pages_of(j_first, pages);
+    fetch(j_first, pages);
     stash(j_first, 0);
-    if (j_first + 32 < walk_end) fetch(j_first + 32, page_1);
+    if (j_first + KB < walk_end) {
+      pages_of(j_first + KB, pages);
+      fetch(j_first + KB, pages);
+    }
+    pages_of(j_first + 2 * KB, pages_ahead);
     __syncthreads();
   } else {
+    page_0 = page_at(j_first), page_1 = page_at(j_first + 32), page_2 = page_at(j_first + 64);
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -304,11 +323,15 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   }
 
   int half = 0;
-  for (int j0 = j_first; j0 < walk_end; j0 += 32) {
-    const bool tail = j0 + 32 > kv_len;  // some of the 32 keys are not written yet
-    const bool more = j0 + 32 < walk_end;
-    const int page_3 = page_at(j0 + 96);
-    if constexpr (!SHARED) {
+  for (int j0 = j_first; j0 < walk_end; j0 += KB) {
+    const bool tail = j0 + KB > kv_len;  // some of the keys are not written yet
+    const bool more = j0 + KB < walk_end;
+    int page_3 = 0;
+    int pages_later[SUBS];
+    if constexpr (SHARED) {
+      pages_of(j0 + 3 * KB, pages_later);
+    } else {
+      page_3 = page_at(j0 + 96);
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) vf[dt] = load_value_frag(j0, page_0, dt);
       if (more) {
@@ -318,66 +341,75 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
           for (int ks = 0; ks < KT; ++ks) knext[t][ks] = load_key_frag(j0 + 32, page_1, t, ks);
       }
     }
-    if constexpr (SHARED) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int ks = 0; ks < KT; ++ks)
-          kcur[t][ks] = __builtin_bit_cast(bf16x8, frag_lds[half][t * KT + ks][lane]);
-    }
 
-    // ---- S^T = K Q^T for 32 keys (two tiles of 16), all row tiles ------------------
-    f32x4 s[RT][2];
+    // ---- S^T = K Q^T for KB keys (tiles of 16), all row tiles ----------------------
+    f32x4 s[RT][SUBS][2];
     bool active[RT];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      // a block wholly after the tile's last row or before its first row's window
-      // does nothing for this tile
-      active[rt] = j0 <= p_last[rt] && j0 + 31 >= lo_first[rt] && j0 < kv_end && j0 + 32 > kv_begin;
+    for (int rt = 0; rt < RT; ++rt)
+      // a step wholly after the tile's last row or before its first row's window does
+      // nothing for this tile
+      active[rt] = j0 <= p_last[rt] && j0 + KB - 1 >= lo_first[rt] && j0 < kv_end && j0 + KB > kv_begin;
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        s[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (active[rt]) {
+    for (int u = 0; u < SUBS; ++u) {
+      if constexpr (SHARED) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int ks = 0; ks < KT; ++ks)
-            s[rt][t] =
-                __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][ks], bq[rt][ks], s[rt][t], 0, 0, 0);
+            kcur[t][ks] = __builtin_bit_cast(bf16x8, frag_lds[half][u * NF + t * KT + ks][lane]);
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          s[rt][u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+          if (active[rt]) {
+#pragma unroll
+            for (int ks = 0; ks < KT; ++ks)
+              s[rt][u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][ks], bq[rt][ks],
+                                                                    s[rt][u][t], 0, 0, 0);
+          }
         }
       }
     }
 
-    bf16x8 pb[RT];
+    bf16x8 pb[RT][SUBS];
     float alpha[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       alpha[rt] = 1.f;
-      pb[rt] = zero8();
-      if (!active[rt]) continue;
-      // ---- mask and online softmax: this lane has keys j0 + quad*8 + e, e = 0..7 --
-      float sv[8];
-      float m_tile = -INFINITY;
-      const bool full = j0 >= kv_begin && j0 + 32 <= kv_end && j0 + 31 <= p_first[rt] &&
-                        j0 >= lo_last[rt];
-      if (full) {  // every key of the block is visible to every row of the tile
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          sv[e] = s[rt][e / 4][e % 4] * scale_log2e;
-          m_tile = fmaxf(m_tile, sv[e]);
+      for (int u = 0; u < SUBS; ++u) pb[rt][u] = zero8();
+      if (!active[rt]) continue;
+      // ---- mask and online softmax: of every block of 32 keys this lane has the keys
+      // quad*8 + e, e = 0..7.  Raw scores; the scale (positive) goes into the exponent's
+      // multiply-add.
+      float sv[SUBS * 8];
+      float m_raw = -INFINITY;
+      const bool full = j0 >= kv_begin && j0 + KB <= kv_end && j0 + KB - 1 <= p_first[rt] &&
+                        j0 >= lo_last[rt];
+      if (full) {  // every key of the step is visible to every row of the tile
+#pragma unroll
+        for (int e = 0; e < SUBS * 8; ++e) {
+          sv[e] = s[rt][e / 8][(e % 8) / 4][e % 4];
+          m_raw = fmaxf(m_raw, sv[e]);
         }
       } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int j = j0 + quad * 8 + e;
+        for (int e = 0; e < SUBS * 8; ++e) {
+          const int j = j0 + (e / 8) * 32 + quad * 8 + e % 8;
           const bool ok =
               row_ok[rt] && j >= kv_begin && j < kv_end && j >= lo_row[rt] && j <= p_row[rt];
-          sv[e] = ok ? s[rt][e / 4][e % 4] * scale_log2e : -INFINITY;
-          m_tile = fmaxf(m_tile, sv[e]);
+          sv[e] = ok ? s[rt][e / 8][(e % 8) / 4][e % 4] : -INFINITY;
+          m_raw = fmaxf(m_raw, sv[e]);
         }
       }
-      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, HAL_WAVE));
-      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, HAL_WAVE));
+      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 16, HAL_WAVE));
+      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, HAL_WAVE));
+      const float m_tile = m_raw * scale_log2e;
       // The running maximum only has to keep exp2(s - m) in range, so it is raised
-      // only when the block's maximum exceeds it by more than 2^RESCALE_SLACK: then
+      // only when the step's maximum exceeds it by more than 2^RESCALE_SLACK: then
       // the accumulated sums are rarely rescaled (and a partial result's m, l and sums
       // stay consistent with each other, which is all the merge needs).
       const float m_new = m_tile > m[rt] + RESCALE_SLACK ? m_tile : m[rt];
@@ -385,18 +417,21 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       // gives exp2(-inf) = 0 everywhere without a branch
       const float m_sub = m_new == -INFINITY ? 0.f : m_new;
       alpha[rt] = fast_exp2(m[rt] - m_sub);
-      float pv[8];
+      float pv[SUBS * 8];
       float psum = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        pv[e] = fast_exp2(sv[e] - m_sub);
+      for (int e = 0; e < SUBS * 8; ++e) {
+        pv[e] = fast_exp2(__builtin_fmaf(sv[e], scale_log2e, -m_sub));
         psum += pv[e];
       }
       l[rt] = l[rt] * alpha[rt] + psum;
       m[rt] = m_new;
-      u32x4 praw = {pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]),
-                    pack2(pv[6], pv[7])};
-      pb[rt] = __builtin_bit_cast(bf16x8, praw);
+#pragma unroll
+      for (int u = 0; u < SUBS; ++u) {
+        u32x4 praw = {pack2(pv[u * 8 + 0], pv[u * 8 + 1]), pack2(pv[u * 8 + 2], pv[u * 8 + 3]),
+                      pack2(pv[u * 8 + 4], pv[u * 8 + 5]), pack2(pv[u * 8 + 6], pv[u * 8 + 7])};
+        pb[rt][u] = __builtin_bit_cast(bf16x8, praw);
+      }
     }
 
     // ---- O^T += V^T P^T ------------------------------------------------------------
@@ -410,37 +445,43 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
           for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha[rt];
       }
     }
-    if constexpr (SHARED) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-        vf[dt] = __builtin_bit_cast(bf16x8, frag_lds[half][2 * KT + dt][lane]);
-    } else if (tail) {
+    for (int u = 0; u < SUBS; ++u) {
+      if constexpr (SHARED) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) vf[dt] = clear_unwritten(j0, vf[dt]);
+        for (int dt = 0; dt < DT; ++dt)
+          vf[dt] = __builtin_bit_cast(bf16x8, frag_lds[half][u * NF + 2 * KT + dt][lane]);
+      } else if (tail) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = clear_unwritten(j0, vf[dt]);
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if (!active[rt]) continue;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          o[rt][dt] =
+              __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb[rt][u], o[rt][dt], 0, 0, 0);
+      }
     }
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      if (!active[rt]) continue;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-        o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb[rt], o[rt][dt], 0, 0, 0);
-    }
     if constexpr (SHARED) {
-      // the other half was read in the block before this one, and every wave has passed
+      // the other half was read in the step before this one, and every wave has passed
       // the barrier since
-      if (more) stash(j0 + 32, half ^ 1);
-      if (j0 + 64 < walk_end) fetch(j0 + 64, page_2);
+      if (more) stash(j0 + KB, half ^ 1);
+      if (j0 + 2 * KB < walk_end) fetch(j0 + 2 * KB, pages_ahead);
       __syncthreads();
       half ^= 1;
+#pragma unroll
+      for (int u = 0; u < SUBS; ++u) pages_ahead[u] = pages_later[u];
     } else {
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int ks = 0; ks < KT; ++ks) kcur[t][ks] = knext[t][ks];
+      page_0 = page_1;
+      page_1 = page_2;
+      page_2 = page_3;
     }
-    page_0 = page_1;
-    page_1 = page_2;
-    page_2 = page_3;
   }
 
 #pragma unroll
@@ -573,6 +614,11 @@ extern "C" int hal_attention_mfma_head_dim() { return D; }
 #define HAL_RT_BIG (D <= 64 ? 4 : (D <= 128 ? 2 : 1))
 #endif
 #define RT_BIG HAL_RT_BIG
+// Keys per step of the kernel for long segments: 64 where two halves of that fit 64 KB of LDS.
+#ifndef HAL_KB_BIG
+#define HAL_KB_BIG (D <= 128 ? 64 : 32)
+#endif
+#define KB_BIG HAL_KB_BIG
 
 extern "C" int hal_attention_mfma_rows_per_big_item() { return 16 * RT_BIG; }
 
@@ -610,13 +656,13 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   if ((page_size & (page_size - 1)) == 0)
     for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
   const int waves = WAVES;
-#define LAUNCH_ATTENTION(RT_, SHARED_, LIST, MAX, COUNT)                                          \
+#define LAUNCH_ATTENTION(RT_, SHARED_, KB_, LIST, MAX, COUNT)                                      \
   {                                                                                               \
     dim3 grid(((MAX) + waves - 1) / waves, K);                                                    \
-    auto kernel = attention_mfma_kernel<RT_, false, false, SHARED_, false>;                       \
-    if (tiled) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, D % 32 == 0>;             \
-    else if (page_shift >= 5) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, false>;    \
-    else if (page_shift >= 0) kernel = attention_mfma_kernel<RT_, true, false, SHARED_, false>;   \
+    auto kernel = attention_mfma_kernel<RT_, false, false, SHARED_, false, KB_>;                  \
+    if (tiled) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, D % 32 == 0, KB_>;        \
+    else if (page_shift >= 5) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, false, KB_>; \
+    else if (page_shift >= 0) kernel = attention_mfma_kernel<RT_, true, false, SHARED_, false, KB_>; \
     hipLaunchKernelGGL(kernel, grid, dim3(waves * HAL_WAVE), 0, stream, (const bf16_t*)q,         \
                        q_row_stride, (bf16_t*)out, out_row_stride, LIST, COUNT, seg_q_start,      \
                        seg_q_len, seg_kv_len, block_table, bt_stride, (const bf16_t*)k_pages,     \
@@ -624,8 +670,8 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
                        scale_log2e, window);                                                      \
     HAL_LAUNCH_CHECK();                                                                           \
   }
-  if (max_items > 0) LAUNCH_ATTENTION(1, false, items, max_items, counts)
-  if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, true, big_items, max_big, counts + 1)
+  if (max_items > 0) LAUNCH_ATTENTION(1, false, 32, items, max_items, counts)
+  if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, true, KB_BIG, big_items, max_big, counts + 1)
 #undef LAUNCH_ATTENTION
   if (max_merges > 0) {
     hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K, 16), dim3(256), 0, stream,
