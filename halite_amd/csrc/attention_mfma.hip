@@ -65,9 +65,9 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // item: {segment, first row of tile 0, first key, end key, first partial slot or -1,
 //        first row of tile 1, of tile 2, of tile 3 (or -1)}
 // A wave works on up to RT tiles of 16 rows of one segment; the keys and values it
-// loads serve all of them.  The tiles need not be neighbours: pairing an early tile of
-// a prompt with a late one gives every wave the same amount of causal work.  A tile
-// skips the blocks of keys that lie wholly outside its own range.  Row tile rt of an
+// loads serve all of them.  The tiles need not be neighbours (the host lists neighbours:
+// they share nearly all of their keys).  A tile skips the steps whose keys lie wholly
+// outside its own range.  Row tile rt of an
 // item writes partial slot `first partial slot + rt`.
 #define N_XCD 8
 #define WAVES 4  // per workgroup

@@ -82,9 +82,9 @@ def test_long_decode_is_split_and_prefill_is_not():
     assert plan.n_merges == 8 and plan.n_items > 8 * 4 and plan.n_big == 0
     plan = plan_items(np.array([2048]), np.array([2048]), 4, 8, 0)
     assert plan.n_merges == 0 and plan.n_big == 2048 * 4 // 64 and plan.n_items == 0
-    # zigzag: an early tile rides with a late one, every item reaches far
+    # neighbouring tiles ride together
     pair = plan_items(np.array([2048]), np.array([2048]), 4, 8, 0, 32)
-    assert pair.n_big == 256 and (pair.big_items[:, 3] > 1024).all()
+    assert pair.n_big == 256 and (pair.big_items[:, 5] == pair.big_items[:, 1] + 16).all()
     assert sorted(pair.big_items[:, 1].tolist() + pair.big_items[:, 5].tolist()) == list(range(0, 8192, 16))
     # a short portion of a prompt against a long context: few big tiles, so they are cut
     q_len, kv_len = np.array([64]), np.array([20000])
