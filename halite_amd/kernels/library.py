@@ -192,11 +192,10 @@ def attention_library(head_dim: int) -> ctypes.CDLL:
 def build_all(head_dims=(16, 32, 64, 128), force=True, prune=True) -> list[str]:
     """Compile every library for the given head sizes (the build check); with
     ``prune`` builds of older sources are removed from the in-tree build folder."""
-    paths = [build_library("core", CORE_SOURCES, {}, force=force)]
-    for d in head_dims:
-        paths.append(
-            build_library(f"attn_d{d}", ATTENTION_SOURCES, {"HAL_HEAD_DIM": d}, force=force)
-        )
+    jobs = [("core", CORE_SOURCES, {})]
+    jobs += [(f"attn_d{d}", ATTENTION_SOURCES, {"HAL_HEAD_DIM": d}) for d in head_dims]
+    with ThreadPoolExecutor(max_workers=4) as pool:  # each job compiles its sources in parallel too
+        paths = list(pool.map(lambda j: build_library(*j, force=force), jobs))
     if prune:
         folder = _build_dirs()[0]
         keep = {os.path.basename(p) for p in paths}
