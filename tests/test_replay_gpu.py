@@ -221,3 +221,39 @@ def test_decode_through_a_captured_graph(folders, dtype):
         for p in rows[rid]:
             d = float((rows[rid][p] - rows_eager[rid][p]).abs().max())
             assert d <= (1e-6 if dtype == "float32" else 2e-2), (rid, p, d)
+
+
+ODD = {
+    # a head size that is no multiple of 16 and a width that is no multiple of 8: the plain
+    # attention kernel and the library product serve the bfloat16 path
+    "head20": dict(tiny.TINY_A, hidden_size=60, num_attention_heads=3, num_key_value_heads=1, head_dim=20,
+                   intermediate_size=70, vocab_size=101),
+    "head24": dict(tiny.TINY_A, hidden_size=72, num_attention_heads=3, num_key_value_heads=3, head_dim=24,
+                   intermediate_size=100, vocab_size=257),
+    # heads of 96 and 256: tiled pages; 256 is the largest head and takes steps of 32 keys
+    "head96": dict(tiny.TINY_A, hidden_size=192, num_attention_heads=2, num_key_value_heads=1, head_dim=96,
+                   intermediate_size=520, vocab_size=1000, max_position_embeddings=512),
+    "head256": dict(tiny.TINY_A, hidden_size=256, num_attention_heads=2, num_key_value_heads=2, head_dim=256,
+                    intermediate_size=384, vocab_size=333, max_position_embeddings=512, tie_word_embeddings=True),
+    # no head_dim in the file: hidden_size / heads
+    "derived": {k: v for k, v in dict(tiny.TINY_A, hidden_size=96, num_attention_heads=6, num_key_value_heads=2,
+                                      intermediate_size=128).items() if k != "head_dim"},
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(ODD))
+def test_other_sizes(name, dtype, tmp_path):
+    cfg = ODD[name]
+    weights = tiny.random_weights(cfg, seed=3, std=0.06)
+    longest = 128 if cfg["max_position_embeddings"] < 200 else 300
+    requests = {f"r{i}": tiny.random_tokens(cfg, n, 50 + i) for i, n in enumerate([70, 9, longest, 33])}
+    folder = str(tmp_path / "model")
+    tiny.write_model_folder(folder, cfg, weights, torch.float32 if dtype == "float32" else torch.bfloat16)
+    pc, pw = plain_llama.read_model_folder(folder)
+    ref = {rid: plain_llama.forward(pc, pw, toks) for rid, toks in requests.items()}
+    for make in (replay.tail_one_by_one, replay.portions, replay.mixed):
+        trace = make(requests)
+        runner = make_runner(folder, dtype, replay.peak_tokens(trace))
+        rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
+        replay.compare(rows, ref, TOL[dtype])
