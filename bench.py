@@ -119,7 +119,7 @@ def engine_workload(args) -> int:
     server = ServerConfig(
         kv_cache_num_tokens=pool, max_seqs_per_forward=len(lengths), max_tokens_per_forward=8192,
         chunked_prefill_size=chunk, max_prefill_tokens=8192, use_cudagraph=not args.no_graph,
-        cudagraph_max_batch_size=len(lengths),
+        cudagraph_max_batch_size=len(lengths), scheduling_steps_ahead=args.steps_ahead,
     )
     t0 = time.perf_counter()
     runner = ModelRunner.from_random(cfg, seed=0, server_config=server, model_config=ModelConfig(dtype=args.dtype, context_len=8192))
@@ -174,12 +174,14 @@ def engine_workload(args) -> int:
             "prefill_portion": chunk,
             "page_size": runner.cache.page_size,
             "hip_graph": not args.no_graph,
+            "steps_ahead": args.steps_ahead,
             "parallelism": "single GPU",
         },
         "seconds": round(dt, 3),
         "total_tokens_per_second": round((generated + sum(lengths)) / dt, 1),
         "mean_tokens_per_step": round(sum(per_step) / max(1, len(per_step)), 1),
         "retractions": engine.stats.retractions - before[1],
+        "steps_launched_ahead": engine.steps_launched_ahead,
         "weights_gb": round(runner.model.param_bytes() / 1e9, 2),
     }
     print(json.dumps(record), flush=True)
@@ -199,6 +201,8 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the prefill (for profiles)")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill measurement")
+    ap.add_argument("--steps-ahead", type=int, default=1, choices=[0, 1],
+                    help="scheduler workloads: launch decode steps before the tokens of the step before are read")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b"],
                     help="decode8b: the headline line; the others run requests through the scheduler")
     args = ap.parse_args()

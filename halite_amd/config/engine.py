@@ -40,6 +40,12 @@ class ServerConfig(BaseModel):
     max_seqs_per_forward: StrictInt = Field(default=256, gt=0)
     """Most requests that are live (own a slot) at a time."""
 
+    scheduling_steps_ahead: StrictInt = Field(default=0, ge=0, le=1)
+    """1: a decode step is launched before the tokens of the step before it have been
+    read; they reach it on the device (the reference's second engine schedules ahead
+    too, tokainfer/types.py:100-104).  A request that turns out to have stopped leaves
+    one unused row behind."""
+
     # -- ours -----------------------------------------------------------------
     decode_weight_copy: Literal["auto", "on", "off"] = "auto"
     """A second copy of the bf16 matrices in the small-batch kernel's tiled order

@@ -41,6 +41,25 @@ __global__ void embedding_vec_kernel(const int* __restrict__ ids, const TT* __re
   }
 }
 
+// Token ids that an earlier step left on the device: tokens[i] holds a row of `src` on
+// entry and that row's value on return.
+__global__ void take_tokens_kernel(const int* __restrict__ src, int n_src, int* __restrict__ tokens,
+                                   int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int r = tokens[i];
+  tokens[i] = (r >= 0 && r < n_src) ? src[r] : 0;
+}
+
+extern "C" int hal_take_tokens(const int* src, int n_src, int* tokens, int n, hipStream_t stream) {
+  HAL_REQUIRE(n >= 0 && n_src > 0, "hal_take_tokens: bad sizes n=%d n_src=%d", n, n_src);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(take_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, src, n_src,
+                     tokens, n);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" int hal_embedding(const int* ids, const void* table, int table_dtype, float* out,
                              int n_tokens, int d, int vocab, hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && d > 0 && vocab > 0, "hal_embedding: bad sizes T=%d d=%d V=%d",

@@ -14,6 +14,8 @@ int hal_version();
 int hal_embedding(const int* ids, const void* table, int table_dtype, float* out, int n_tokens,
                   int d, int vocab, hipStream_t stream);
 
+int hal_take_tokens(const int* src, int n_src, int* tokens, int n, hipStream_t stream);
+
 int hal_rmsnorm(float* h, const void* delta, const int* rows, const void* w, int w_dtype,
                 float eps, void* out, int dtype, int n_rows, int d, int update_h,
                 hipStream_t stream);

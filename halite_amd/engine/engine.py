@@ -16,6 +16,48 @@ from .scheduler import Request, Scheduler, StepPlan
 from .types import InferenceRequest, InferenceResult
 
 
+class _PinnedRing:
+    """Pinned host buffers for results in flight, used in turn (at most two steps are
+    in flight at a time)."""
+
+    def __init__(self, n=4):
+        self.bufs = [None] * n
+        self.i = 0
+
+    def take(self, words: int) -> torch.Tensor:
+        self.i = (self.i + 1) % len(self.bufs)
+        if self.bufs[self.i] is None or self.bufs[self.i].numel() < words:
+            self.bufs[self.i] = torch.empty(max(2 * words, 1024), dtype=torch.int32, pin_memory=True)
+        return self.bufs[self.i][:words]
+
+
+class _InFlight:
+    """A step on the GPU whose tokens are on their way to the host."""
+
+    def __init__(self, plan: StepPlan, rows: list[Request], pinned: "_PinnedRing"):
+        self.plan, self.rows, self._pinned = plan, rows, pinned
+        self.row_of = {id(r): i for i, r in enumerate(rows)}
+        self.tokens = None  # int32 on the device
+        self._host = self._event = None
+
+    def fetch(self, tokens: torch.Tensor, logprobs: torch.Tensor) -> None:
+        self.tokens = tokens
+        n = tokens.numel()
+        # the two results are the halves of one buffer: one copy
+        both = torch.as_strided(tokens, (2 * n,), (1,)) if tokens.data_ptr() + 4 * n == logprobs.data_ptr() else torch.cat((tokens, logprobs.view(torch.int32)))
+        self._host = self._pinned.take(2 * n)
+        self._host.copy_(both, non_blocking=True)
+        self._event = torch.cuda.Event()
+        self._event.record()
+
+    def result(self) -> tuple[list[int], list[float]]:
+        if self._host is None:
+            return [], []
+        self._event.synchronize()
+        n = self._host.numel() // 2
+        return self._host[:n].tolist(), self._host[n:].view(torch.float32).tolist()
+
+
 class InferenceEngine:
     """``InferenceEngine(model_runner, tokenizer).infer_batch(requests)``.
 
@@ -33,6 +75,8 @@ class InferenceEngine:
         self.model_config = model_runner.model_config
         self.seed = seed
         self.sampler = Sampler(model_runner.device)
+        self._pinned = _PinnedRing()
+        self.steps_launched_ahead = 0
         stop = set(getattr(getattr(model_runner, "config", None), "stop_token_ids", ()) or ())
         if tokenizer is not None:
             if getattr(tokenizer, "eos_id", None) is not None:
@@ -49,29 +93,90 @@ class InferenceEngine:
         return cls(ModelRunner.from_pretrained(folder, server_config, model_config), tokenizer, seed)
 
     # -- the step under the scheduler ------------------------------------------------
-    def _run_step(self, plan: StepPlan):
+    def _launch(self, plan: StepPlan, before: "_InFlight | None" = None) -> "_InFlight":
+        """Puts a step on the GPU and asks for its tokens; does not wait.  ``before`` is a
+        step whose tokens have not been read yet: the requests of ``plan`` (one token
+        each) are one position further than the scheduler knows, and take that token
+        from ``before``'s result on the device."""
         segments, rows = [], []
+        ahead = 0 if before is None else 1
         for i, (r, k) in enumerate(plan.entries):
-            ids = r.ids_between(r.n_cached, r.n_cached + k)
-            wants = plan.wants_logits(i)
-            segments.append(Segment(r.slot, r.n_cached, np.asarray(ids, dtype=np.int32), [k - 1] if wants else []))
+            start = r.n_cached
+            if before is not None:
+                # the scheduler has not counted ``before`` yet; the cache has
+                start = self.model_runner.cache.length(r.slot)
+                ids, wants = [before.row_of[id(r)]], True  # the row of the token, not the token
+            else:
+                ids = r.ids_between(start, start + k)
+                wants = plan.wants_logits(i)
+            segments.append(Segment(r.slot, start, np.asarray(ids, dtype=np.int32), [k - 1] if wants else []))
             if wants:
                 rows.append(r)
-        logits = self.model_runner.step(segments)
-        if not rows:
-            return [], []
-        tokens, logprobs = self.sampler.forward(
-            logits,
-            [r.sampling_params for r in rows],
-            [r.seed for r in rows],
-            [len(r.output_ids) for r in rows],
-        )
-        # the two results are the halves of one buffer: one copy, one wait
-        n = tokens.numel()
-        if tokens.data_ptr() + 4 * n == logprobs.data_ptr():
-            host = torch.as_strided(tokens, (2 * n,), (1,)).cpu()
-            return host[:n].tolist(), host[n:].view(torch.float32).tolist()
-        return tokens.tolist(), logprobs.tolist()
+        logits = self.model_runner.step(segments, token_feed=None if before is None else before.tokens)
+        flight = _InFlight(plan, rows, self._pinned)
+        if rows:
+            tokens, logprobs = self.sampler.forward(
+                logits,
+                [r.sampling_params for r in rows],
+                [r.seed for r in rows],
+                [len(r.output_ids) + ahead for r in rows],
+            )
+            flight.fetch(tokens, logprobs)
+        return flight
+
+    def _run_step(self, plan: StepPlan):
+        return self._launch(plan).result()
+
+    def _decode_again(self, flight: "_InFlight") -> StepPlan | None:
+        """The step after ``flight`` if it can be told without ``flight``'s tokens: nothing
+        waits, every running request gets a token from ``flight``, and those that do not
+        end by length with it decode once more."""
+        sched = self.scheduler
+        if sched.waiting or len(flight.rows) != len(flight.plan.entries):
+            return None
+        if len(sched.running) != len(flight.rows) or any(r.slot is None for r in flight.rows):
+            return None
+        again = [
+            r for r in flight.rows
+            if not r.finished()
+            and len(r.output_ids) + 1 < r.sampling_params.max_new_tokens
+            and r.n_total + 2 <= self.model_runner.context_len
+        ]
+        if not again:
+            return None
+        return StepPlan([(r, 1) for r in again], n_decode=len(again))
+
+    def _run(self) -> None:
+        """Schedules and runs steps until nothing is left.  With
+        ``scheduling_steps_ahead`` a decode step whose requests are known is launched
+        before the tokens of the step before it are read."""
+        from ..cache import NoSpace
+
+        sched = self.scheduler
+        ahead = self.server_config.scheduling_steps_ahead > 0
+        flight = None
+        while True:
+            if flight is None:
+                plan = sched.schedule()
+                if plan is None:
+                    sched.new_token_ratio = sched.init_new_token_ratio
+                    return
+                flight = self._launch(plan)
+                if not ahead:
+                    sched.process_results(plan, *flight.result())
+                    flight = None
+                continue
+            nxt = self._decode_again(flight)
+            following = None
+            if nxt is not None:
+                try:
+                    following = self._launch(nxt, before=flight)
+                    self.steps_launched_ahead += 1
+                    sched.new_token_ratio = max(sched.new_token_ratio - sched.new_token_ratio_decay, sched.min_new_token_ratio)
+                except NoSpace:
+                    following = None  # the scheduler decides what gives way
+            sched.process_results(flight.plan, *flight.result())
+            flight = following
 
     # -- requests ----------------------------------------------------------------------
     def build_batch_request(self, requests) -> list[Request]:
@@ -129,7 +234,7 @@ class InferenceEngine:
                 c.seed = request_seed(req.sampling_params, req.id, self.seed) + j
                 clones.append((req, c))
                 self.scheduler.add_request(c)
-        self.scheduler.run_to_completion()
+        self._run()
         self.scheduler.check_idle()
         self.last_elapsed = time.perf_counter() - t0
         by_id: dict = {}

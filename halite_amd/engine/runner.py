@@ -20,6 +20,7 @@ from ..config.registry import read_config
 from ..parts.decoder import Decoder
 from ..weights import fill_random, load_weights
 from ..kernels import attention as attention_kernels
+from ..kernels import ops
 from .batch import Segment, StaticLayout, StepContext, _Staging
 
 _TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
@@ -87,6 +88,7 @@ class ModelRunner:
         self._graphs: dict[int, dict] = {}
         self._ahead = None  # (requests and positions, cache version, context) of a step put together ahead
         self.steps_taken_ahead = 0
+        self._token_feed = None
         kv_heads = [n.n_kv_heads for n in needs.values()] or [1]
         self._min_kv_heads = min(kv_heads)
         self.graph_replays = 0
@@ -165,7 +167,8 @@ class ModelRunner:
         self.cache.free(slot)
 
     # -- the step ---------------------------------------------------------------------
-    def check_segments(self, segments: list[Segment]) -> None:
+    def check_segments(self, segments: list[Segment], n_ids: int | None = None) -> None:
+        n_ids = self.vocab_size if n_ids is None else n_ids
         seen = set()
         for s in segments:
             if s.slot in seen:
@@ -180,20 +183,28 @@ class ModelRunner:
             if s.start + n > self.context_len:
                 raise StepError(f"slot {s.slot}: {s.start + n} tokens exceed the context length {self.context_len}")
         every = np.concatenate([s.tokens for s in segments]) if len(segments) > 1 else segments[0].tokens
-        if int(every.min()) < 0 or int(every.max()) >= self.vocab_size:
+        if int(every.min()) < 0 or int(every.max()) >= n_ids:
             for s in segments:
                 lo, hi = int(s.tokens.min()), int(s.tokens.max())
-                if lo < 0 or hi >= self.vocab_size:
-                    raise StepError(f"slot {s.slot}: token id {lo if lo < 0 else hi} outside the vocabulary of {self.vocab_size}")
+                if lo < 0 or hi >= n_ids:
+                    raise StepError(f"slot {s.slot}: token id {lo if lo < 0 else hi} outside the vocabulary of {n_ids}")
 
     @torch.no_grad()
-    def step(self, segments: list[Segment]) -> torch.Tensor:
+    def step(self, segments: list[Segment], token_feed=None) -> torch.Tensor:
         """Runs the tokens of ``segments`` and returns float32 logits
         ``[wanted rows, vocab]`` in the order of the segments and of their ``want``.
-        Raises ``NoSpace`` (and changes nothing) if the pages do not suffice."""
+        Raises ``NoSpace`` (and changes nothing) if the pages do not suffice.
+
+        ``token_feed``: int32 token ids on the device (what an earlier step sampled and
+        the host has not read yet).  Every segment then has one token, and
+        ``segments[i].tokens[0]`` is not a token id but the row of ``token_feed`` that
+        holds it."""
         if not segments:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
-        self.check_segments(segments)
+        if token_feed is not None and any(s.tokens.size != 1 for s in segments):
+            raise StepError("tokens can be fed on the device only to segments of one token")
+        self._token_feed = token_feed
+        self.check_segments(segments, self.vocab_size if token_feed is None else token_feed.numel())
         spans = [(s.slot, s.start + s.tokens.size) for s in segments]
         graph_step = (
             self.server_config.use_cudagraph
@@ -210,12 +221,20 @@ class ModelRunner:
             ctx = StepContext(segments, self.cache, self.device, self._staging)
             for run in self.model.runs:
                 self.model.mixer_of_run(run.index).prepare(ctx, run)
+            self._feed_tokens(ctx)
             logits = self.model.forward(ctx)
         for slot, new_len in spans:
             self.cache.advance(slot, new_len)
         if graph_step:
             self._put_step_ahead(segments)
         return logits
+
+    def _feed_tokens(self, ctx) -> None:
+        """Token ids that are still on the device go straight into the step's array, whose
+        entries name their rows until then."""
+        feed, self._token_feed = self._token_feed, None
+        if feed is not None:
+            ops.take_tokens(feed, ctx.tokens)
 
     # While the GPU works on a decode step, the host puts the next one together as far as
     # it can without the tokens: the same requests, one position on.  If that is what
@@ -271,6 +290,7 @@ class ModelRunner:
         if not ctx.fits_static():
             return None
         ctx.upload()
+        self._feed_tokens(ctx)
         if entry["graph"] is None:
             logits = self.model.forward(ctx)  # this step, for real
             graph = torch.cuda.CUDAGraph()

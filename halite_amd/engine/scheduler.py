@@ -297,10 +297,15 @@ class Scheduler:
         return StepPlan(entries, n_decode=len(decoding), n_prefill_tokens=n_prefill)
 
     def process_results(self, plan: StepPlan, tokens: list[int], logprobs: list[float]) -> list[Request]:
-        """Advances the requests of a step that has run; returns those that finished."""
+        """Advances the requests of a step that has run; returns those that finished.  A
+        request that had finished before this step's results were read (the step was
+        launched ahead) is passed over: its row is void."""
         finished = []
         j = 0
         for i, (r, k) in enumerate(plan.entries):
+            if r.finished():
+                j += 1  # only steps of one token each are launched ahead
+                continue
             wants = plan.wants_logits(i)
             r.n_cached += k
             if not wants:

@@ -78,6 +78,16 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None =
     return out
 
 
+def take_tokens(src: torch.Tensor, tokens: torch.Tensor) -> None:
+    """``tokens[i] = src[tokens[i]]`` in place: token ids that an earlier step left on the
+    device go into a step's array without a round over the host."""
+    lib = library.core_library()
+    _dev(src, tokens)
+    _i32(src, "src")
+    _i32(tokens, "tokens")
+    _check(lib, lib.hal_take_tokens(_ptr(src), src.numel(), _ptr(tokens), tokens.numel(), _stream()))
+
+
 def rmsnorm(
     h: torch.Tensor,
     weight: torch.Tensor,

@@ -131,6 +131,45 @@ def test_portions_retraction_and_page_reuse_keep_the_tokens(models):
     assert tight.model_runner.cache.idle()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("graph", [False, True])
+def test_steps_launched_ahead_give_the_same_tokens(models, dtype, graph):
+    """``scheduling_steps_ahead=1``: decode steps are launched before the tokens of the
+    step before them are read.  Lengths that differ, stop tokens that end requests at
+    unknown steps (their next row is void), sampling with seeds, requests that wait for a
+    slot: the outputs equal those of the engine that waits for every step."""
+    folder, pc, pw = models[("B", dtype)]
+    prompts = [tiny.random_tokens(tiny.TINY_B, n, 300 + n) for n in (3, 40, 17, 64, 9, 30)]
+    plain = InferenceEngine.from_pretrained(
+        folder, ServerConfig(kv_cache_num_tokens=2048, max_seqs_per_forward=4, use_cudagraph=graph), ModelConfig(dtype=dtype))
+    ahead = InferenceEngine.from_pretrained(
+        folder, ServerConfig(kv_cache_num_tokens=2048, max_seqs_per_forward=4, use_cudagraph=graph, scheduling_steps_ahead=1),
+        ModelConfig(dtype=dtype))
+    # greedy with stop tokens taken from what the model really generates, so that requests end early
+    free_run = plain.infer_batch([(p, {"max_new_tokens": 24, "temperature": 0.0}) for p in prompts])
+    stops = {r.output_ids[0][5 + i] for i, r in enumerate(free_run)}
+    for params in (
+        [{"max_new_tokens": 5 + 3 * i, "temperature": 0.0} for i in range(6)],
+        [{"max_new_tokens": 24, "temperature": 0.0, "stop_token_ids": sorted(stops)} for _ in range(6)],
+        [{"max_new_tokens": 12, "temperature": 0.9, "top_p": 0.8, "seed": 11 + i} for i in range(6)],
+        [{"max_new_tokens": 1 if i % 2 else 7, "temperature": 0.0} for i in range(6)],
+    ):
+        want = plain.infer_batch(list(zip(prompts, params)))
+        got = ahead.infer_batch(list(zip(prompts, params)))
+        if dtype == "float32" or params[0]["temperature"] == 0.0:
+            assert [r.output_ids for r in got] == [r.output_ids for r in want]
+            assert [r.finish_reason for r in got] == [r.finish_reason for r in want]
+        for a, b in zip(got, want):
+            assert len(a.output_ids[0]) == len(a.output_logprobs[0])
+            if a.output_ids == b.output_ids:
+                assert max(abs(x - y) for x, y in zip(a.output_logprobs[0], b.output_logprobs[0])) < 1e-5
+        if "stop_token_ids" in params[0]:
+            assert sum(r.finish_reason == ["stop"] for r in want) >= 3
+        assert ahead.model_runner.cache.idle() and plain.model_runner.cache.idle()
+    # some steps really were launched ahead
+    assert ahead.steps_launched_ahead > 10 and plain.steps_launched_ahead == 0
+
+
 def test_new_weights_for_a_running_engine(models, tmp_path):
     """``load_state_dict`` takes tensors named as in a model folder: afterwards the
     engine generates what an engine built from those weights generates (graphs that were

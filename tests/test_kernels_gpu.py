@@ -37,6 +37,17 @@ def test_embedding(gpu, dtype, vocab, d):
     assert torch.isnan(bad).all()  # an id outside the table shows, it does not fault
 
 
+def test_take_tokens(gpu):
+    src = torch.randint(0, 50000, (300,), generator=torch.Generator().manual_seed(3), dtype=torch.int32)
+    rows = torch.randperm(300, generator=torch.Generator().manual_seed(4))[:270].to(torch.int32)
+    tokens = rows.to(gpu)
+    ops.take_tokens(src.to(gpu), tokens)
+    assert torch.equal(tokens.cpu(), src[rows.long()])
+    outside = torch.tensor([300, -1, 5], dtype=torch.int32, device=gpu)
+    ops.take_tokens(src.to(gpu), outside)
+    assert outside.tolist() == [0, 0, int(src[5])]  # a row outside the source reads nothing
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("d", [120, 1000, 4096])
 def test_rmsnorm(gpu, dtype, d):
