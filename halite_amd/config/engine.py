@@ -43,7 +43,7 @@ class ServerConfig(BaseModel):
     scheduling_steps_ahead: StrictInt = Field(default=0, ge=0, le=1)
     """1: a decode step is launched before the tokens of the step before it have been
     read; they reach it on the device (the reference's second engine schedules ahead
-    too, tokainfer/types.py:100-104).  A request that turns out to have stopped leaves
+    too, tokainfer/types.py:99).  A request that turns out to have stopped leaves
     one unused row behind."""
 
     # -- ours -----------------------------------------------------------------
