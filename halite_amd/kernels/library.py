@@ -110,9 +110,8 @@ def build_library(name: str, sources: list[str], defines: dict[str, int], force=
     for d in _build_dirs():
         try:
             os.makedirs(d, exist_ok=True)
-            probe = os.path.join(d, f".w{os.getpid()}")
-            with open(probe, "w"):
-                pass
+            fd, probe = tempfile.mkstemp(prefix=".w", dir=d)  # a name of its own: builds run side by side
+            os.close(fd)
             os.remove(probe)
             out_dir = d
             break
