@@ -257,3 +257,36 @@ def test_other_sizes(name, dtype, tmp_path):
         runner = make_runner(folder, dtype, replay.peak_tokens(trace))
         rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
         replay.compare(rows, ref, TOL[dtype])
+
+
+LLAMA_8B_LAYERS = dict(
+    architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=4096, num_attention_heads=32,
+    num_key_value_heads=8, head_dim=128, intermediate_size=14336, vocab_size=128256, num_hidden_layers=2,
+    rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=8192, tie_word_embeddings=False,
+    hidden_act="silu", attention_bias=False, mlp_bias=False,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_of_the_8b_shape(dtype, tmp_path):
+    """Two layers with every size of Llama-3.1-8B (width 4096, 32 heads over 8 groups of
+    128, feed-forward 14336, vocabulary 128256, llama3 frequency scaling), weights
+    N(0, 0.02): the kernels at the sizes that the benchmark runs."""
+    cfg = LLAMA_8B_LAYERS
+    weights = tiny.random_weights(cfg, seed=11, std=0.02)
+    requests = {f"r{i}": tiny.random_tokens(cfg, n, 70 + i) for i, n in enumerate([70, 9, 200, 33])}
+    folder = str(tmp_path / "model")
+    tiny.write_model_folder(folder, cfg, weights, torch.float32 if dtype == "float32" else torch.bfloat16)
+    del weights
+    pc, pw = plain_llama.read_model_folder(folder)
+    ref = {rid: plain_llama.forward(pc, pw, toks) for rid, toks in requests.items()}
+    del pw
+    runner = None
+    for make in (replay.tail_one_by_one, replay.portions, replay.mixed):
+        trace = make(requests)
+        del runner
+        runner = make_runner(folder, dtype, replay.peak_tokens(trace))
+        rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
+        replay.compare(rows, ref, TOL[dtype])
