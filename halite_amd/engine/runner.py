@@ -11,6 +11,8 @@ decode passes; the mixed flat batch is the ``tokainfer`` engine's
 
 from __future__ import annotations
 
+import gc
+
 import numpy as np
 import torch
 
@@ -294,8 +296,17 @@ class ModelRunner:
         if entry["graph"] is None:
             logits = self.model.forward(ctx)  # this step, for real
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                entry["logits"] = self.model.forward(ctx)  # recorded, not run
+            # No garbage collection while the stream records: a graph of an engine that
+            # is no longer used would be destroyed in the middle of it, which HIP refuses.
+            gc.collect()
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    entry["logits"] = self.model.forward(ctx)  # recorded, not run
+            finally:
+                if collecting:
+                    gc.enable()
             entry["graph"], entry["ctx"] = graph, ctx
             return logits
         entry["graph"].replay()

@@ -216,3 +216,25 @@ def test_command_line(models, tmp_path):
     proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "halite_make_random_model"), "--config", str(cfgfile),
                            "--out", str(out), "--seed", "3", "--dtype", "float32"], capture_output=True, text=True)
     assert proc.returncode == 0 and (out / "model.safetensors").exists() and (out / "config.json").exists()
+
+
+def test_a_dropped_engine_does_not_disturb_a_capture(models):
+    """An engine that is no longer referenced still holds captured graphs until the garbage
+    collector finds it; that must not happen while another engine records one."""
+    import gc
+
+    folder, pc, pw = models[("A", "float32")]
+    server = ServerConfig(kv_cache_num_tokens=512, use_cudagraph=True)
+    prompt = tiny.random_tokens(tiny.TINY_A, 12, 3)
+    params = {"max_new_tokens": 6, "temperature": 0.0}
+    first = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="float32"))
+    want = first.infer_batch([(prompt, params)])[0].output_ids[0]
+    assert first.model_runner._graphs
+    del first  # garbage with reference cycles: only the collector frees it
+    old = gc.get_threshold()
+    gc.set_threshold(1, 1, 1)  # collect at every opportunity
+    try:
+        second = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="float32"))
+        assert second.infer_batch([(prompt, params)])[0].output_ids[0] == want
+    finally:
+        gc.set_threshold(*old)
