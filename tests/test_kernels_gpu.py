@@ -294,6 +294,63 @@ def test_attention_mfma_split_keys(gpu):
     attention_case(gpu, "bfloat16", 4, 1, 64, 32, [(3000, 50), (0, 600)], 700, seed=46, use="mfma", tiled=True)
 
 
+@pytest.mark.parametrize("tiled", [False, True])
+def test_attention_mfma_hundred_thousand_keys(gpu, tiled):
+    """One decoded token against 100,003 cached keys: the key range is cut into far more
+    pieces than a wave of the merge kernel joins at once.  The key that decides the
+    result lies in the middle of a piece far from both ends."""
+    H, K, D, page, n = 8, 2, 128, 64, 100_003
+    dt = torch.bfloat16
+    k = rnd(n, K, D, seed=60).to(dt).float()
+    v = rnd(n, K, D, seed=61).to(dt).float()
+    q = rnd(1, H, D, seed=62).to(dt).float()
+    far = 61_007
+    k[far] = 0
+    k[far, :, 1] = 10.0
+    q[0, :, 1] = 16.0  # the far key gets about as much weight as all the others together
+    v[far] = 3.0
+    scale = D**-0.5
+    want = torch.empty(H, D, dtype=torch.float64)
+    for h in range(H):
+        g = h // (H // K)
+        p = torch.softmax((k[:, g].double() @ q[0, h].double()) * scale, dim=0)
+        want[h] = p @ v[:, g].double()
+    assert float(want.abs().max()) > 1.0  # the far key carries weight
+    n_logical = -(-n // page)
+    perm = torch.randperm(n_logical + 3, generator=torch.Generator().manual_seed(63))[:n_logical] + 1
+    pad = n_logical * page - n
+    kl = torch.cat((k, torch.full((pad, K, D), float("nan")))).view(n_logical, page, K, D)
+    vl = torch.cat((v, torch.full((pad, K, D), float("nan")))).view(n_logical, page, K, D)
+    kp = torch.full((n_logical + 4, K, page, D), float("nan"))
+    vp = torch.full((n_logical + 4, K, D, page), float("nan"))
+    kp[perm] = kl.permute(0, 2, 1, 3)
+    vp[perm] = vl.permute(0, 2, 3, 1)
+    kp, vp = kp.to(dt), vp.to(dt)
+    if tiled:
+        kp, vp = to_tiled(kp, vp)
+    q_len, kv_len = np.array([1], dtype=np.int32), np.array([n], dtype=np.int32)
+    plan = attn_kernels.plan_items(q_len, kv_len, H // K, K, 0, attn_kernels.rows_per_big_item(D))
+    assert plan.n_merges == 1 and plan.n_items > 64  # more than 64 partial results per row
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+
+    class Ctx:
+        n_tokens = 1
+        seg_q_start = dev(np.array([0], dtype=np.int32))
+        seg_q_len = dev(q_len)
+        seg_kv_len = dev(kv_len)
+
+    class Group:
+        block_table = perm.to(torch.int32).view(1, -1).to(gpu)
+
+    class KV:
+        pass
+
+    KV.k, KV.v, KV.tiled = kp.to(gpu), vp.to(gpu), tiled
+    out = attn_kernels.attention_mfma(q.view(1, H * D).to(dt).to(gpu), H * D, attn_kernels.upload_plan(plan, gpu),
+                                      Ctx, Group, KV, H, scale, 0)
+    close(out, want.float().view(1, H * D), 1.2e-2, "attention over 100,003 keys")
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 256, 64), (5, 331, 120), (64, 200, 352), (130, 96, 1000), (3, 4096, 4096)])
 def test_gemm_f32(gpu, M, N, K):
     a, w = rnd(M, K, seed=50), rnd(N, K, seed=51)
