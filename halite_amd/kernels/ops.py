@@ -290,6 +290,18 @@ def sample(
 
 SKINNY_MAX_ROWS = 64  # what the kernel takes
 SKINNY_ROWS = 16  # up to here it beats the library product
+# ... if the weights lie in its tiled order.  On row-major weights (a model too large for
+# the second copy) it wins only on small matrices or a single row: measured on Llama-3.1-70B
+# shapes at 8 and 16 rows, the library reads 4.7-5.5 TB/s where the kernel reads 3.2-4.6.
+ROW_MAJOR_SKINNY_ELEMENTS = 32 * 1024 * 1024
+
+
+def skinny_pays(m: int, n: int, k: int, tiled: bool) -> bool:
+    """Whether the small-batch kernel is the faster way for ``m`` rows against an
+    ``[n, k]`` bf16 weight."""
+    if m > SKINNY_ROWS:
+        return False
+    return tiled or m == 1 or n * k <= ROW_MAJOR_SKINNY_ELEMENTS
 _MM_OUT_DTYPE = None  # whether torch.mm takes out_dtype (found at first use)
 
 
@@ -360,10 +372,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
     model keeps that copy for small batches.
 
     float32 weights: the true 32-bit kernel (activations are widened if needed).
-    bf16 weights: the hand-written kernel for up to 64 rows; for more rows the
-    library product that the reference itself uses for its linear layers
-    (src/halite/transformers/infer/attention.py:21-24), except where float32
-    output is asked for, which the hand-written kernel gives in passes of 64 rows.
+    bf16 weights: the hand-written kernel where it is the faster one (``skinny_pays``:
+    up to 16 rows); otherwise the library product that the reference itself uses for
+    its linear layers (src/halite/transformers/infer/attention.py:21-24), except where
+    float32 output is asked for and the library cannot give it, which the hand-written
+    kernel does in passes of 64 rows.
     """
     out_dtype = out_dtype or x.dtype
     if w.dtype == torch.float32:
@@ -376,7 +389,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
     skinny_ok = k % 8 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
     if m <= SKINNY_ROWS and tiled is not None and k % 8 == 0:
         return gemm_bf16_skinny(x, tiled, out_dtype=out_dtype, tiled_shape=tuple(w.shape))
-    if skinny_ok and m <= SKINNY_ROWS:
+    if skinny_ok and skinny_pays(m, w.shape[0], k, False):
         return gemm_bf16_skinny(x, w, out_dtype=out_dtype)
     if out_dtype == torch.float32:
         global _MM_OUT_DTYPE

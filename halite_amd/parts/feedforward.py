@@ -71,7 +71,7 @@ class GatedFeedForward(FeedForward):
         fused = (
             w.dtype == torch.bfloat16
             and x.dtype == torch.bfloat16
-            and x.shape[0] <= ops.SKINNY_ROWS
+            and ops.skinny_pays(x.shape[0], f, x.shape[1], False)
             and x.shape[1] % 8 == 0
             and (f * x.shape[1]) % 8 == 0
         )
