@@ -83,7 +83,8 @@ class InferenceEngine:
                 stop.add(tokenizer.eos_id)
             stop.update(getattr(tokenizer, "additional_stop_token_ids", None) or ())
         self.scheduler = Scheduler(
-            model_runner.cache, self.server_config, self._run_step, model_runner.context_len, stop
+            model_runner.cache, self.server_config, self._run_step, model_runner.context_len, stop,
+            vocab_size=model_runner.vocab_size,
         )
         self.initialized = True
 
@@ -233,8 +234,16 @@ class InferenceEngine:
                 c = Request((req.id, j), req.input_ids, req.sampling_params, req.input_text)
                 c.seed = request_seed(req.sampling_params, req.id, self.seed) + j
                 clones.append((req, c))
+        for _, c in clones:  # all of them are looked at before the first is queued
+            self.scheduler.check_request(c)
+        try:
+            for _, c in clones:
                 self.scheduler.add_request(c)
-        self._run()
+            self._run()
+        except BaseException:
+            # nothing of a failed batch stays behind: the engine serves the next one
+            self.scheduler.abort_all()
+            raise
         self.scheduler.check_idle()
         self.last_elapsed = time.perf_counter() - t0
         by_id: dict = {}

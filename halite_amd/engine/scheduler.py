@@ -133,11 +133,13 @@ class Scheduler:
         run_step: RunStep,
         context_len: int,
         stop_token_ids=(),
+        vocab_size: int | None = None,
     ):
         self.cache = cache
         self.conf = server_config
         self.run_step = run_step
         self.context_len = context_len
+        self.vocab_size = vocab_size
         self.stop_token_ids = set(stop_token_ids)
         c = server_config
         self.init_new_token_ratio = min(c.default_init_new_token_ratio * c.schedule_conservativeness, 1.0)
@@ -154,10 +156,17 @@ class Scheduler:
         self.stats = SchedulerStats()
 
     # -- submission -----------------------------------------------------------------
-    def add_request(self, req: Request) -> None:
+    def check_request(self, req: Request) -> None:
+        """Raises ``ValueError`` for a request that can never be served."""
         p = req.sampling_params
         if not req.input_ids:
             raise ValueError(f"request {req.id!r}: empty prompt")
+        if self.vocab_size is not None:
+            lo, hi = min(req.input_ids), max(req.input_ids)
+            if lo < 0 or hi >= self.vocab_size:
+                raise ValueError(
+                    f"request {req.id!r}: token id {lo if lo < 0 else hi} outside the vocabulary of {self.vocab_size}"
+                )
         longest = len(req.input_ids) + p.max_new_tokens
         if longest > self.context_len:
             raise ValueError(
@@ -169,7 +178,21 @@ class Scheduler:
                 f"request {req.id!r}: {longest} tokens can never fit the cache pool of "
                 f"{self.cache.token_capacity} tokens"
             )
+
+    def add_request(self, req: Request) -> None:
+        self.check_request(req)
         self.waiting.append(req)
+
+    def abort_all(self) -> None:
+        """Drops every request, waiting or running, and gives back what they hold (after
+        an error in the middle of a batch)."""
+        for req in self.running:
+            if req.slot is not None:
+                self.cache.free(req.slot)
+                req.slot = None
+        self.waiting.clear()
+        self.running = []
+        self.new_token_ratio = self.init_new_token_ratio
 
     def _pages_for(self, n_tokens: int) -> int:
         return max(g.pages_per_token_span(n_tokens) for g in self.cache.groups)

@@ -238,3 +238,43 @@ def test_a_dropped_engine_does_not_disturb_a_capture(models):
         assert second.infer_batch([(prompt, params)])[0].output_ids[0] == want
     finally:
         gc.set_threshold(*old)
+
+
+def test_the_engine_serves_on_after_a_refused_or_failed_batch(models):
+    """Requests that can never be served are refused before any of the batch is queued,
+    and whatever fails later leaves nothing behind: the next batch gives what it gave
+    before."""
+    folder, pc, pw = models[("A", "float32")]
+    cfg = tiny.TINY_A
+    engine = InferenceEngine.from_pretrained(folder, ServerConfig(kv_cache_num_tokens=64, page_size=16), ModelConfig(dtype="float32"))
+    good = (tiny.random_tokens(cfg, 10, 1), {"max_new_tokens": 5, "temperature": 0.0})
+    want = engine.infer_batch([good])[0].output_ids
+    refused = [
+        ((tiny.random_tokens(cfg, 100, 2), {"max_new_tokens": 20}), "can never fit"),
+        ((tiny.random_tokens(cfg, 200, 2), {"max_new_tokens": 2}), "exceeds the context length"),
+        (([5, cfg["vocab_size"]], {"max_new_tokens": 2}), "outside the vocabulary"),
+        (([], {"max_new_tokens": 2}), "empty prompt"),
+        ((tiny.random_tokens(cfg, 5, 2), {"max_new_tokens": 2, "temperature": -1.0}), "temperature"),
+        ((tiny.random_tokens(cfg, 5, 2), {"nonsense": 2}), "nonsense"),
+    ]
+    for bad, message in refused:
+        with pytest.raises((ValueError, TypeError), match=message):
+            engine.infer_batch([good, bad])  # the good request before it is not left waiting
+        assert not engine.scheduler.waiting and not engine.scheduler.running
+        assert engine.infer_batch([good])[0].output_ids == want
+    # a failure in the middle of the run (the step function raises): the batch is dropped
+    calls = {"n": 0}
+    step = engine.model_runner.step
+
+    def failing_step(segments, token_feed=None):
+        calls["n"] += 1
+        if calls["n"] == 3:
+            raise RuntimeError("stand-in for a failure inside a step")
+        return step(segments, token_feed=token_feed)
+
+    engine.model_runner.step = failing_step
+    with pytest.raises(RuntimeError, match="stand-in"):
+        engine.infer_batch([good, (tiny.random_tokens(cfg, 7, 3), {"max_new_tokens": 9, "temperature": 0.0})])
+    engine.model_runner.step = step
+    assert engine.model_runner.cache.idle()
+    assert engine.infer_batch([good])[0].output_ids == want

@@ -205,3 +205,29 @@ def test_admission_reserves_for_running_requests():
     done = sched.run_to_completion()
     assert len(done) == 3 and sched.stats.retractions == 0
     assert sched.stats.max_running == 2  # 2 * 40 tokens fit 80, the third waits
+
+
+def test_requests_are_checked_before_they_wait_and_a_batch_can_be_dropped():
+    sched, model, cache = make()
+    sched.vocab_size = 97
+    with pytest.raises(ValueError, match="outside the vocabulary of 97"):
+        sched.add_request(Request("bad", [3, 97, 5], SamplingParams(max_new_tokens=4)))
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        sched.add_request(Request("neg", [3, -1], SamplingParams(max_new_tokens=4)))
+    with pytest.raises(ValueError, match="empty prompt"):
+        sched.add_request(Request("empty", [], SamplingParams(max_new_tokens=4)))
+    assert not sched.waiting
+    # a batch that is given up half way: slots and pages come back, the queues are empty
+    for i in range(3):
+        sched.add_request(Request(i, [1 + i] * (9 + i), SamplingParams(max_new_tokens=30, ignore_eos=True)))
+    for _ in range(4):
+        plan = sched.schedule()
+        sched.process_results(plan, *model(plan))
+    assert sched.running and not cache.idle()
+    sched.abort_all()
+    assert not sched.running and not sched.waiting and cache.idle()
+    cache.check()
+    sched.add_request(Request("next", [5, 6, 7], SamplingParams(max_new_tokens=6, ignore_eos=True)))
+    while (plan := sched.schedule()) is not None:
+        sched.process_results(plan, *model(plan))
+    assert cache.idle()
