@@ -33,8 +33,8 @@ def parse_args(argv=None):
     ap.add_argument("--prompt-seed", type=int, default=0)
     ap.add_argument("--seed", type=int, default=0, help="engine seed for sampling streams")
     ap.add_argument("--stats", action="store_true", help="print scheduler statistics to stderr")
-    ap.add_argument("opts", default=None, nargs=argparse.REMAINDER, help="key=value overrides")
-    return ap.parse_args(argv)
+    ap.add_argument("opts", default=[], nargs="*", help="key=value overrides")
+    return ap.parse_intermixed_args(argv)  # overrides and options in any order
 
 
 def split_overrides(opts):
@@ -48,7 +48,20 @@ def split_overrides(opts):
 
 
 def main(argv=None) -> int:
+    """Runs ``generate`` and turns what a user can get wrong (a folder, an option, a
+    request) into one line on stderr and exit status 2."""
+    from ..config.registry import ConfigError
+    from ..weights import WeightError
+
     args = parse_args(argv)
+    try:
+        return generate(args)
+    except (ConfigError, WeightError, ValueError, TypeError, FileNotFoundError) as e:
+        print(f"halite_generate: error: {e}", file=sys.stderr)
+        return 2
+
+
+def generate(args) -> int:
     over = split_overrides(args.opts)
     from ..engine import InferenceEngine
     from ..sampling import SamplingParams

@@ -123,3 +123,15 @@ def test_engine_options_and_overrides():
         ModelConfig(dtype="float16")
     with pytest.raises(ValueError, match="key=value"):
         parse_overrides(["page_size"])
+
+
+def test_command_line_takes_overrides_and_options_in_any_order():
+    from halite_amd.cli.generate import parse_args, split_overrides
+
+    args = parse_args(["--model", "DIR", "sampling.max_new_tokens=4", "--prompt-ids", "1,2,3",
+                       "server.page_size=16", "--stats", "model.dtype=float32"])
+    assert args.model == "DIR" and args.prompt_ids == ["1,2,3"] and args.stats
+    over = split_overrides(args.opts)
+    assert over == {"sampling": {"max_new_tokens": 4}, "server": {"page_size": 16}, "model": {"dtype": "float32"}}
+    with pytest.raises(SystemExit):
+        split_overrides(["foo=1"])
