@@ -290,3 +290,25 @@ def test_layers_of_the_8b_shape(dtype, tmp_path):
         runner = make_runner(folder, dtype, replay.peak_tokens(trace))
         rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
         replay.compare(rows, ref, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompts_with_the_heads_of_the_8b_shape(dtype, tmp_path):
+    """Prompts of thousands of tokens through two layers with 32 heads over 8 groups of
+    128 (a small vocabulary keeps the test short): the prompt kernels walk dozens of
+    blocks of keys, whole, in portions and mixed with other requests."""
+    cfg = dict(LLAMA_8B_LAYERS, vocab_size=4096)
+    weights = tiny.random_weights(cfg, seed=11, std=0.02)
+    requests = {f"r{i}": tiny.random_tokens(cfg, n, 70 + i) for i, n in enumerate([3000, 700, 33])}
+    folder = str(tmp_path / "model")
+    tiny.write_model_folder(folder, cfg, weights, torch.float32 if dtype == "float32" else torch.bfloat16)
+    del weights
+    pc, pw = plain_llama.read_model_folder(folder)
+    ref = {rid: plain_llama.forward(pc, pw, toks) for rid, toks in requests.items()}
+    del pw
+    for make in (replay.whole, replay.portions, replay.mixed):
+        trace = make(requests)
+        runner = make_runner(folder, dtype, replay.peak_tokens(trace))
+        rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
+        replay.compare(rows, ref, TOL[dtype])
+        del runner
