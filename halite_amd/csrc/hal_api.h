@@ -44,19 +44,6 @@ int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, float* C, int
 int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const void* W2, int ldw, void* C,
                          int ldc, int out_mode, int M, int N, int K, hipStream_t stream);
 
-// The same for at most 16 rows with what surrounds the product in a layer folded in.  With
-// xh, X is not read: its rows are RMSNorm(xh) with weight norm_w (bf16 or float32, by
-// norm_w_dtype), computed from the float32 stream xh [M, ldxh] and ss_parts partial sums of
-// squares of its rows, ss_in [ss_parts][ss_ld].  With ss_out (out_mode 2, one weight), block b
-// of the hal_gemm_bf16_skinny_blocks(M, N, 0) blocks writes the sums of squares of its columns
-// of the new C to ss_out[b * ss_out_ld + row].
-int hal_gemm_bf16_skinny_blocks(int M, int N, int gated);
-int hal_gemm_bf16_skinny_fused(const void* W, const void* W2, int ldw, void* C, int ldc,
-                               int out_mode, int M, int N, int K, const void* X, int ldx,
-                               const float* xh, int ldxh, const float* ss_in, int ss_parts,
-                               int ss_ld, const void* norm_w, int norm_w_dtype, float eps,
-                               float* ss_out, int ss_out_ld, hipStream_t stream);
-
 int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temperature,
                const int* top_k, const float* top_p, const float* min_p, const uint64_t* seeds,
                const int* draw_index, int* out_token, float* out_logprob, uint32_t* key_rows,

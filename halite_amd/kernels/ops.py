@@ -320,51 +320,19 @@ def tile_weight(w: torch.Tensor) -> torch.Tensor:
     return t.contiguous().view(-1)
 
 
-SS_ROWS = 16  # rows of a table of partial sums of squares
-
-
-class NormedRows:
-    """Rows of ``rmsnorm(h) * weight`` that are not computed yet: the float32 stream ``h``
-    ``[rows, d]`` (at most 16 rows), partial sums of squares of its rows ``ss``
-    ``[parts, SS_ROWS]``, the norm's weight and eps, and the activation type.  The
-    small-batch product computes them while it loads them; ``tensor()`` computes them
-    with the norm kernel for everything else."""
-
-    def __init__(self, h, ss, weight, eps, dtype):
-        self.h, self.ss, self.weight, self.eps, self.dtype = h, ss, weight, eps, dtype
-        self.shape, self.device = h.shape, h.device
-
-    def tensor(self) -> torch.Tensor:
-        return rmsnorm(self.h, self.weight, self.eps, self.dtype)
-
-
 def gemm_bf16_skinny(
-    x,
+    x: torch.Tensor,
     w: torch.Tensor,
     w_up: torch.Tensor | None = None,
     out_dtype: torch.dtype = torch.bfloat16,
     add_to: torch.Tensor | None = None,
     tiled_shape: tuple[int, int] | None = None,
-    sums_of_squares: bool = False,
 ):
     """``x @ w.T`` for at most 64 rows of bf16 ``x``; with ``w_up`` the gated form
-    ``(x @ w_up.T) * silu(x @ w.T)``; ``add_to`` (float32) receives ``+=``.
-
-    ``x`` may be ``NormedRows`` (at most 16 rows).  ``sums_of_squares`` (with ``add_to``, at
-    most 16 rows): also returns partial sums of squares of the new rows of ``add_to``,
-    ``[parts, SS_ROWS]``, as ``NormedRows`` takes them."""
+    ``(x @ w_up.T) * silu(x @ w.T)``; ``add_to`` (float32) receives ``+=``."""
     lib = library.core_library()
-    normed = x if isinstance(x, NormedRows) else None
-    if normed is not None:
-        _dev(normed.h, normed.ss, normed.weight, add_to)
-        _need(normed.h.dtype == torch.float32 and normed.ss.dtype == torch.float32 and normed.h.dim() == 2
-              and normed.h.shape[0] <= SS_ROWS and normed.ss.dim() == 2 and normed.ss.shape[1] == SS_ROWS
-              and normed.weight.numel() == normed.h.shape[1]
-              and normed.weight.dtype in (torch.float32, torch.bfloat16) and normed.dtype == torch.bfloat16,
-              "skinny gemm: rows to be normalised")
-    else:
-        _dev(x, add_to)
-        _need(x.dtype == torch.bfloat16, "skinny gemm takes bf16")
+    _dev(x, add_to)
+    _need(x.dtype == torch.bfloat16, "skinny gemm takes bf16")
     m, k = x.shape
     if tiled_shape is not None:  # weights from tile_weight()
         n, k2 = tiled_shape
@@ -389,30 +357,13 @@ def gemm_bf16_skinny(
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
         mode = 0 if out_dtype == torch.bfloat16 else 1
         _need(out_dtype in (torch.bfloat16, torch.float32), "skinny gemm: output dtype")
-    if normed is None and not sums_of_squares:
-        _check(
-            lib,
-            lib.hal_gemm_bf16_skinny(
-                _ptr(x), k, _ptr(w), _ptr(w_up), ldw, _ptr(out), n, mode, m, n, k, _stream()
-            ),
-        )
-        return out
-    ss_out = None
-    if sums_of_squares:
-        _need(add_to is not None and m <= SS_ROWS and w_up is None, "skinny gemm: sums of squares")
-        ss_out = torch.empty((lib.hal_gemm_bf16_skinny_blocks(m, n, 0), SS_ROWS), dtype=torch.float32, device=out.device)
     _check(
         lib,
-        lib.hal_gemm_bf16_skinny_fused(
-            _ptr(w), _ptr(w_up), ldw, _ptr(out), n, mode, m, n, k,
-            _ptr(None if normed else x), 0 if normed else k,
-            _ptr(normed.h if normed else None), k if normed else 0,
-            _ptr(normed.ss if normed else None), normed.ss.shape[0] if normed else 0, SS_ROWS,
-            _ptr(normed.weight if normed else None), dtype_code(normed.weight.dtype) if normed else 0,
-            ctypes.c_float(normed.eps if normed else 0.0), _ptr(ss_out), SS_ROWS, _stream(),
+        lib.hal_gemm_bf16_skinny(
+            _ptr(x), k, _ptr(w), _ptr(w_up), ldw, _ptr(out), n, mode, m, n, k, _stream()
         ),
     )
-    return (out, ss_out) if sums_of_squares else out
+    return out
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None,

@@ -390,59 +390,6 @@ def test_gemm_bf16_skinny(gpu, M, N, K):
     assert torch.equal(a, b)
 
 
-@pytest.mark.parametrize("wdt", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("M,N,K", [(1, 256, 64), (5, 331, 120), (8, 1000, 352), (16, 4096, 4096), (3, 200, 4104)])
-def test_gemm_bf16_skinny_with_the_norm_before_and_the_sums_after(gpu, M, N, K, wdt):
-    """The product takes its rows from the float32 stream and normalises them on the way
-    (partial sums of squares come in), and after adding into the stream it hands out the
-    partial sums of squares of the new rows: a chain of two such products against the
-    plain formulas."""
-    eps = 2e-6
-    h = rnd(M, K, seed=64, scale=1.5)
-    nw = (1 + 0.2 * rnd(K, seed=65)).to(wdt)
-    w = rnd(N, K, seed=66, scale=0.05).to(torch.bfloat16)
-    w2 = rnd(N, K, seed=67, scale=0.05).to(torch.bfloat16)
-    parts = 7  # partial sums over seven unequal runs of columns
-    cuts = [0] + sorted(torch.randperm(K - 1, generator=torch.Generator().manual_seed(68))[: parts - 1].add(1).tolist()) + [K]
-    ss = torch.zeros(parts, ops.SS_ROWS)
-    for p in range(parts):
-        ss[p, :M] = h[:, cuts[p] : cuts[p + 1]].pow(2).sum(-1)
-    x = (nw.float() * (h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + eps)).to(torch.bfloat16).float()).to(torch.bfloat16)
-    want = x.float() @ w.float().T
-    hg, wg, w2g = h.to(gpu), w.to(gpu), w2.to(gpu)
-    normed = ops.NormedRows(hg, ss.to(gpu), nw.to(gpu), eps, torch.bfloat16)
-    close(normed.tensor(), x.float(), 1e-2, "the rows by the norm kernel")
-    close(ops.gemm_bf16_skinny(normed, wg, out_dtype=torch.float32), want, 4e-3, "normalised on the way")
-    tw, tw2 = ops.tile_weight(wg), ops.tile_weight(w2g)
-    a = ops.gemm_bf16_skinny(normed, wg, out_dtype=torch.float32)
-    assert torch.equal(a, ops.gemm_bf16_skinny(normed, tw, out_dtype=torch.float32, tiled_shape=(N, K)))
-    # against the same rows computed first: the sums of squares are added in another order,
-    # so a value may fall on the other side of a rounding now and then
-    close(a, ops.gemm_bf16_skinny(normed.tensor(), wg, out_dtype=torch.float32), 4e-3, "both ways")
-    up = x.float() @ w2.float().T
-    close(ops.gemm_bf16_skinny(normed, tw, w_up=tw2, out_dtype=torch.float32, tiled_shape=(N, K)),
-          up * want * torch.sigmoid(want), 4e-3, "gated, normalised on the way")
-    # adding into a stream and the sums of squares of what comes out
-    base = rnd(M, N, seed=69)
-    acc = base.to(gpu).clone()
-    xb = x.to(gpu)
-    out, sums = ops.gemm_bf16_skinny(xb, wg, add_to=acc, sums_of_squares=True)
-    assert out.data_ptr() == acc.data_ptr() and sums.shape[1] == ops.SS_ROWS
-    close(acc, base + want, 2e-5, "added")
-    got = sums[:, :M].sum(0).cpu()
-    assert torch.allclose(got, (base + want).pow(2).sum(-1), rtol=2e-5), "sums of squares"
-    # ... which feed the next product
-    nw2 = (1 + 0.2 * rnd(N, seed=70)).to(wdt)
-    w3 = rnd(77, N, seed=71, scale=0.05).to(torch.bfloat16)
-    if N % 8 == 0:
-        nxt = ops.gemm_bf16_skinny(ops.NormedRows(acc, sums, nw2.to(gpu), eps, torch.bfloat16), w3.to(gpu), out_dtype=torch.float32)
-        h2 = base + want
-        x2 = (nw2.float() * (h2 * torch.rsqrt(h2.pow(2).mean(-1, keepdim=True) + eps)).to(torch.bfloat16).float()).to(torch.bfloat16)
-        close(nxt, x2.float() @ w3.float().T, 4e-3, "the chain")
-    with pytest.raises(ops.KernelError):
-        ops.gemm_bf16_skinny(ops.NormedRows(rnd(17, K).to(gpu), ss.to(gpu), nw.to(gpu), eps, torch.bfloat16), wg)
-
-
 def test_linear_dispatch(gpu):
     x = rnd(100, 352, seed=70).to(torch.bfloat16).to(gpu)
     w = rnd(331, 352, seed=71, scale=0.05)
