@@ -13,7 +13,6 @@ from dataclasses import dataclass
 import torch
 
 from ..config.spec import ModelSpec
-from ..kernels import ops
 from .base import (
     ARRANGEMENTS,
     EMBEDDINGS,

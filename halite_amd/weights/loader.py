@@ -15,8 +15,6 @@ tables become int32.
 
 from __future__ import annotations
 
-import re
-
 import torch
 
 from ..parts.decoder import Decoder

@@ -7,9 +7,6 @@ the way that program does; ``collect`` puts the logits back together per request
 
 import random
 
-import numpy as np
-import torch
-
 from halite_amd.engine.batch import Segment
 
 

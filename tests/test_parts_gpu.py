@@ -3,7 +3,6 @@ layer that runs twice, a layer that reads another layer's cache, and toy parts t
 defined here and registered without touching the framework: a mixer with state of its
 own, a feed-forward that routes tokens to experts, and another position encoding."""
 
-import numpy as np
 import pytest
 import torch
 from pydantic import BaseModel
