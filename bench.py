@@ -201,6 +201,8 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the prefill (for profiles)")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill measurement")
+    ap.add_argument("--prefill-portion", type=int, default=0,
+                    help="run the prompt of the prefill measurement in portions of this many tokens (0: whole)")
     ap.add_argument("--steps-ahead", type=int, default=1, choices=[0, 1],
                     help="scheduler workloads: launch decode steps before the tokens of the step before are read")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b"],
@@ -286,7 +288,10 @@ def main() -> int:
             s = runner.admit()
             sync()
             t0 = time.perf_counter()
-            logits = runner.step([Segment(s, 0, ids, [T - 1])])
+            portion = args.prefill_portion or T
+            for start in range(0, T, portion):  # the whole prompt, or one portion a step
+                end = min(start + portion, T)
+                logits = runner.step([Segment(s, start, ids[start:end], [end - start - 1] if end == T else [])])
             tok, _ = sampler.forward(logits, [greedy], [0], [0])
             tok.tolist()
             sync()
