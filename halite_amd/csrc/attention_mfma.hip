@@ -46,6 +46,7 @@ static_assert(HAL_HEAD_DIM % 16 == 0 && HAL_HEAD_DIM >= 16 && HAL_HEAD_DIM <= 25
 #define DT (D / 16)         // 16-wide tiles of the head dimension for P V
 #define ITEM_INTS 8
 #define RESCALE_SLACK 8.0f  // in powers of two
+#define MERGE_FEW_PARTS 8   // up to here a merge item is one wave's work
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -607,6 +608,58 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
   }
 }
 
+// The same for merge items of few partials (prompt portions whose key range was cut in
+// two or three): a wave per row, four rows per block, no LDS and no barrier; the
+// partials are added in their order.
+__global__ void __launch_bounds__(256)
+attention_merge_few_kernel(bf16_t* __restrict__ out, int out_row_stride,
+                           const int* __restrict__ merges, const int* __restrict__ n_merges_ptr,
+                           const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
+                           const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                           int H, int K) {
+  constexpr int NC = (D + 127) / 128;
+  const int mi = blockIdx.x;
+  if (mi >= *n_merges_ptr) return;
+  const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
+  const int g = blockIdx.y, row = blockIdx.z * 4 + wave;
+  const int G = H / K;
+  const int* mg = merges + (size_t)mi * ITEM_INTS;
+  const int seg = mg[0], rho0 = mg[1], first = mg[2], n = mg[3], stride = mg[4];
+  const int q_start = seg_q_start[seg], q_len = seg_q_len[seg];
+  const int rho = rho0 + row;
+  if (rho >= q_len * G) return;
+  auto slot_row = [&](int i) { return ((size_t)(first + i * stride) * K + g) * 16 + row; };
+  float m_all = -INFINITY;
+  for (int i = 0; i < n; ++i) m_all = fmaxf(m_all, part_ml[slot_row(i) * 2]);
+  float acc[NC][2];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) acc[c][0] = acc[c][1] = 0.f;
+  float l_all = 0.f;
+  for (int i = 0; i < n; ++i) {
+    const size_t base = slot_row(i);
+    const float2 ml = *(const float2*)(part_ml + base * 2);
+    const float w = ml.x == -INFINITY ? 0.f : exp2f(ml.x - m_all);
+    l_all += w * ml.y;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int d = c * 128 + lane * 2;
+      if (d >= D) continue;
+      const float2 v = *(const float2*)(part_o + base * D + d);
+      acc[c][0] += w * v.x;
+      acc[c][1] += w * v.y;
+    }
+  }
+  const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
+  const int qi = rho / G, head = g * G + rho % G;
+  bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int d = c * 128 + lane * 2;
+    if (d >= D) continue;
+    *(uint32_t*)(op + d) = pack2(acc[c][0] * inv, acc[c][1] * inv);
+  }
+}
+
 extern "C" int hal_attention_mfma_head_dim() { return D; }
 
 // How many 16-row tiles a wave takes in the kernel for long segments.
@@ -635,7 +688,7 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
                                   const int* block_table, int bt_stride, const void* k_pages,
                                   const void* v_pages, float* part_o, float* part_ml, int H, int K,
                                   int head_dim, int page_size, int tiled, float scale,
-                                  int window, hipStream_t stream) {
+                                  int window, int merge_parts, hipStream_t stream) {
   HAL_REQUIRE(head_dim == D, "hal_attention_mfma: built for head size %d, called with %d", D,
               head_dim);
   HAL_REQUIRE(H > 0 && K > 0 && H % K == 0, "hal_attention_mfma: %d heads, %d kv heads", H, K);
@@ -674,9 +727,14 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, true, KB_BIG, big_items, max_big, counts + 1)
 #undef LAUNCH_ATTENTION
   if (max_merges > 0) {
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K, 16), dim3(256), 0, stream,
-                       (bf16_t*)out, out_row_stride, merges, counts + 2, seg_q_start, seg_q_len,
-                       part_o, part_ml, H, K);
+    if (merge_parts > 0 && merge_parts <= MERGE_FEW_PARTS)
+      hipLaunchKernelGGL(attention_merge_few_kernel, dim3(max_merges, K, 4), dim3(256), 0, stream,
+                         (bf16_t*)out, out_row_stride, merges, counts + 2, seg_q_start,
+                         seg_q_len, part_o, part_ml, H, K);
+    else
+      hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K, 16), dim3(256), 0, stream,
+                         (bf16_t*)out, out_row_stride, merges, counts + 2, seg_q_start,
+                         seg_q_len, part_o, part_ml, H, K);
     HAL_LAUNCH_CHECK();
   }
   return 0;

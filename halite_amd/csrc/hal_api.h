@@ -55,6 +55,8 @@ int hal_sample_greedy(const float* logits, int ld, int n_rows, int V, float* par
 
 int hal_attention_mfma_head_dim();
 int hal_attention_mfma_rows_per_big_item();
+// merge_parts: the most partial results that any merge item joins, or 0 if not known (the
+// kernel for many partials is taken then).
 int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_stride,
                        const int* items, int max_items, const int* big_items, int max_big,
                        const int* merges, int max_merges, const int* counts,
@@ -62,6 +64,6 @@ int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_s
                        const int* block_table, int bt_stride, const void* k_pages,
                        const void* v_pages, float* part_o, float* part_ml, int H, int K,
                        int head_dim, int page_size, int tiled, float scale, int window,
-                       hipStream_t stream);
+                       int merge_parts, hipStream_t stream);
 
 }  // extern "C"

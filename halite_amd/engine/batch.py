@@ -201,6 +201,7 @@ class StepContext:
             cap = self.static.max_items if self.static is not None else None
             if cap is not None:  # decode only: no long segments
                 plan.cap_items, plan.cap_merges, plan.cap_partials = cap, min(cap, self.n_segs), cap
+                plan.max_parts = 0  # the launches are recorded once for all later plans
             self._packer.add(plan.name + "_items", plan.items, None if cap is None else cap * 8)
             self._packer.add(plan.name + "_big", plan.big_items)
             self._packer.add(plan.name + "_merges", plan.merges, None if cap is None else plan.cap_merges * 8)

@@ -298,7 +298,6 @@ class ModelRunner:
             graph = torch.cuda.CUDAGraph()
             # No garbage collection while the stream records: a graph of an engine that
             # is no longer used would be destroyed in the middle of it, which HIP refuses.
-            gc.collect()
             collecting = gc.isenabled()
             gc.disable()
             try:

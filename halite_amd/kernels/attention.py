@@ -46,8 +46,13 @@ class AttentionPlan:
     cap_big: int = 0
     cap_merges: int = 0
     cap_partials: int = 0
+    # the most partial results that a merge item joins; 0: not known (a static layout,
+    # whose kernel launches are fixed while the plans change)
+    max_parts: int = 0
 
     def __post_init__(self):
+        if len(self.merges) and self.max_parts == 0:
+            self.max_parts = int(self.merges[:, 3].max())
         self.cap_items = max(self.cap_items, len(self.items))
         self.cap_big = max(self.cap_big, len(self.big_items))
         self.cap_merges = max(self.cap_merges, len(self.merges))
@@ -244,7 +249,7 @@ def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, wi
         P(ctx.seg_q_start), P(ctx.seg_q_len), P(ctx.seg_kv_len),
         P(group.block_table), group.block_table.shape[1], P(kv.k), P(kv.v), P(part_o), P(part_ml),
         n_heads, n_kv, head_dim, page_size, 1 if getattr(kv, "tiled", False) else 0,
-        ctypes.c_float(scale), window, ops._stream(),
+        ctypes.c_float(scale), window, plan.max_parts, ops._stream(),
     )
     ops._check(lib, rc)
     return out
