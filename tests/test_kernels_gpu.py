@@ -292,6 +292,13 @@ def test_attention_mfma_split_keys(gpu):
     attention_case(gpu, "bfloat16", 8, 2, 128, 64, segs, 0, seed=44, use="mfma", tiled=True)
     attention_case(gpu, "bfloat16", 8, 2, 128, 64, [(5000, 40), (2500, 100)], 0, seed=45, use="mfma", tiled=True)
     attention_case(gpu, "bfloat16", 4, 1, 64, 32, [(3000, 50), (0, 600)], 700, seed=46, use="mfma", tiled=True)
+    # few partial results per row: the merge kernel of one wave per row
+    for segs, heads in (([(512, 256)], (8, 2)), ([(300, 200), (0, 64)], (4, 1))):
+        q_len, kv_len = np.array([n for _, n in segs]), np.array([b + n for b, n in segs])
+        plan = attn_kernels.plan_items(q_len, kv_len, heads[0] // heads[1], heads[1], 0, attn_kernels.rows_per_big_item(128))
+        assert 1 < plan.max_parts <= 8 and plan.n_merges > 0
+        attention_case(gpu, "bfloat16", heads[0], heads[1], 128, 64, segs, 0, seed=47, use="mfma")
+        attention_case(gpu, "bfloat16", heads[0], heads[1], 128, 64, segs, 0, seed=48, use="mfma", tiled=True)
 
 
 @pytest.mark.parametrize("tiled", [False, True])
