@@ -134,6 +134,8 @@ def engine_workload(args) -> int:
     # an untimed pass over a few short requests: libraries, graphs of the small batches
     engine.infer_batch([(torch.randint(0, cfg.vocab_size, (64,), generator=gen).tolist(),
                          SamplingParams(max_new_tokens=4, temperature=0.0, ignore_eos=True)) for _ in range(2)])
+    engine.initialize(capture_graphs=not args.no_graph)  # as a server does before it takes requests
+    graphs_before = len(runner._graphs)
     before = engine.stats.steps, engine.stats.retractions, len(engine.stats.tokens_per_step)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -182,6 +184,7 @@ def engine_workload(args) -> int:
         "mean_tokens_per_step": round(sum(per_step) / max(1, len(per_step)), 1),
         "retractions": engine.stats.retractions - before[1],
         "steps_launched_ahead": engine.steps_launched_ahead,
+        "graphs_recorded_before": graphs_before,
         "weights_gb": round(runner.model.param_bytes() / 1e9, 2),
     }
     print(json.dumps(record), flush=True)

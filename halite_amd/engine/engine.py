@@ -266,7 +266,12 @@ class InferenceEngine:
     def stats(self):
         return self.scheduler.stats
 
-    def initialize(self):
+    def initialize(self, capture_graphs: bool = False):
+        """``capture_graphs``: record the decode graphs of every batch size now (the
+        reference does so in its ``initialize``, engine.py:33-41) instead of at the first
+        step of each size."""
+        if capture_graphs:
+            self.model_runner.capture_graphs()
         self.initialized = True
 
     def load_state_dict(self, state_dict: dict, assign: bool = True):

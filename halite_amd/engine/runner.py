@@ -168,6 +168,32 @@ class ModelRunner:
     def free(self, slot: int) -> None:
         self.cache.free(slot)
 
+    def capture_graphs(self, batch_sizes=None) -> list[int]:
+        """Records the decode graphs of the given batch sizes now instead of at their
+        first use (the reference records its graphs when the engine is set up,
+        src/halite/transformers/infer/engine/model_runner.py:159-239).  Needs an idle
+        cache: every size is run once with one-token requests that are freed again.
+        Returns the sizes that have a graph afterwards."""
+        if not self.server_config.use_cudagraph:
+            return []
+        if not self.cache.idle():
+            raise RuntimeError("graphs are recorded ahead of time only while no request is live")
+        most = min(self.server_config.cudagraph_max_batch_size, self.server_config.max_seqs_per_forward)
+        for b in sorted(set(batch_sizes) if batch_sizes is not None else range(1, most + 1)):
+            entry = self._graphs.get(b)
+            if b < 1 or b > most or (entry is not None and entry["graph"] is not None):
+                continue
+            slots = [self.admit() for _ in range(b)]
+            try:
+                self.step([Segment(slot, 0, [0], [0]) for slot in slots])
+            except NoSpace:
+                break  # the pool is smaller than this many pages: larger sizes cannot occur
+            finally:
+                for slot in slots:
+                    self.free(slot)
+        self._ahead = None
+        return sorted(b for b, e in self._graphs.items() if e["graph"] is not None)
+
     # -- the step ---------------------------------------------------------------------
     def check_segments(self, segments: list[Segment], n_ids: int | None = None) -> None:
         n_ids = self.vocab_size if n_ids is None else n_ids

@@ -278,3 +278,27 @@ def test_the_engine_serves_on_after_a_refused_or_failed_batch(models):
     engine.model_runner.step = step
     assert engine.model_runner.cache.idle()
     assert engine.infer_batch([good])[0].output_ids == want
+
+
+def test_graphs_recorded_ahead_of_time(models):
+    """``initialize(capture_graphs=True)`` records the decode graph of every batch size while
+    the engine is idle; generation then replays them and gives the tokens of an engine
+    that records at first use."""
+    folder, pc, pw = models[("B", "bfloat16")]
+    server = ServerConfig(kv_cache_num_tokens=2048, max_seqs_per_forward=6, use_cudagraph=True)
+    prompts = [tiny.random_tokens(tiny.TINY_B, n, 500 + n) for n in (3, 40, 17, 9)]
+    batch = [(p, {"max_new_tokens": 10 + 2 * i, "temperature": 0.0}) for i, p in enumerate(prompts)]
+    lazy = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="bfloat16"))
+    want = [r.output_ids for r in lazy.infer_batch(batch)]
+    eager = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="bfloat16"))
+    eager.initialize(capture_graphs=True)
+    runner = eager.model_runner
+    assert sorted(runner._graphs) == [1, 2, 3, 4, 5, 6] and runner.cache.idle()
+    replays = runner.graph_replays
+    assert [r.output_ids for r in eager.infer_batch(batch)] == want
+    assert runner.graph_replays > replays and sorted(runner._graphs) == [1, 2, 3, 4, 5, 6]
+    assert runner.capture_graphs([2, 3]) == [1, 2, 3, 4, 5, 6]  # nothing to do
+    # without graphs there is nothing to record
+    plain = InferenceEngine.from_pretrained(folder, ServerConfig(kv_cache_num_tokens=512), ModelConfig(dtype="bfloat16"))
+    plain.initialize(capture_graphs=True)
+    assert plain.model_runner._graphs == {}
