@@ -84,7 +84,7 @@ class InferenceEngine:
             stop.update(getattr(tokenizer, "additional_stop_token_ids", None) or ())
         self.scheduler = Scheduler(
             model_runner.cache, self.server_config, self._run_step, model_runner.context_len, stop,
-            vocab_size=model_runner.vocab_size,
+            vocab_size=model_runner.vocab_size, tokenizer=tokenizer,
         )
         self.initialized = True
 

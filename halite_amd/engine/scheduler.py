@@ -37,7 +37,7 @@ CLIP_MAX_NEW_TOKENS = 4096  # schedule_policy.py:38, 82
 @dataclass
 class FinishReason:
     reason: str  # "length" | "stop"
-    matched: int | None = None
+    matched: int | str | None = None  # the stop token or the stop string
     length: int | None = None
 
 
@@ -57,6 +57,7 @@ class Request:
         self.is_retracted = False
         self.n_retractions = 0
         self.seed = 0
+        self._stop_window: int | None = None  # tokens of the longest stop string
 
     @property
     def all_ids(self) -> list[int]:
@@ -87,7 +88,9 @@ class Request:
     def finished(self) -> bool:
         return self.finished_reason is not None
 
-    def check_finished(self, stop_token_ids=()):
+    def check_finished(self, stop_token_ids=(), tokenizer=None):
+        """batch.py:180-215 of the reference: by length, by a stop token, by a stop string
+        in the text of the last tokens (as many as the longest stop string has, and one)."""
         if self.finished():
             return
         p = self.sampling_params
@@ -97,6 +100,21 @@ class Request:
         last = self.output_ids[-1]
         if not p.ignore_eos and (last in p.stop_token_ids or last in stop_token_ids):
             self.finished_reason = FinishReason("stop", matched=last)
+        if p.stop and tokenizer is not None:
+            if self._stop_window is None:
+                self._stop_window = max(len(_encode_plain(tokenizer, s)) for s in p.stop)
+            tail = tokenizer.decode(self.output_ids[-(self._stop_window + 1):])
+            for s in p.stop:
+                if s in tail:
+                    self.finished_reason = FinishReason("stop", matched=s)
+                    return
+
+
+def _encode_plain(tokenizer, text: str) -> list:
+    try:
+        return list(tokenizer.encode(text, add_special_tokens=False))
+    except TypeError:
+        return list(tokenizer.encode(text))
 
 
 @dataclass
@@ -134,7 +152,9 @@ class Scheduler:
         context_len: int,
         stop_token_ids=(),
         vocab_size: int | None = None,
+        tokenizer=None,
     ):
+        self.tokenizer = tokenizer  # only for stop strings
         self.cache = cache
         self.conf = server_config
         self.run_step = run_step
@@ -340,7 +360,7 @@ class Scheduler:
             else:
                 r.output_ids.append(int(tok))
                 r.output_logprobs.append(float(lp))
-                r.check_finished(self.stop_token_ids)
+                r.check_finished(self.stop_token_ids, self.tokenizer)
             if r.finished():
                 self.cache.free(r.slot)
                 r.slot = None

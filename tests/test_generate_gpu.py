@@ -302,3 +302,38 @@ def test_graphs_recorded_ahead_of_time(models):
     plain = InferenceEngine.from_pretrained(folder, ServerConfig(kv_cache_num_tokens=512), ModelConfig(dtype="bfloat16"))
     plain.initialize(capture_graphs=True)
     assert plain.model_runner._graphs == {}
+
+
+class LetterTokenizer:
+    """Token t is the letter chr(97 + t % 26); no end-of-text token."""
+
+    eos_id = None
+    additional_stop_token_ids = None
+
+    def encode(self, text, add_special_tokens=True):
+        return [ord(c) - 97 for c in text]
+
+    def decode(self, ids):
+        return "".join(chr(97 + t % 26) for t in ids)
+
+
+@pytest.mark.parametrize("ahead", [0, 1])
+def test_stop_strings_through_the_engine(models, ahead):
+    """Stop strings need a tokenizer; with one, a request ends with the token that
+    completes the string, also when the step after it was launched already."""
+    folder, pc, pw = models[("B", "float32")]
+    tok = LetterTokenizer()
+    server = ServerConfig(kv_cache_num_tokens=2048, use_cudagraph=True, scheduling_steps_ahead=ahead)
+    engine = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="float32"), tokenizer=tok)
+    prompts = [tiny.random_tokens(tiny.TINY_B, n, 600 + n) for n in (5, 12, 30)]
+    free = engine.infer_batch([(p, {"max_new_tokens": 30, "temperature": 0.0}) for p in prompts])
+    texts = [tok.decode(r.output_ids[0]) for r in free]
+    stops = [t[10:13] for t in texts]
+    got = engine.infer_batch([(p, {"max_new_tokens": 30, "temperature": 0.0, "stop": s}) for p, s in zip(prompts, stops)])
+    for r, full, text, s in zip(got, free, texts, stops):
+        cut = text.index(s) + len(s)
+        assert r.output_ids[0] == full.output_ids[0][:cut] and r.finish_reason == ["stop"]
+    assert engine.model_runner.cache.idle()
+    with pytest.raises(ValueError, match="tokenizer"):
+        InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="float32")).infer_batch(
+            [(prompts[0], {"max_new_tokens": 3, "stop": "ab"})])

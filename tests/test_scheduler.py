@@ -231,3 +231,38 @@ def test_requests_are_checked_before_they_wait_and_a_batch_can_be_dropped():
     while (plan := sched.schedule()) is not None:
         sched.process_results(plan, *model(plan))
     assert cache.idle()
+
+
+class LetterTokenizer:
+    """Token t is the letter chr(97 + t % 26)."""
+
+    eos_id = None
+    additional_stop_token_ids = None
+
+    def encode(self, text, add_special_tokens=True):
+        return [ord(c) - 97 for c in text]
+
+    def decode(self, ids):
+        return "".join(chr(97 + t % 26) for t in ids)
+
+
+def test_stop_strings():
+    """A request ends when the text of its last tokens holds one of its stop strings
+    (src/halite/transformers/infer/engine/batch.py:206-215); the tokens that spell it
+    are part of the output."""
+    sched, model, cache = make()
+    sched.tokenizer = tok = LetterTokenizer()
+    p = [3, 1, 4, 1, 5]
+    full = expected(p, 40)
+    text = tok.decode(full)
+    stop = text[6:9]  # three letters that the request will write
+    first = text.index(stop) + len(stop)
+    sched.add_request(Request(0, p, SamplingParams(max_new_tokens=40, stop=stop)))
+    sched.add_request(Request(1, p, SamplingParams(max_new_tokens=40, stop=["zzzzzz", stop])))
+    sched.add_request(Request(2, p, SamplingParams(max_new_tokens=40, stop="qqqqqqqq")))
+    done = {r.id: r for r in sched.run_to_completion()}
+    assert done[0].output_ids == full[:first] and done[0].finished_reason.reason == "stop"
+    assert done[0].finished_reason.matched == stop
+    assert done[1].output_ids == full[:first]
+    assert done[2].output_ids == full and done[2].finished_reason.reason == "length"
+    assert cache.idle()
