@@ -161,6 +161,34 @@ def test_trace_run_program(folders, dtype, tmp_path):
     replay.compare(rows, ref, TOL[dtype])
 
 
+def test_trace_run_step_by_step(folders, tmp_path):
+    """A step is sent only after the line ``done <step>`` of the one before has come back;
+    by then the step's file is complete."""
+    folder, requests, ref = folders[("A", "float32")]
+    trace = replay.portions({k: requests[k] for k in list(requests)[:3]})
+    out = tmp_path / "out"
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+           "--out", str(out), "--max-tokens", str(replay.peak_tokens(trace))]
+    proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)
+    logits = {}
+    try:
+        for s in trace:
+            proc.stdin.write(json.dumps(s) + "\n")
+            proc.stdin.flush()
+            assert proc.stdout.readline().strip() == f"done {s['step']}"
+            n_want = sum(len(e["want"]) for e in s["entries"])
+            if n_want:
+                data = np.fromfile(out / f"{s['step']}.f32", dtype="<f4")
+                assert data.size == n_want * 256
+                logits[s["step"]] = torch.from_numpy(data.reshape(n_want, 256))
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+    replay.compare(replay.collect(trace, logits, 256), ref, TOL["float32"])
+
+
 def test_refusals(folders):
     from halite_amd.cache import NoSpace
     from halite_amd.engine.batch import Segment
