@@ -73,6 +73,26 @@ class LlamaConfig(BaseModel):
     bos_token_id: int | list[int] | None = None
     eos_token_id: int | list[int] | None = None
 
+    @model_validator(mode="before")
+    @classmethod
+    def _accept_other_spellings(cls, data):
+        """Folders written by newer tools carry ``rope_parameters`` (the base and the
+        scaling arguments in one dict) instead of ``rope_theta`` and ``rope_scaling``,
+        and may name the unscaled frequencies ``"default"``."""
+        if not isinstance(data, dict):
+            return data
+        data = dict(data)
+        merged = data.get("rope_parameters")
+        if isinstance(merged, dict):
+            if "rope_theta" not in data and "rope_theta" in merged:
+                data["rope_theta"] = merged["rope_theta"]
+            if "rope_scaling" not in data:
+                data["rope_scaling"] = {k: v for k, v in merged.items() if k != "rope_theta"}
+        scaling = data.get("rope_scaling")
+        if isinstance(scaling, dict) and scaling.get("rope_type", scaling.get("type")) == "default":
+            data["rope_scaling"] = None
+        return data
+
     @model_validator(mode="after")
     def _check(self):
         if self.num_key_value_heads is None:

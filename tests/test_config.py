@@ -35,6 +35,29 @@ def test_defaults_that_have_a_meaning():
     assert cfg.num_key_value_heads == 4 and cfg.head_dim == 16 and cfg.rope_scaling is None
 
 
+def test_other_spellings_of_the_rotation_keys():
+    # base and scaling arguments in one dict, as newer writers of such folders do
+    raw = dict(tiny.TINY_B)
+    merged = dict(raw.pop("rope_scaling"), rope_theta=raw.pop("rope_theta"))
+    raw["rope_parameters"] = merged
+    _, cfg = parse_config(raw)
+    _, ref = parse_config(tiny.TINY_B)
+    assert cfg.rope_theta == ref.rope_theta and cfg.rope_scaling == ref.rope_scaling
+    # "default" names the unscaled frequencies
+    raw = dict(tiny.TINY_A, rope_scaling={"rope_type": "default"})
+    assert parse_config(raw)[1].rope_scaling is None
+    raw = dict(tiny.TINY_A)
+    raw["rope_parameters"] = {"rope_type": "default", "rope_theta": raw.pop("rope_theta")}
+    cfg = parse_config(raw)[1]
+    assert cfg.rope_scaling is None and cfg.rope_theta == tiny.TINY_A["rope_theta"]
+    # and still no default for the base
+    raw = dict(tiny.TINY_A)
+    del raw["rope_theta"]
+    raw["rope_parameters"] = {"rope_type": "default"}
+    with pytest.raises(ConfigError, match="rope_theta"):
+        parse_config(raw)
+
+
 @pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
                                  "intermediate_size", "rms_norm_eps", "rope_theta", "max_position_embeddings"])
 def test_no_size_has_a_default_in_code(key):
