@@ -65,6 +65,9 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 // item: {segment, first row of tile 0, first key, end key, first partial slot or -1,
 //        first row of tile 1, of tile 2, of tile 3 (or -1)}
+// An item of the one-tile kernel carries its segment's first token, number of tokens and
+// number of keys in the last three places instead, so that the wave need not wait for the
+// item before it can ask for them.
 // A wave works on up to RT tiles of 16 rows of one segment; the keys and values it
 // loads serve all of them.  The tiles need not be neighbours (the host lists neighbours:
 // they share nearly all of their keys).  A tile skips the steps whose keys lie wholly
@@ -84,7 +87,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                       const int* __restrict__ block_table, int bt_stride,
                       const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                       float* __restrict__ part_o, float* __restrict__ part_ml, int H, int K,
-                      int page_size, int page_shift, float scale_log2e, int window) {
+                      int page_size, int page_shift, float scale_log2e, int window,
+                      int max_items) {
   const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
   // Workgroups go to the eight XCDs in turn (linear id modulo 8) and each XCD has an L2 of
   // its own: the ids are renumbered so that an XCD gets a contiguous run of (kv head, item
@@ -102,8 +106,17 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   // everything that describes the item is the same for the whole wave: kept in scalar
   // registers, so that loop control, block-level masks and page lookups cost no vector work
   auto uniform = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
-  const int n_items = *n_items_ptr;
   const int item = uniform(bx * WAVES + wave);
+  // the item is asked for together with the live count (an index past the list's end is
+  // clamped for the address only): one trip to memory instead of two
+  constexpr bool INLINE_SEG = !SHARED && RT == 1;
+  int pre[ITEM_INTS];
+  if constexpr (INLINE_SEG) {
+    const int* ip = items + (size_t)(item < max_items ? item : max_items - 1) * ITEM_INTS;
+#pragma unroll
+    for (int i = 0; i < ITEM_INTS; ++i) pre[i] = ip[i];
+  }
+  const int n_items = *n_items_ptr;
   // SHARED: the four waves of a workgroup have items of one segment (the host lists them
   // so) and walk the union of their key ranges together; the keys and values of a block
   // are loaded once, by all four, into LDS.  A wave without an item of its own (the list
@@ -111,10 +124,14 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   if (SHARED ? bx * WAVES >= n_items : item >= n_items) return;
   const bool have_item = item < n_items;
   const int* it = items + (size_t)(have_item ? item : bx * WAVES) * ITEM_INTS;
-  const int seg = uniform(it[0]);
-  const int rho0 = have_item ? uniform(it[1]) : -1;
-  const int kv_begin = have_item ? uniform(it[2]) : 0, kv_end = have_item ? uniform(it[3]) : 0;
-  const int partial = have_item ? uniform(it[4]) : -1;
+  auto iv = [&](int i) {
+    if constexpr (INLINE_SEG) return pre[i];
+    else return it[i];
+  };
+  const int seg = uniform(iv(0));
+  const int rho0 = have_item ? uniform(iv(1)) : -1;
+  const int kv_begin = have_item ? uniform(iv(2)) : 0, kv_end = have_item ? uniform(iv(3)) : 0;
+  const int partial = have_item ? uniform(iv(4)) : -1;
   int walk_begin = kv_begin, walk_end = kv_end;  // the keys this wave walks through
   if constexpr (SHARED) {
     walk_begin = 0x7fffffff, walk_end = 0;
@@ -130,8 +147,13 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     if (walk_begin >= walk_end) return;  // the same for all four waves
   }
   const int G = H / K;
-  const int q_start = uniform(seg_q_start[seg]), q_len = uniform(seg_q_len[seg]),
-            kv_len = uniform(seg_kv_len[seg]);
+  int q_start, q_len, kv_len;
+  if constexpr (INLINE_SEG) {
+    q_start = uniform(pre[5]), q_len = uniform(pre[6]), kv_len = uniform(pre[7]);
+  } else {
+    q_start = uniform(seg_q_start[seg]), q_len = uniform(seg_q_len[seg]);
+    kv_len = uniform(seg_kv_len[seg]);
+  }
   const int pos0 = kv_len - q_len;  // position of the segment's first token
   const int* bt = block_table + (size_t)seg * bt_stride;
 
@@ -144,7 +166,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   float m[RT], l[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int tile0 = rt == 0 ? rho0 : (have_item ? uniform(it[4 + rt]) : -1);
+    const int tile0 = rt == 0 ? rho0 : (have_item ? uniform(iv(4 + rt)) : -1);
     const int rho = tile0 + col;
     row_ok[rt] = tile0 >= 0 && rho < q_len * G;
     qi[rt] = row_ok[rt] ? rho / G : 0;
@@ -172,7 +194,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   int p_first[RT], p_last[RT], lo_first[RT], lo_last[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int r_first = rt == 0 ? rho0 : (have_item ? uniform(it[4 + rt]) : -1);
+    const int r_first = rt == 0 ? rho0 : (have_item ? uniform(iv(4 + rt)) : -1);
     int r_last = r_first + 15;
     if (r_last > q_len * G - 1) r_last = q_len * G - 1;
     if (r_last < r_first) r_last = r_first;
@@ -517,14 +539,13 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 }
 
 // merge item: {segment, first row (of 16), first partial slot, number of partials,
-// slots from one partial to the next, 0, 0, 0}
+// slots from one partial to the next, the segment's first token, its number of tokens, 0}
 // One block per (merge item, kv head, row of the tile).  The four waves take every
 // fourth partial each, four loads in flight at a time, a lane two dimensions; their sums
 // are added in wave order through LDS (deterministic).
 __global__ void __launch_bounds__(256)
 attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
                        const int* __restrict__ merges, const int* __restrict__ n_merges_ptr,
-                       const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                        const float* __restrict__ part_o, const float* __restrict__ part_ml, int H,
                        int K) {
   constexpr int NC = (D + 127) / 128;  // a lane's pairs of dimensions
@@ -533,16 +554,36 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
   __shared__ float red_l[MW];
   __shared__ float scratch[16];
   const int mi = blockIdx.x;
-  if (mi >= *n_merges_ptr) return;
   const int g = blockIdx.y, row = blockIdx.z;
   const int G = H / K;
+  // the item is asked for together with the live count (blockIdx.x is below the list's
+  // capacity), and it carries what the kernel needs of its segment
   const int* mg = merges + (size_t)mi * ITEM_INTS;
-  const int seg = mg[0], rho0 = mg[1], first = mg[2], n = mg[3], stride = mg[4];
-  const int q_start = seg_q_start[seg], q_len = seg_q_len[seg];
+  const int rho0 = mg[1], first = mg[2], n = mg[3], stride = mg[4], q_start = mg[5], q_len = mg[6];
+  if (mi >= *n_merges_ptr) return;
   const int rho = rho0 + row;
   if (rho >= q_len * G) return;  // the whole block
   const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
   auto slot_row = [&](int i) { return ((size_t)(first + i * stride) * K + g) * 16 + row; };
+
+  // A wave's partials go four at a time; the loads of the first four go out before the
+  // row's largest maximum is known, which needs a pass over all maxima and a barrier.
+  float2 ml[4];
+  float2 v[4][NC];
+  auto ask = [&](int i0) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * MW;
+      const size_t base = slot_row(i < n ? i : i0);
+      ml[u] = *(const float2*)(part_ml + base * 2);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int d = c * 128 + lane * 2;
+        v[u][c] = d < D ? *(const float2*)(part_o + base * D + d) : float2{0.f, 0.f};
+      }
+    }
+  };
+  if (wave < n) ask(wave);
 
   // the largest running maximum of the row
   float m_all = -INFINITY;
@@ -554,29 +595,16 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
   for (int c = 0; c < NC; ++c) acc[c][0] = acc[c][1] = 0.f;
   float l_all = 0.f;
   for (int i0 = wave; i0 < n; i0 += MW * 4) {
-    float w[4], li[4];
-    float2 v[4][NC];
+    if (i0 != wave) ask(i0);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int i = i0 + u * MW;
-      const bool ok = i < n;
-      const size_t base = slot_row(ok ? i : i0);
-      const float2 ml = *(const float2*)(part_ml + base * 2);
-      w[u] = (!ok || ml.x == -INFINITY) ? 0.f : exp2f(ml.x - m_all);
-      li[u] = ml.y;
+      const bool ok = i0 + u * MW < n;
+      const float w = (!ok || ml[u].x == -INFINITY) ? 0.f : exp2f(ml[u].x - m_all);
+      l_all += w * ml[u].y;
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
-        const int d = c * 128 + lane * 2;
-        v[u][c] = d < D ? *(const float2*)(part_o + base * D + d) : float2{0.f, 0.f};
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      l_all += w[u] * li[u];
-#pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        acc[c][0] += w[u] * v[u][c].x;
-        acc[c][1] += w[u] * v[u][c].y;
+        acc[c][0] += w * v[u][c].x;
+        acc[c][1] += w * v[u][c].y;
       }
     }
   }
@@ -614,18 +642,16 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
 __global__ void __launch_bounds__(256)
 attention_merge_few_kernel(bf16_t* __restrict__ out, int out_row_stride,
                            const int* __restrict__ merges, const int* __restrict__ n_merges_ptr,
-                           const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                            const float* __restrict__ part_o, const float* __restrict__ part_ml,
                            int H, int K) {
   constexpr int NC = (D + 127) / 128;
   const int mi = blockIdx.x;
-  if (mi >= *n_merges_ptr) return;
   const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
   const int g = blockIdx.y, row = blockIdx.z * 4 + wave;
   const int G = H / K;
   const int* mg = merges + (size_t)mi * ITEM_INTS;
-  const int seg = mg[0], rho0 = mg[1], first = mg[2], n = mg[3], stride = mg[4];
-  const int q_start = seg_q_start[seg], q_len = seg_q_len[seg];
+  const int rho0 = mg[1], first = mg[2], n = mg[3], stride = mg[4], q_start = mg[5], q_len = mg[6];
+  if (mi >= *n_merges_ptr) return;
   const int rho = rho0 + row;
   if (rho >= q_len * G) return;
   auto slot_row = [&](int i) { return ((size_t)(first + i * stride) * K + g) * 16 + row; };
@@ -720,7 +746,7 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
                        q_row_stride, (bf16_t*)out, out_row_stride, LIST, COUNT, seg_q_start,      \
                        seg_q_len, seg_kv_len, block_table, bt_stride, (const bf16_t*)k_pages,     \
                        (const bf16_t*)v_pages, part_o, part_ml, H, K, page_size, page_shift,      \
-                       scale_log2e, window);                                                      \
+                       scale_log2e, window, MAX);                                                 \
     HAL_LAUNCH_CHECK();                                                                           \
   }
   if (max_items > 0) LAUNCH_ATTENTION(1, false, 32, items, max_items, counts)
@@ -729,12 +755,10 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   if (max_merges > 0) {
     if (merge_parts > 0 && merge_parts <= MERGE_FEW_PARTS)
       hipLaunchKernelGGL(attention_merge_few_kernel, dim3(max_merges, K, 4), dim3(256), 0, stream,
-                         (bf16_t*)out, out_row_stride, merges, counts + 2, seg_q_start,
-                         seg_q_len, part_o, part_ml, H, K);
+                         (bf16_t*)out, out_row_stride, merges, counts + 2, part_o, part_ml, H, K);
     else
       hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K, 16), dim3(256), 0, stream,
-                         (bf16_t*)out, out_row_stride, merges, counts + 2, seg_q_start,
-                         seg_q_len, part_o, part_ml, H, K);
+                         (bf16_t*)out, out_row_stride, merges, counts + 2, part_o, part_ml, H, K);
     HAL_LAUNCH_CHECK();
   }
   return 0;

@@ -145,12 +145,16 @@ __global__ void rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ 
   T* o = out + (size_t)r * d;
   const int nv = d / 4;
 
-  float x[RMS_MAXV][4];
+  // the weight does not depend on the row: asked for with the row, not after the sum
+  float x[RMS_MAXV][4], wv[RMS_MAXV][4];
   float ss = 0.f;
 #pragma unroll
   for (int u = 0; u < RMS_MAXV; ++u) {
     const int v = threadIdx.x + u * blockDim.x;
-    if (v < nv) load4(hr + v * 4, x[u]);
+    if (v < nv) {
+      load4(hr + v * 4, x[u]);
+      load4_any(w, w_dtype, (size_t)v * 4, wv[u]);
+    }
   }
   if (dr) {
 #pragma unroll
@@ -179,10 +183,9 @@ __global__ void rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ 
   for (int u = 0; u < RMS_MAXV; ++u) {
     const int v = threadIdx.x + u * blockDim.x;
     if (v < nv) {
-      float wv[4], y[4];
-      load4_any(w, w_dtype, (size_t)v * 4, wv);
+      float y[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) y[i] = wv[i] * to_f32(from_f32<T>(x[u][i] * rstd));
+      for (int i = 0; i < 4; ++i) y[i] = wv[u][i] * to_f32(from_f32<T>(x[u][i] * rstd));
       store4(o + v * 4, y);
     }
   }
@@ -407,14 +410,33 @@ __global__ void rope_append_vec_kernel(T* __restrict__ qkv, int row_stride,
                                        int n_pages, bool tiled) {
   const int t = blockIdx.x;
   const int pos = positions[t];
+  const int seg = K > 0 ? token_seg[t] : 0;
   T* row = qkv + (size_t)t * row_stride;
   const int half = rot / 2;
+  // A step of few tokens (decode) is a chain of trips to memory, so everything that does not
+  // depend on the position is asked for before the position is looked at: this token's
+  // values here, and the neighbours that decide further down who writes the values.
+  const int d8 = D / 8;
+  const bool early_values = K > 0 && gridDim.x <= 64 && K * d8 <= (int)blockDim.x;
+  uint4 vpre[sizeof(T) / 2];
+  if (early_values && (int)threadIdx.x < K * d8) {
+    const uint4* vr = (const uint4*)(row + (size_t)(H + K) * D + (size_t)threadIdx.x * 8);
+#pragma unroll
+    for (int i = 0; i < (int)(sizeof(T) / 2); ++i) vpre[i] = vr[i];
+  }
   if (rot > 0 && (pos < 0 || pos >= table_len)) return;
   long long page = -1;
   int off = 0;
+  bool whole = false;
   if (K > 0) {
-    page = block_table[(size_t)token_seg[t] * bt_stride + pos / page_size];
+    page = block_table[(size_t)seg * bt_stride + pos / page_size];
     off = pos % page_size;
+    if (page_size % 8 == 0) {
+      const int t0 = t - off % 8;  // where the first token of this token's group of eight would be
+      if (t0 >= 0 && t0 + 7 < (int)gridDim.x)
+        whole = token_seg[t0] == seg && token_seg[t0 + 7] == seg &&
+                positions[t0] == pos - off % 8 && positions[t0 + 7] == pos - off % 8 + 7;
+    }
     if (page < 0 || page >= n_pages) page = -1;
   }
   const float* cp = cos_t + (size_t)pos * half;
@@ -492,40 +514,37 @@ __global__ void rope_append_vec_kernel(T* __restrict__ qkv, int row_stride,
   // layouts).  Where this token and the seven after it are one request's positions
   // 8j .. 8j+7, the block of the first writes the values of all eight, eight at a time;
   // the other seven leave theirs to it.
-  if (page_size % 8 == 0) {
-    const int t0 = t - off % 8;  // where the group's first token would be
-    const int seg = token_seg[t];
-    const bool whole = t0 >= 0 && t0 + 7 < (int)gridDim.x && token_seg[t0] == seg &&
-                       token_seg[t0 + 7] == seg && positions[t0] == pos - off % 8 &&
-                       positions[t0 + 7] == pos - off % 8 + 7;
-    if (whole) {
-      if (t != t0) return;
-      for (int idx = threadIdx.x; idx < K * D; idx += blockDim.x) {
-        const int g = idx / D, d = idx % D;
-        __attribute__((aligned(16))) T vals[8];
+  if (whole) {
+    if (off % 8 != 0) return;
+    for (int idx = threadIdx.x; idx < K * D; idx += blockDim.x) {
+      const int g = idx / D, d = idx % D;
+      __attribute__((aligned(16))) T vals[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          vals[e] = qkv[(size_t)(t + e) * row_stride + (size_t)(H + K + g) * D + d];
-        T* vp = v_pages + ((size_t)page * K + g) * D * page_size +
-                kv_value_offset(tiled, page_size, D, off, d);
-        // eight elements in one or two 16-byte stores (the offset is a multiple of 8)
-        if constexpr (sizeof(T) == 2) {
-          *(uint4*)vp = *(const uint4*)vals;
-        } else {
-          *(uint4*)vp = *(const uint4*)vals;
-          *(uint4*)(vp + 4) = *(const uint4*)(vals + 4);
-        }
+      for (int e = 0; e < 8; ++e)
+        vals[e] = qkv[(size_t)(t + e) * row_stride + (size_t)(H + K + g) * D + d];
+      T* vp = v_pages + ((size_t)page * K + g) * D * page_size +
+              kv_value_offset(tiled, page_size, D, off, d);
+      // eight elements in one or two 16-byte stores (the offset is a multiple of 8)
+      if constexpr (sizeof(T) == 2) {
+        *(uint4*)vp = *(const uint4*)vals;
+      } else {
+        *(uint4*)vp = *(const uint4*)vals;
+        *(uint4*)(vp + 4) = *(const uint4*)(vals + 4);
       }
-      return;
     }
+    return;
   }
-  const int d8 = D / 8;
   for (int idx = threadIdx.x; idx < K * d8; idx += blockDim.x) {
     const int g = idx / d8, i = (idx % d8) * 8;
-    const T* vr = row + (size_t)(H + K + g) * D + i;
-    T vals[8];
+    __attribute__((aligned(16))) T vals[8];
+    if (early_values) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) vals[e] = vr[e];
+      for (int u = 0; u < (int)(sizeof(T) / 2); ++u) ((uint4*)vals)[u] = vpre[u];
+    } else {
+      const uint4* vr = (const uint4*)(row + (size_t)(H + K + g) * D + i);
+#pragma unroll
+      for (int u = 0; u < (int)(sizeof(T) / 2); ++u) ((uint4*)vals)[u] = vr[u];
+    }
     T* vp = v_pages + ((size_t)page * K + g) * D * page_size;
 #pragma unroll
     for (int e = 0; e < 8; ++e) vp[kv_value_offset(tiled, page_size, D, off, i + e)] = vals[e];
@@ -549,7 +568,8 @@ extern "C" int hal_rope_append(void* qkv, int dtype, int row_stride, const int* 
   HAL_REQUIRE(!tiled || (page_size % 32 == 0 && D % 32 == 0),
               "hal_rope_append: the tiled page layout needs pages and heads of a multiple of 32 "
               "(page %d, head %d)", page_size, D);
-  const bool vec = D % 8 == 0 && row_stride % 8 == 0 && (interleaved ? rot % 8 == 0 : rot % 16 == 0);
+  const bool vec = D % 8 == 0 && row_stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
+                   (interleaved ? rot % 8 == 0 : rot % 16 == 0);
   if (vec) {
     int items = (H + K) * (rot / 8) / (interleaved ? 1 : 2);
     if (K * (D / 8) > items) items = K * (D / 8);

@@ -29,11 +29,14 @@ WAVES_PER_GROUP = 4  # waves of a workgroup of the kernel for long segments: the
 class AttentionPlan:
     """Work lists of the matrix-core kernel for one step (rows are (token, head of the
     group) pairs, token-major):
-    ``items`` [n, 8]: segment, first row, first key, end key, first partial slot or -1 —
-    tiles of 16 rows of segments with at most 16 rows (decode tokens);
-    ``big_items`` the same for longer segments, ``rows_big`` rows per tile;
+    ``items`` [n, 8]: segment, first row, first key, end key, first partial slot or -1,
+    then the segment's first token, number of tokens and number of keys — tiles of 16 rows
+    of segments with at most 16 rows (decode tokens);
+    ``big_items`` [n, 8] for longer segments: the first five the same, then the first rows
+    of the item's further tiles (-1: none), ``rows_big`` rows per item;
     ``merges`` [n, 8]: segment, first row of a 16-row tile, first partial slot, number of
-    partials, slots between partials."""
+    partials, slots between partials, the segment's first token and number of tokens.
+    A segment's first token is the sum of the lengths of the segments before it."""
 
     items: np.ndarray
     big_items: np.ndarray
@@ -106,10 +109,12 @@ def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick):
     return seg_ids, r0, b, e
 
 
-def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_seg, more_tiles=None, group=1):
+def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, seg_scalars, more_tiles=None, group=1):
     """Items and merge entries of tiles whose key ranges are cut into pieces of
     ``chunk`` keys (pieces end on multiples of 32 keys).  ``more_tiles`` [n, k] holds
-    the first rows of an item's further 16-row tiles (-1: none)."""
+    the first rows of an item's further 16-row tiles (-1: none); without it the items
+    carry their segment's row of ``seg_scalars`` [segments, 3] (first token, tokens,
+    keys) in those places."""
     n_tiles = len(seg_ids)
     if n_tiles == 0:
         return np.zeros((0, 8), np.int32), np.zeros((0, 8), np.int32), first_slot
@@ -127,6 +132,8 @@ def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_
     items[:, 5:] = -1
     if more_tiles is not None:
         items[:, 5 : 5 + more_tiles.shape[1]] = more_tiles[tile_of]
+    else:
+        items[:, 5:8] = seg_scalars[items[:, 0]]
     split = n_pieces[tile_of] > 1
     items[:, 4] = -1
     n_split = int(split.sum())
@@ -145,6 +152,7 @@ def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, rows_of_
     merges[:, 2] = items[first_item[rows_of], 4] + sub[keep]
     merges[:, 3] = n_pieces[rows_of]
     merges[:, 4] = slots_per_tile
+    merges[:, 5:7] = seg_scalars[merges[:, 0], :2]
     if group > 1:
         items = _group_items(items, piece, group)
     else:
@@ -212,7 +220,8 @@ def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: 
     (decode tokens) gives one-tile items; a longer one gives items of ``rows_big / 16``
     tiles that share the keys a wave loads.  Where there are too few items to fill the
     GPU, an item's key range is cut into pieces whose partial results are merged."""
-    rows_of_seg = [int(q) * group_size for q in seg_q_len]
+    ql = np.asarray(seg_q_len, dtype=np.int64).reshape(-1)
+    seg_scalars = np.stack((np.cumsum(ql) - ql, ql, np.asarray(seg_kv_len, dtype=np.int64).reshape(-1)), axis=1)
     per_item = max(1, rows_big // ROWS_PER_ITEM)
     small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: (r <= ROWS_PER_ITEM) | (per_item == 1))
     big = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: (r > ROWS_PER_ITEM) & (per_item > 1))
@@ -226,8 +235,8 @@ def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: 
         total = int((small[3] - small[2]).sum() + (big[3] - big[2]).sum()) * n_kv_heads
         chunk = -(-total // TARGET_WAVES)
         chunk = max(MIN_SPLIT_KEYS, -(-chunk // KEYS_PER_BLOCK) * KEYS_PER_BLOCK)
-    items, merges_s, slot = _cut(*small, chunk, 1, 0, rows_of_seg)
-    big_items, merges_b, slot = _cut(*big, chunk, per_item, slot, rows_of_seg, more, group=WAVES_PER_GROUP)
+    items, merges_s, slot = _cut(*small, chunk, 1, 0, seg_scalars)
+    big_items, merges_b, slot = _cut(*big, chunk, per_item, slot, seg_scalars, more, group=WAVES_PER_GROUP)
     merges = np.concatenate((merges_s, merges_b)) if len(merges_s) or len(merges_b) else np.zeros((0, 8), np.int32)
     return AttentionPlan(items, big_items, merges, slot, rows_big)
 

@@ -25,8 +25,8 @@ def check_plan(plan, q_len, kv_len, group, window):
             assert (rows > 16 and per_item > 1) == is_big
             assert 0 <= b < e <= kv_len[seg]
             tiles = tuple([rho0] + [m for m in more[: per_item - 1] if m >= 0]) if is_big else (rho0,)
-            if not is_big:
-                assert more == [-1, -1, -1]
+            if not is_big:  # the segment's first token, tokens and keys ride along
+                assert more == [int(sum(q_len[:seg])), int(q_len[seg]), int(kv_len[seg])]
             assert all(t % 16 == 0 and 0 <= t < rows for t in tiles)
             groups.setdefault((seg, tiles), []).append((b, e, partial))
     for s in range(len(q_len)):
@@ -57,7 +57,8 @@ def check_plan(plan, q_len, kv_len, group, window):
         assert slots == list(range(slots[0], slots[0] + stride * len(slots), stride))
         for sub, t in enumerate(tiles):
             match = [m for m in plan.merges.tolist() if m[0] == seg and m[1] == t]
-            assert match == [[seg, t, slots[0] + sub, len(slots), stride, 0, 0, 0]]
+            assert match == [[seg, t, slots[0] + sub, len(slots), stride,
+                              int(sum(q_len[:seg])), int(q_len[seg]), 0]]
             n_merges += 1
         for s0 in slots:
             for sub in range(stride):
