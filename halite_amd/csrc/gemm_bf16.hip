@@ -10,6 +10,13 @@
 // can add into a float32 destination (the residual stream), and in the gated form
 // computes up * silu(gate) from two weights at once
 // (src/halite/transformers/feedforward.py:204-212).
+//
+// A third epilogue serves the packed q, k, v projection of few tokens: it rotates q and k
+// by the tokens' positions and appends the rotated k and v to the cache pages, which
+// otherwise is a kernel of its own between this one and attention
+// (src/halite/transformers/position.py:287-291, infer/engine/memory_pool.py:139-141).  The
+// two elements of a rotation pair lie half a head apart; the weight's rows are reordered
+// for this epilogue so that a tile of 16 rows holds eight pairs.
 #include "hal_common.h"
 #include "hal_api.h"
 #include <stdlib.h>
@@ -26,11 +33,28 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* p, bool valid) {
 
 enum { SK_OUT_BF16 = 0, SK_OUT_F32 = 1, SK_OUT_F32_ADD = 2 };
 
-template <int NT, int MT, bool GATED, int U>
+// What the rotating epilogue needs beside the product.  Row r' = head * D + 16 * j + c of
+// the reordered weight is row head * D + 8 * j + c of the stored one for c < 8 and row
+// head * D + D / 2 + 8 * j + (c - 8) for c >= 8: a tile holds dimensions 8j .. 8j + 7 and
+// their partners.  Heads [0, H) are q, [H, H + K) k, [H + K, H + 2K) v.
+struct RopeEpilogue {
+  const int* positions;    // [M]
+  const int* token_seg;    // [M] row of the block table
+  const int* block_table;  // [segments, bt_stride] page numbers
+  int bt_stride;
+  const float* cos_t;  // [table_len, D / 2]
+  const float* sin_t;
+  int table_len;
+  bf16_t* k_pages;
+  bf16_t* v_pages;
+  int H, K, D, page_size, n_pages, tiled;
+};
+
+template <int NT, int MT, bool GATED, int U, bool ROPE = false>
 __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
                                    const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
                                    int ldw, void* __restrict__ C, int ldc, int out_mode, int M,
-                                   int N, int K, int slots) {
+                                   int N, int K, int slots, RopeEpilogue rope = RopeEpilogue{}) {
   extern __shared__ float red[];  // [waves][sets][NT*MT][64][4]
   const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
   const int n_waves = blockDim.x / HAL_WAVE;
@@ -152,6 +176,54 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   }
   __syncthreads();
 
+  if constexpr (ROPE) {
+    static_assert(NT == 1 && MT == 1 && !GATED, "the rotating epilogue takes one tile");
+    // pair p: elements c and c + 8 of the tile, for token m; C is q alone, [M, H * D]
+    const int D = rope.D, half = D / 2, tiles_per_head = D / 16;
+    for (int p = tid; p < 128; p += blockDim.x) {
+      const int c = p / 16, m = p % 16;
+      if (m >= M) continue;
+      const int idx0 = ((c / 4) * 16 + m) * 4 + c % 4, idx1 = idx0 + 128;
+      float v0 = 0.f, v1 = 0.f;
+      for (int w = 0; w < slots; ++w) {
+        v0 += red[(size_t)w * TILE + idx0];
+        v1 += red[(size_t)w * TILE + idx1];
+      }
+      // the product is rounded to bf16 before the rotation, as the unfused way stores it
+      const float x0 = bf16_to_f32(f32_to_bf16(v0)), x1 = bf16_to_f32(f32_to_bf16(v1));
+      const int head = blockIdx.x / tiles_per_head, d0 = (blockIdx.x % tiles_per_head) * 8 + c;
+      const int d1 = d0 + half;
+      const int pos = rope.positions[m];
+      if (pos < 0 || pos >= rope.table_len) continue;  // checked on the host
+      float y0 = x0, y1 = x1;
+      if (head < rope.H + rope.K) {
+        const float cs = rope.cos_t[(size_t)pos * half + d0], sn = rope.sin_t[(size_t)pos * half + d0];
+        y0 = x0 * cs - x1 * sn;
+        y1 = x0 * sn + x1 * cs;
+      }
+      if (head < rope.H) {
+        bf16_t* q = (bf16_t*)C + (size_t)m * ldc + (size_t)head * D;
+        q[d0] = f32_to_bf16(y0);
+        q[d1] = f32_to_bf16(y1);
+        continue;
+      }
+      const long long page =
+          rope.block_table[(size_t)rope.token_seg[m] * rope.bt_stride + pos / rope.page_size];
+      if (page < 0 || page >= rope.n_pages) continue;  // checked on the host
+      const int off = pos % rope.page_size;
+      if (head < rope.H + rope.K) {
+        bf16_t* kp = rope.k_pages + ((size_t)page * rope.K + (head - rope.H)) * rope.page_size * D;
+        kp[kv_key_offset(rope.tiled, rope.page_size, D, off, d0)] = f32_to_bf16(y0);
+        kp[kv_key_offset(rope.tiled, rope.page_size, D, off, d1)] = f32_to_bf16(y1);
+      } else {
+        bf16_t* vp =
+            rope.v_pages + ((size_t)page * rope.K + (head - rope.H - rope.K)) * D * rope.page_size;
+        vp[kv_value_offset(rope.tiled, rope.page_size, D, off, d0)] = f32_to_bf16(y0);
+        vp[kv_value_offset(rope.tiled, rope.page_size, D, off, d1)] = f32_to_bf16(y1);
+      }
+    }
+    return;
+  }
   // element (f, t, lane, i) of the accumulator tile is row n_base + f*16 + (lane/16)*4 + i
   // of W (column of C) and row t*16 + lane%16 of X (row of C)
   for (int idx = tid; idx < NT * MT * 256; idx += blockDim.x) {
@@ -261,4 +333,44 @@ extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const
 #undef SK_LAUNCH
 #undef SK_CASE
   return hal_fail("hal_gemm_bf16_skinny: no kernel for nt=%d mt=%d", nt, mt);
+}
+
+// The packed q, k, v projection of at most 16 tokens with rotation and append in its
+// epilogue.  W is the projection's weight with its rows reordered (see RopeEpilogue) and
+// then laid out in tiles as for hal_gemm_bf16_skinny with ldw == 0; q_out [M, H * D]
+// receives the rotated queries; rotated keys and the values go to the pages of each
+// token's request.  Pairs are (j, j + D/2) and the whole head is rotated.
+extern "C" int hal_qkv_rope_append(const void* X, int ldx, const void* W, void* q_out, int M,
+                                   int K_in, const int* positions, const int* token_seg,
+                                   const int* block_table, int bt_stride, const float* cos_t,
+                                   const float* sin_t, int table_len, void* k_pages,
+                                   void* v_pages, int H, int K, int D, int page_size, int n_pages,
+                                   int tiled, hipStream_t stream) {
+  HAL_REQUIRE(M >= 0 && M <= 16, "hal_qkv_rope_append: M=%d (at most 16 tokens)", M);
+  HAL_REQUIRE(H > 0 && K > 0 && D > 0 && D % 16 == 0, "hal_qkv_rope_append: heads %d, %d, size %d",
+              H, K, D);
+  HAL_REQUIRE(K_in > 0 && K_in % 8 == 0 && ldx >= K_in && ldx % 8 == 0,
+              "hal_qkv_rope_append: inner size %d, leading dimension %d", K_in, ldx);
+  HAL_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0,
+              "hal_qkv_rope_append: operands must be 16-byte aligned");
+  HAL_REQUIRE(positions && token_seg && block_table && cos_t && sin_t && k_pages && v_pages &&
+                  q_out && page_size > 0 && n_pages > 0 && table_len > 0,
+              "hal_qkv_rope_append: arguments missing");
+  HAL_REQUIRE(!tiled || (page_size % 32 == 0 && D % 32 == 0),
+              "hal_qkv_rope_append: the tiled page layout needs pages and heads of a multiple "
+              "of 32 (page %d, head %d)", page_size, D);
+  if (M == 0) return 0;
+  const int N = (H + 2 * K) * D;
+  const int blocks = N / 16, steps = (K_in + 31) / 32;
+  int waves = 4;  // as hal_gemm_bf16_skinny chooses them
+  while (waves < 16 && blocks * waves < 4096 && steps / (waves * 2) >= 4) waves *= 2;
+  RopeEpilogue rope{positions, token_seg, block_table, bt_stride, cos_t, sin_t, table_len,
+                    (bf16_t*)k_pages, (bf16_t*)v_pages, H, K, D, page_size, n_pages, tiled};
+  const size_t smem = (size_t)waves * 256 * sizeof(float);
+  hipLaunchKernelGGL((skinny_gemm_kernel<1, 1, false, 8, true>), dim3(blocks),
+                     dim3(waves * HAL_WAVE), smem, stream, (const bf16_t*)X, ldx,
+                     (const bf16_t*)W, (const bf16_t*)nullptr, 0, q_out, H * D, SK_OUT_BF16, M, N,
+                     K_in, waves, rope);
+  HAL_LAUNCH_CHECK();
+  return 0;
 }

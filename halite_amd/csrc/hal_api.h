@@ -44,6 +44,16 @@ int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, float* C, int
 int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const void* W2, int ldw, void* C,
                          int ldc, int out_mode, int M, int N, int K, hipStream_t stream);
 
+// The packed q, k, v projection of M <= 16 tokens with the rotation of q and k (pairs
+// (j, j + D/2), whole head) and the append of k and v to the pages in its epilogue.  W:
+// the weight's rows reordered per head to [8j .. 8j+7, D/2 + 8j .. D/2 + 8j+7] for
+// j = 0 .. D/16 - 1, then tiled as for ldw == 0 above.  q_out [M, H * D] bf16.
+int hal_qkv_rope_append(const void* X, int ldx, const void* W, void* q_out, int M, int K_in,
+                        const int* positions, const int* token_seg, const int* block_table,
+                        int bt_stride, const float* cos_t, const float* sin_t, int table_len,
+                        void* k_pages, void* v_pages, int H, int K, int D, int page_size,
+                        int n_pages, int tiled, hipStream_t stream);
+
 int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temperature,
                const int* top_k, const float* top_p, const float* min_p, const uint64_t* seeds,
                const int* draw_index, int* out_token, float* out_logprob, uint32_t* key_rows,

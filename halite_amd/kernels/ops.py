@@ -197,6 +197,71 @@ def rope_append(
     )
 
 
+def pair_rows_for_rotation(w_qkv: torch.Tensor, head_dim: int) -> torch.Tensor:
+    """The packed q, k, v weight with the rows of every head reordered to
+    ``[8j .. 8j+7, D/2 + 8j .. D/2 + 8j+7]`` for ``j = 0 .. D/16 - 1``, so that a tile of
+    16 rows holds eight rotation pairs ``(d, d + D/2)``: the order ``qkv_rope_append``
+    takes (after ``tile_weight``)."""
+    n, _ = w_qkv.shape
+    _need(head_dim % 16 == 0 and n % head_dim == 0, "pair_rows_for_rotation: head size in steps of 16")
+    within = torch.arange(head_dim, device=w_qkv.device).view(2, head_dim // 16, 8).permute(1, 0, 2).reshape(-1)
+    heads = torch.arange(n // head_dim, device=w_qkv.device) * head_dim
+    return w_qkv[(heads[:, None] + within[None, :]).reshape(-1)]
+
+
+def qkv_rope_append(
+    x: torch.Tensor,
+    w_paired_tiled: torch.Tensor,
+    positions: torch.Tensor,
+    cos: torch.Tensor,
+    sin: torch.Tensor,
+    n_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    token_seg: torch.Tensor,
+    block_table: torch.Tensor,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    page_size: int,
+    tiled: bool = False,
+) -> torch.Tensor:
+    """The packed q, k, v projection of at most 16 bf16 rows, the rotation of q and k
+    (pairs ``(j, j + D/2)``, the whole head) and the append of k and v to the pages, in
+    one kernel.  ``w_paired_tiled`` is ``tile_weight(pair_rows_for_rotation(w_qkv, D))``.
+    Returns the rotated queries ``[rows, n_heads * head_dim]``."""
+    lib = library.core_library()
+    _dev(x, w_paired_tiled, positions, cos, sin, token_seg, block_table, k_pages, v_pages)
+    _i32(positions, "positions"), _i32(token_seg, "token_seg"), _i32(block_table, "block_table")
+    m, k = x.shape
+    n = (n_heads + 2 * n_kv_heads) * head_dim
+    _need(x.dtype == torch.bfloat16 and x.stride(1) == 1 and m <= SKINNY_ROWS, "qkv_rope_append: up to 16 bf16 rows")
+    _need(head_dim % 16 == 0 and k % 8 == 0, "qkv_rope_append: head size in steps of 16, width in steps of 8")
+    _need(
+        w_paired_tiled.dtype == torch.bfloat16 and w_paired_tiled.is_contiguous()
+        and w_paired_tiled.numel() == n * (-(-k // 32) * 32),
+        "qkv_rope_append: tiled weight",
+    )
+    _need(positions.numel() == m and token_seg.numel() == m and block_table.dim() == 2, "qkv_rope_append: step arrays")
+    _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape
+          and cos.dim() == 2 and cos.shape[1] == head_dim // 2 and cos.is_contiguous() and sin.is_contiguous(),
+          "qkv_rope_append: rotation tables")
+    n_pages = k_pages.shape[0]
+    _need(k_pages.dtype == torch.bfloat16 and v_pages.dtype == torch.bfloat16
+          and k_pages.shape == (n_pages, n_kv_heads, page_size, head_dim)
+          and v_pages.shape == (n_pages, n_kv_heads, head_dim, page_size), "qkv_rope_append: pages")
+    q = torch.empty((m, n_heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    _check(
+        lib,
+        lib.hal_qkv_rope_append(
+            _ptr(x), x.stride(0), _ptr(w_paired_tiled), _ptr(q), m, k, _ptr(positions), _ptr(token_seg),
+            _ptr(block_table), block_table.shape[1], _ptr(cos), _ptr(sin), cos.shape[0],
+            _ptr(k_pages), _ptr(v_pages), n_heads, n_kv_heads, head_dim, page_size, n_pages,
+            1 if tiled else 0, _stream(),
+        ),
+    )
+    return q
+
+
 def attention_simple(
     q: torch.Tensor,
     q_row_stride: int,

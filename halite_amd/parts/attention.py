@@ -72,14 +72,22 @@ class Attention(Mixer):
         }
 
     def finalize(self):
-        self.t_qkv = self.t_q = self.t_out = None
+        self.t_qkv = self.t_q = self.t_out = self.t_qkv_paired = None
         if self.build.tiled_weights and self.w_qkv.dtype == torch.bfloat16 and self.w_qkv.is_cuda:
-            self.t_qkv = ops.tile_weight(self.w_qkv)
+            p = self.p
             self.t_out = ops.tile_weight(self.w_out) if self.w_out.dtype == torch.bfloat16 else None
-            n_q = self.p.n_heads * self.p.head_dim
-            if n_q % 16 == 0:  # the q rows are whole tiles at the front
-                steps = -(-self.p.hidden_size // 32)
-                self.t_q = self.t_qkv[: (n_q // 16) * steps * 512]
+            pos = self.position
+            if (pos is not None and not pos.interleaved and pos.rotary_dim == p.head_dim
+                    and p.head_dim % 16 == 0 and p.hidden_size % 8 == 0 and self.build.dtype == torch.bfloat16):
+                # few tokens: projection, rotation and append are one kernel, which takes
+                # the rows of a head in an order of its own
+                self.t_qkv_paired = ops.tile_weight(ops.pair_rows_for_rotation(self.w_qkv, p.head_dim))
+            else:
+                self.t_qkv = ops.tile_weight(self.w_qkv)
+                n_q = p.n_heads * p.head_dim
+                if n_q % 16 == 0:  # the q rows are whole tiles at the front
+                    steps = -(-p.hidden_size // 32)
+                    self.t_q = self.t_qkv[: (n_q // 16) * steps * 512]
 
     def cache_need(self):
         return PagedKVNeed(self.p.n_kv_heads, self.p.head_dim, self.p.window)
@@ -94,6 +102,15 @@ class Attention(Mixer):
         kv = run.kv
         group = ctx.group(kv.group_id)
         n_q = p.n_heads * p.head_dim
+        if (run.appends and self.t_qkv_paired is not None and x.shape[0] <= ops.SKINNY_ROWS
+                and x.dtype == torch.bfloat16 and kv.k.dtype == torch.bfloat16):
+            cos, sin = self.position.tables(ctx.max_position + 1)
+            q = ops.qkv_rope_append(
+                x, self.t_qkv_paired, ctx.positions, cos, sin, p.n_heads, p.n_kv_heads, p.head_dim,
+                ctx.token_seg, group.block_table, kv.k, kv.v, group.page_size, kv.tiled,
+            )
+            out = ctx.attention(q, q.shape[1], kv, group, p.n_heads, p.scale, p.window or 0)
+            return ops.linear(out, self.w_out, tiled=self.t_out)
         if run.appends:
             qkv = ops.linear(x, self.w_qkv, tiled=self.t_qkv)
             n_kv_append = p.n_kv_heads

@@ -192,6 +192,51 @@ def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page, tiled):
     assert float(vpc.abs().sum(dim=(1, 2))[~written].sum()) == 0
 
 
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("H,K,D,width,page,tiled", [
+    (4, 2, 16, 64, 8, False), (6, 3, 48, 120, 16, False), (5, 1, 80, 200, 4, False),
+    (8, 2, 64, 352, 32, True), (32, 8, 128, 4096, 64, True), (2, 2, 160, 96, 64, True),
+])
+def test_qkv_rope_append_in_one_kernel(gpu, M, H, K, D, width, page, tiled):
+    """Projection, rotation and append in one kernel against the three steps one by one
+    (the same kernels' unfused forms) and against the plain rotation."""
+    dt = torch.bfloat16
+    n_seg, table_w = 3, -(-64 // page)
+    # tokens of three requests: a run of neighbouring positions, and single ones
+    lens = [M - 2, 1, 1] if M > 2 else [M]
+    starts = [11, 40, 0][: len(lens)]
+    positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).to(torch.int32)
+    token_seg = torch.cat([torch.full((n,), i) for i, n in enumerate(lens)]).to(torch.int32)
+    n_pages = n_seg * table_w + 5
+    bt = (torch.randperm(n_pages - 1, generator=torch.Generator().manual_seed(2))[: n_seg * table_w]
+          .view(n_seg, table_w) + 1).to(torch.int32)
+    w = (rnd((H + 2 * K) * D, width, seed=3) * 0.2).to(dt).to(gpu)
+    x = rnd(M, width, seed=4).to(dt).to(gpu)
+    cos, sin = P.rotation_table(torch.arange(64), P.inverse_frequencies(D, 10000.0))
+    cos, sin = cos.contiguous().to(gpu), sin.contiguous().to(gpu)
+    pages = lambda: (torch.zeros(n_pages, K, page, D, dtype=dt, device=gpu), torch.zeros(n_pages, K, D, page, dtype=dt, device=gpu))
+
+    paired = ops.tile_weight(ops.pair_rows_for_rotation(w, D))
+    kp, vp = pages()
+    q = ops.qkv_rope_append(x, paired, positions.to(gpu), cos, sin, H, K, D, token_seg.to(gpu), bt.to(gpu),
+                            kp, vp, page, tiled)
+
+    qkv = ops.gemm_bf16_skinny(x, ops.tile_weight(w), tiled_shape=tuple(w.shape))
+    plain_qkv = qkv.float().cpu()
+    kp2, vp2 = pages()
+    ops.rope_append(qkv, positions.to(gpu), cos, sin, H, K, D, D, False, token_seg=token_seg.to(gpu),
+                    block_table=bt.to(gpu), k_pages=kp2, v_pages=vp2, page_size=page, tiled=tiled)
+    # the same sums in the same order, rounded at the same places
+    close(q, qkv[:, : H * D], 4e-3, "rotated q, fused against unfused")
+    close(kp, kp2, 4e-3, "key pages")
+    assert torch.equal(vp, vp2)
+    # and the rotation itself against the plain one, from the unrotated product
+    c, s_ = cos.cpu()[positions.long()], sin.cpu()[positions.long()]
+    want_q = P.rotate_half_split(plain_qkv[:, : H * D].view(M, H, D), c, s_)
+    close(q.view(M, H, D), want_q, 8e-3, "rotated q against the plain rotation")
+    assert float(kp.float().abs().sum()) > 0
+
+
 def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use, tiled=False):
     """``segs``: list of (cached before, new tokens).  Builds one dense sequence per
     segment, pages it, and compares the rows of the new tokens with plain attention
