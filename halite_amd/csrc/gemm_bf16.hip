@@ -17,6 +17,14 @@
 // (src/halite/transformers/position.py:287-291, infer/engine/memory_pool.py:139-141).  The
 // two elements of a rotation pair lie half a head apart; the weight's rows are reordered
 // for this epilogue so that a tile of 16 rows holds eight pairs.
+//
+// With at most 16 rows the RMSNorm between two products (src/halite/nn/normalization.py:
+// 43-57, src/halite/transformers/block.py:56-74) needs no kernel of its own.  The product
+// before it (PREP) adds its result into the float32 residual stream h, writes
+// bf16(w * bf16(h)) for the norm's weight w, and leaves one sum of h^2 per row and
+// workgroup; the product after it (SCALED) adds those sums up in a fixed order and
+// multiplies its float32 accumulators by rsqrt(mean(h^2) + eps), which is the same number
+// up to the place of one bf16 rounding (the norm's kernel rounds h * rstd, this way rounds h).
 #include "hal_common.h"
 #include "hal_api.h"
 #include <stdlib.h>
@@ -50,11 +58,35 @@ struct RopeEpilogue {
   int H, K, D, page_size, n_pages, tiled;
 };
 
-template <int NT, int MT, bool GATED, int U, bool ROPE = false>
+// The norm folded into the products around it (at most 16 rows).
+struct NormFusion {
+  // SCALED: X holds bf16(w * bf16(h)); sums of h^2, [n_parts][16], one row of 16 per
+  // workgroup of the product before; the norm's eps (its size is this product's K)
+  const float* ss_in;
+  int n_parts;
+  float eps;
+  // PREP: C is h (float32, added into); the next norm's weight [N], where bf16(w * bf16(h))
+  // goes ([M, N] bf16) and where this workgroup's sums of h^2 go ([workgroups][16])
+  const void* norm_w;
+  int norm_w_dtype;
+  bf16_t* xw_out;
+  float* ss_out;
+};
+enum { SK_ROPE = 1, SK_SCALED = 2, SK_PREP = 4 };
+#define SK_MAX_PART_LOADS 4  // float4 loads of partial sums per thread, at most
+
+// PL: float4 loads of partial sums per thread (SCALED), held in registers through the loop
+template <int NT, int MT, bool GATED, int U, int FLAGS = 0, int PL = 1>
 __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
                                    const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
                                    int ldw, void* __restrict__ C, int ldc, int out_mode, int M,
-                                   int N, int K, int slots, RopeEpilogue rope = RopeEpilogue{}) {
+                                   int N, int K, int slots, RopeEpilogue rope = RopeEpilogue{},
+                                   NormFusion nf = NormFusion{}) {
+  constexpr bool ROPE = (FLAGS & SK_ROPE) != 0, SCALED = (FLAGS & SK_SCALED) != 0,
+                 PREP = (FLAGS & SK_PREP) != 0;
+  static_assert(!(SCALED || PREP) || MT == 1, "the folded norm serves at most 16 rows");
+  static_assert(!PREP || (NT == 1 && !GATED && !ROPE && !SCALED), "PREP takes one plain tile");
+  __shared__ float row_sums[16][16];  // SCALED: [wave][row]; PREP: [column of the tile][row]
   extern __shared__ float red[];  // [waves][sets][NT*MT][64][4]
   const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
   const int n_waves = blockDim.x / HAL_WAVE;
@@ -66,6 +98,21 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   const int per_wave = (steps + n_waves - 1) / n_waves;
   const int s_begin = wave * per_wave;
   const int s_end = s_begin + per_wave < steps ? s_begin + per_wave : steps;
+
+  // SCALED: this thread's share of the partial sums is asked for before anything else, so
+  // that it has arrived long before the epilogue; float4 f holds rows 4 (f % 4) .. + 3 of
+  // part f / 4, and f % 4 == lane % 4 for every f of a thread
+  // (a load past the end is clamped here and dropped where the sums are added)
+  float4 my_parts[PL];
+  if constexpr (SCALED) {
+    const float4* pp = (const float4*)nf.ss_in;
+    const int last = nf.n_parts * 4 - 1;
+#pragma unroll
+    for (int k = 0; k < PL; ++k) {
+      const int f = tid + k * (int)blockDim.x;
+      my_parts[k] = pp[f < last ? f : last];
+    }
+  }
 
   f32x4 acc[SETS][NT][MT];
 #pragma unroll
@@ -174,7 +221,29 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
         for (int t = 0; t < MT; ++t)
           *(f32x4*)(mine + ((s * NT + f) * MT + t) * 256 + lane * 4) = acc[s][f][t];
   }
+  if constexpr (SCALED) {
+    // sums over the parts in a fixed order: this thread's loads, then the lanes that hold
+    // the same rows (a butterfly), then the waves (by whoever needs a row, in wave order)
+    float4 sum = float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < PL; ++k) {
+      if (tid + k * (int)blockDim.x < nf.n_parts * 4)
+        sum.x += my_parts[k].x, sum.y += my_parts[k].y, sum.z += my_parts[k].z, sum.w += my_parts[k].w;
+    }
+#pragma unroll
+    for (int off = 4; off < HAL_WAVE; off <<= 1) {
+      sum.x += __shfl_xor(sum.x, off, HAL_WAVE), sum.y += __shfl_xor(sum.y, off, HAL_WAVE);
+      sum.z += __shfl_xor(sum.z, off, HAL_WAVE), sum.w += __shfl_xor(sum.w, off, HAL_WAVE);
+    }
+    if (lane < 4) *(float4*)&row_sums[wave][lane * 4] = sum;
+  }
   __syncthreads();
+  // rsqrt(mean(h^2) + eps) of row m, as the norm's own kernel computes it
+  auto row_scale = [&](int m) {
+    float total = 0.f;
+    for (int w = 0; w < n_waves; ++w) total += row_sums[w][m];
+    return 1.0f / sqrtf(total / (float)K + nf.eps);
+  };
 
   if constexpr (ROPE) {
     static_assert(NT == 1 && MT == 1 && !GATED, "the rotating epilogue takes one tile");
@@ -188,6 +257,10 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
       for (int w = 0; w < slots; ++w) {
         v0 += red[(size_t)w * TILE + idx0];
         v1 += red[(size_t)w * TILE + idx1];
+      }
+      if constexpr (SCALED) {
+        const float rs = row_scale(m);
+        v0 *= rs, v1 *= rs;
       }
       // the product is rounded to bf16 before the rotation, as the unfused way stores it
       const float x0 = bf16_to_f32(f32_to_bf16(v0)), x1 = bf16_to_f32(f32_to_bf16(v1));
@@ -224,6 +297,34 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
     }
     return;
   }
+  if constexpr (PREP) {
+    // thread (column c of the tile, row m): h += product (rounded to bf16 first, as the
+    // unfused way hands it on), the next norm's input, and h^2 for the row's sum
+    if (tid < 256) {
+      const int c = tid / 16, m = tid % 16, n = n_base + c;
+      const int idx = ((c / 4) * 16 + m) * 4 + c % 4;
+      float sq = 0.f;
+      if (n < N && m < M) {
+        float v = 0.f;
+        for (int w = 0; w < slots; ++w) v += red[(size_t)w * TILE + idx];
+        float* hp = (float*)C + (size_t)m * ldc + n;
+        const float h = *hp + bf16_to_f32(f32_to_bf16(v));
+        *hp = h;
+        const float wn = load_as_f32(nf.norm_w, nf.norm_w_dtype, n);
+        nf.xw_out[(size_t)m * N + n] = f32_to_bf16(wn * bf16_to_f32(f32_to_bf16(h)));
+        sq = h * h;
+      }
+      row_sums[c][m] = sq;
+    }
+    __syncthreads();
+    if (tid < 16) {
+      float total = 0.f;
+#pragma unroll
+      for (int c = 0; c < 16; ++c) total += row_sums[c][tid];
+      nf.ss_out[(size_t)blockIdx.x * 16 + tid] = total;
+    }
+    return;
+  }
   // element (f, t, lane, i) of the accumulator tile is row n_base + f*16 + (lane/16)*4 + i
   // of W (column of C) and row t*16 + lane%16 of X (row of C)
   for (int idx = tid; idx < NT * MT * 256; idx += blockDim.x) {
@@ -237,6 +338,10 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
       v += red[(size_t)w * TILE + idx];
       if (GATED) v2 += red[(size_t)w * TILE + NT * MT * 256 + idx];
     }
+    if constexpr (SCALED) {
+      const float rs = row_scale(m);
+      v *= rs, v2 *= rs;
+    }
     if (GATED) v = v2 * (v / (1.0f + expf(-v)));  // set 0 is the gate, set 1 is up
     const size_t o = (size_t)m * ldc + n;
     if (out_mode == SK_OUT_BF16)
@@ -248,10 +353,11 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   }
 }
 
-template <int NT, int MT, bool GATED, int U>
+template <int NT, int MT, bool GATED, int U, int FLAGS = 0, int PL = 1>
 static int launch_skinny(const bf16_t* X, int ldx, const bf16_t* W, const bf16_t* W2, int ldw,
                          void* C, int ldc, int out_mode, int M, int N, int K, int waves,
-                         hipStream_t stream) {
+                         hipStream_t stream, RopeEpilogue rope = RopeEpilogue{},
+                         NormFusion nf = NormFusion{}) {
   constexpr int SETS = GATED ? 2 : 1;
   // LDS for the partial sums of all waves, or of a half, a quarter ... if that is too much
   const size_t per_wave = (size_t)SETS * NT * MT * 256 * sizeof(float);
@@ -259,11 +365,28 @@ static int launch_skinny(const bf16_t* X, int ldx, const bf16_t* W, const bf16_t
   while (slots > 1 && (size_t)slots * per_wave > 64 * 1024) slots /= 2;
   const size_t smem = (size_t)slots * per_wave;
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
-  hipLaunchKernelGGL((skinny_gemm_kernel<NT, MT, GATED, U>), dim3(blocks),
+  if constexpr ((FLAGS & SK_SCALED) != 0 && PL < SK_MAX_PART_LOADS) {
+    if (nf.n_parts * 4 > PL * waves * HAL_WAVE)  // more loads per thread
+      return launch_skinny<NT, MT, GATED, U, FLAGS, PL * 2>(X, ldx, W, W2, ldw, C, ldc, out_mode, M,
+                                                            N, K, waves, stream, rope, nf);
+  }
+  if ((FLAGS & SK_SCALED) && nf.n_parts * 4 > PL * waves * HAL_WAVE)
+    return hal_fail("skinny gemm: %d partial sums per row are more than %d threads take",
+                    nf.n_parts, waves * HAL_WAVE);
+  hipLaunchKernelGGL((skinny_gemm_kernel<NT, MT, GATED, U, FLAGS, PL>), dim3(blocks),
                      dim3(waves * HAL_WAVE), smem, stream, X, ldx, W, W2, ldw, C, ldc, out_mode,
-                     M, N, K, slots);
+                     M, N, K, slots, rope, nf);
   HAL_LAUNCH_CHECK();
   return 0;
+}
+
+// Waves per workgroup, which split K among them: more where there are few workgroups, up
+// to about 1,536 waves in all (measured on the projections of a 4,096-wide model at 1 and
+// 8 rows: beyond that the products of 256 to 384 workgroups get 1 to 2 us slower).
+static int skinny_waves(int blocks, int steps) {
+  int waves = 4;
+  while (waves < 16 && blocks * waves < 1536 && steps / (waves * 2) >= 4) waves *= 2;
+  return waves;
 }
 
 // X [M, K] bf16 (M <= 64), W [N, K] bf16, optional W2 [N, K] (gated form: W is the
@@ -298,8 +421,7 @@ extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const
   const int blocks = (N + 16 * nt - 1) / (16 * nt);
   const int steps = (K + 31) / 32;
   if (waves <= 0) {
-    waves = 4;
-    while (waves < 16 && blocks * waves < 4096 && steps / (waves * 2) >= 4) waves *= 2;
+    waves = skinny_waves(blocks, steps);
   }
   while (waves > 1 && (size_t)sets * nt * mt * 1024 > 64 * 1024) waves /= 2;  // one tile must fit
   // loads in flight per wave: about 16 fragments of 16 bytes
@@ -335,6 +457,47 @@ extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const
   return hal_fail("hal_gemm_bf16_skinny: no kernel for nt=%d mt=%d", nt, mt);
 }
 
+// The same product for at most 16 rows with the RMSNorm before or after it folded in.
+// ss_in (or null): X holds bf16(w * bf16(h)) of the norm before this product and ss_in
+// [n_parts, 16] the partial sums of h^2 that the product before left; the result is scaled
+// by rsqrt(sum / K + eps) per row.  norm_w (or null, not with W2): C is the float32 stream
+// h [M, N]; the result is added into it, xw_out [M, N] receives bf16(norm_w * bf16(h)) and
+// ss_out [ceil(N / 16), 16] this product's partial sums of h^2 for the product after.
+// Without norm_w the result goes to C as bf16.
+extern "C" int hal_gemm_bf16_skinny_norm(const void* X, int ldx, const void* W, const void* W2,
+                                         int ldw, void* C, int ldc, int M, int N, int K,
+                                         const float* ss_in, int n_parts, float eps,
+                                         const void* norm_w, int norm_w_dtype, void* xw_out,
+                                         float* ss_out, hipStream_t stream) {
+  HAL_REQUIRE(M >= 0 && M <= 16, "hal_gemm_bf16_skinny_norm: M=%d (at most 16 rows)", M);
+  HAL_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "hal_gemm_bf16_skinny_norm: N=%d K=%d", N, K);
+  HAL_REQUIRE(ldx >= K && (ldw >= K || ldw == 0) && ldc >= N && ldx % 8 == 0 && ldw % 8 == 0,
+              "hal_gemm_bf16_skinny_norm: leading dimensions %d %d %d", ldx, ldw, ldc);
+  HAL_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)W2 % 16) == 0 &&
+                  ((uintptr_t)ss_in % 16) == 0,
+              "hal_gemm_bf16_skinny_norm: operands must be 16-byte aligned");
+  HAL_REQUIRE((ss_in != nullptr) != (norm_w != nullptr),
+              "hal_gemm_bf16_skinny_norm: the norm before the product or the one after it");
+  HAL_REQUIRE(!ss_in || (n_parts > 0 && eps > 0.f), "hal_gemm_bf16_skinny_norm: parts %d", n_parts);
+  HAL_REQUIRE(!norm_w || (!W2 && xw_out && ss_out && (norm_w_dtype == HAL_F32 || norm_w_dtype == HAL_BF16)),
+              "hal_gemm_bf16_skinny_norm: arguments of the norm after the product");
+  if (M == 0) return 0;
+  const int blocks = (N + 15) / 16, steps = (K + 31) / 32;
+  const int waves = skinny_waves(blocks, steps);
+  NormFusion nf{ss_in, n_parts, eps, norm_w, norm_w_dtype, (bf16_t*)xw_out, ss_out};
+  const bf16_t* x = (const bf16_t*)X;
+  const bf16_t* w = (const bf16_t*)W;
+  const bf16_t* w2 = (const bf16_t*)W2;
+  if (w2)
+    return launch_skinny<1, 1, true, 4, SK_SCALED>(x, ldx, w, w2, ldw, C, ldc, SK_OUT_BF16, M, N, K,
+                                                   waves, stream, RopeEpilogue{}, nf);
+  if (norm_w)
+    return launch_skinny<1, 1, false, 8, SK_PREP>(x, ldx, w, nullptr, ldw, C, ldc, SK_OUT_F32_ADD, M,
+                                                  N, K, waves, stream, RopeEpilogue{}, nf);
+  return launch_skinny<1, 1, false, 8, SK_SCALED>(x, ldx, w, nullptr, ldw, C, ldc, SK_OUT_BF16, M, N,
+                                                  K, waves, stream, RopeEpilogue{}, nf);
+}
+
 // The packed q, k, v projection of at most 16 tokens with rotation and append in its
 // epilogue.  W is the projection's weight with its rows reordered (see RopeEpilogue) and
 // then laid out in tiles as for hal_gemm_bf16_skinny with ldw == 0; q_out [M, H * D]
@@ -345,8 +508,11 @@ extern "C" int hal_qkv_rope_append(const void* X, int ldx, const void* W, void* 
                                    const int* block_table, int bt_stride, const float* cos_t,
                                    const float* sin_t, int table_len, void* k_pages,
                                    void* v_pages, int H, int K, int D, int page_size, int n_pages,
-                                   int tiled, hipStream_t stream) {
+                                   int tiled, const float* ss_in, int n_parts, float eps,
+                                   hipStream_t stream) {
   HAL_REQUIRE(M >= 0 && M <= 16, "hal_qkv_rope_append: M=%d (at most 16 tokens)", M);
+  HAL_REQUIRE(!ss_in || (n_parts > 0 && eps > 0.f && ((uintptr_t)ss_in % 16) == 0),
+              "hal_qkv_rope_append: partial sums of the norm before");
   HAL_REQUIRE(H > 0 && K > 0 && D > 0 && D % 16 == 0, "hal_qkv_rope_append: heads %d, %d, size %d",
               H, K, D);
   HAL_REQUIRE(K_in > 0 && K_in % 8 == 0 && ldx >= K_in && ldx % 8 == 0,
@@ -362,15 +528,15 @@ extern "C" int hal_qkv_rope_append(const void* X, int ldx, const void* W, void* 
   if (M == 0) return 0;
   const int N = (H + 2 * K) * D;
   const int blocks = N / 16, steps = (K_in + 31) / 32;
-  int waves = 4;  // as hal_gemm_bf16_skinny chooses them
-  while (waves < 16 && blocks * waves < 4096 && steps / (waves * 2) >= 4) waves *= 2;
+  const int waves = skinny_waves(blocks, steps);
   RopeEpilogue rope{positions, token_seg, block_table, bt_stride, cos_t, sin_t, table_len,
                     (bf16_t*)k_pages, (bf16_t*)v_pages, H, K, D, page_size, n_pages, tiled};
-  const size_t smem = (size_t)waves * 256 * sizeof(float);
-  hipLaunchKernelGGL((skinny_gemm_kernel<1, 1, false, 8, true>), dim3(blocks),
-                     dim3(waves * HAL_WAVE), smem, stream, (const bf16_t*)X, ldx,
-                     (const bf16_t*)W, (const bf16_t*)nullptr, 0, q_out, H * D, SK_OUT_BF16, M, N,
-                     K_in, waves, rope);
-  HAL_LAUNCH_CHECK();
-  return 0;
+  NormFusion nf{ss_in, n_parts, eps, nullptr, 0, nullptr, nullptr};
+  if (ss_in)
+    return launch_skinny<1, 1, false, 8, SK_ROPE | SK_SCALED>(
+        (const bf16_t*)X, ldx, (const bf16_t*)W, nullptr, 0, q_out, H * D, SK_OUT_BF16, M, N, K_in,
+        waves, stream, rope, nf);
+  return launch_skinny<1, 1, false, 8, SK_ROPE>((const bf16_t*)X, ldx, (const bf16_t*)W, nullptr, 0,
+                                                q_out, H * D, SK_OUT_BF16, M, N, K_in, waves,
+                                                stream, rope, nf);
 }

@@ -47,12 +47,23 @@ int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const void* W2, 
 // The packed q, k, v projection of M <= 16 tokens with the rotation of q and k (pairs
 // (j, j + D/2), whole head) and the append of k and v to the pages in its epilogue.  W:
 // the weight's rows reordered per head to [8j .. 8j+7, D/2 + 8j .. D/2 + 8j+7] for
-// j = 0 .. D/16 - 1, then tiled as for ldw == 0 above.  q_out [M, H * D] bf16.
+// j = 0 .. D/16 - 1, then tiled as for ldw == 0 above.  q_out [M, H * D] bf16.  ss_in (or
+// null), n_parts, eps: the norm before the projection, as for hal_gemm_bf16_skinny_norm.
 int hal_qkv_rope_append(const void* X, int ldx, const void* W, void* q_out, int M, int K_in,
                         const int* positions, const int* token_seg, const int* block_table,
                         int bt_stride, const float* cos_t, const float* sin_t, int table_len,
                         void* k_pages, void* v_pages, int H, int K, int D, int page_size,
-                        int n_pages, int tiled, hipStream_t stream);
+                        int n_pages, int tiled, const float* ss_in, int n_parts, float eps,
+                        hipStream_t stream);
+
+// The product for M <= 16 rows with the RMSNorm before it (ss_in: partial sums of squares
+// [n_parts, 16] left by the product before; X holds bf16(w * bf16(h))) or after it
+// (norm_w: C is the float32 stream h, added into; xw_out [M, N] and ss_out [ceil(N/16), 16]
+// are left for the product after) folded in.
+int hal_gemm_bf16_skinny_norm(const void* X, int ldx, const void* W, const void* W2, int ldw,
+                              void* C, int ldc, int M, int N, int K, const float* ss_in,
+                              int n_parts, float eps, const void* norm_w, int norm_w_dtype,
+                              void* xw_out, float* ss_out, hipStream_t stream);
 
 int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temperature,
                const int* top_k, const float* top_p, const float* min_p, const uint64_t* seeds,

@@ -9,6 +9,7 @@ functions: without a GPU and the built library they raise.
 from __future__ import annotations
 
 import ctypes
+from dataclasses import dataclass
 
 import torch
 
@@ -20,6 +21,43 @@ _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 class KernelError(RuntimeError):
     pass
+
+
+@dataclass
+class NextNorm:
+    """What a part's last product is told about the RMSNorm that reads its result: the
+    float32 residual stream the result is added into, and the norm's weight and eps."""
+
+    h: torch.Tensor
+    weight: torch.Tensor
+    eps: float
+
+
+@dataclass
+class NormedRows:
+    """At most 16 rows on their way through an RMSNorm whose scaling is left to the product
+    that reads them: ``x`` [rows, d] is ``bf16(weight * bf16(h))`` and ``ss_parts``
+    [parts, 16] holds partial sums of ``h^2`` per row, so the norm's output is
+    ``x * rsqrt(ss_parts.sum(0) / d + eps)`` row by row."""
+
+    x: torch.Tensor
+    ss_parts: torch.Tensor
+    eps: float
+    weight: torch.Tensor  # of the norm the rows were prepared for
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+    @property
+    def dtype(self):
+        return self.x.dtype
+
+    def materialize(self) -> torch.Tensor:
+        """The norm's output as a tensor, for a reader that does not scale by itself."""
+        m, d = self.x.shape
+        rstd = torch.rsqrt(self.ss_parts.sum(0)[:m] / d + self.eps)
+        return (self.x.float() * rstd[:, None]).to(self.x.dtype)
 
 
 def dtype_code(dtype: torch.dtype) -> int:
@@ -227,9 +265,13 @@ def qkv_rope_append(
 ) -> torch.Tensor:
     """The packed q, k, v projection of at most 16 bf16 rows, the rotation of q and k
     (pairs ``(j, j + D/2)``, the whole head) and the append of k and v to the pages, in
-    one kernel.  ``w_paired_tiled`` is ``tile_weight(pair_rows_for_rotation(w_qkv, D))``.
+    one kernel.  ``w_paired_tiled`` is ``tile_weight(pair_rows_for_rotation(w_qkv, D))``;
+    ``x`` may be ``NormedRows``, whose scaling the kernel then applies.
     Returns the rotated queries ``[rows, n_heads * head_dim]``."""
     lib = library.core_library()
+    normed = x if isinstance(x, NormedRows) else None
+    if normed is not None:
+        x = normed.x
     _dev(x, w_paired_tiled, positions, cos, sin, token_seg, block_table, k_pages, v_pages)
     _i32(positions, "positions"), _i32(token_seg, "token_seg"), _i32(block_table, "block_table")
     m, k = x.shape
@@ -256,7 +298,9 @@ def qkv_rope_append(
             _ptr(x), x.stride(0), _ptr(w_paired_tiled), _ptr(q), m, k, _ptr(positions), _ptr(token_seg),
             _ptr(block_table), block_table.shape[1], _ptr(cos), _ptr(sin), cos.shape[0],
             _ptr(k_pages), _ptr(v_pages), n_heads, n_kv_heads, head_dim, page_size, n_pages,
-            1 if tiled else 0, _stream(),
+            1 if tiled else 0, _ptr(normed.ss_parts) if normed else None,
+            normed.ss_parts.shape[0] if normed else 0, ctypes.c_float(normed.eps if normed else 0.0),
+            _stream(),
         ),
     )
     return q
@@ -431,10 +475,62 @@ def gemm_bf16_skinny(
     return out
 
 
+def norm_folds(m: int, k: int, tiled: torch.Tensor | None) -> bool:
+    """Whether a product of ``m`` rows over ``k`` columns against a weight with a tiled
+    copy can take an RMSNorm before or after it into itself."""
+    return tiled is not None and 0 < m <= SKINNY_ROWS and k % 8 == 0
+
+
+def gemm_bf16_skinny_norm(
+    x: torch.Tensor | NormedRows,
+    w_tiled: torch.Tensor,
+    tiled_shape: tuple[int, int],
+    w_up_tiled: torch.Tensor | None = None,
+    next_norm: NextNorm | None = None,
+):
+    """``x @ w.T`` for at most 16 rows against a tiled bf16 weight, with the RMSNorm
+    before it (``x`` is ``NormedRows``: the result is scaled per row; with ``w_up_tiled``
+    the gated form) or after it (``next_norm``: the result is added into the float32
+    stream ``next_norm.h`` and ``NormedRows`` for that norm come back) folded in."""
+    lib = library.core_library()
+    normed = x if isinstance(x, NormedRows) else None
+    if normed is not None:
+        x = normed.x
+    _dev(x, w_tiled, w_up_tiled)
+    m, k = x.shape
+    n, k2 = tiled_shape
+    _need(x.dtype == torch.bfloat16 and x.stride(1) == 1, "skinny gemm takes bf16 rows")
+    _need(k == k2 and norm_folds(m, k, w_tiled), "skinny gemm with a folded norm: at most 16 rows, K in steps of 8")
+    _need((normed is None) != (next_norm is None), "skinny gemm with a folded norm: the norm before or the one after")
+    need = (-(-n // 16) * 16) * (-(-k // 32) * 32)
+    for t in (w_tiled, w_up_tiled):
+        if t is not None:
+            _need(t.is_cuda and t.dtype == torch.bfloat16 and t.numel() == need and t.is_contiguous(), "skinny gemm: tiled weight")
+    if next_norm is not None:
+        h, nw = next_norm.h, next_norm.weight
+        _need(w_up_tiled is None, "skinny gemm: the gated form cannot add into the stream")
+        _need(h.dtype == torch.float32 and h.shape == (m, n) and h.is_contiguous(), "skinny gemm: residual stream")
+        _need(nw.numel() == n and nw.dtype in (torch.float32, torch.bfloat16), "skinny gemm: norm weight")
+        xw = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+        parts = torch.empty((-(-n // 16), 16), dtype=torch.float32, device=x.device)
+        _check(lib, lib.hal_gemm_bf16_skinny_norm(
+            _ptr(x), x.stride(0), _ptr(w_tiled), None, 0, _ptr(h), n, m, n, k, None, 0, ctypes.c_float(0.0),
+            _ptr(nw), dtype_code(nw.dtype), _ptr(xw), _ptr(parts), _stream()))
+        return NormedRows(xw, parts, next_norm.eps, nw)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    _check(lib, lib.hal_gemm_bf16_skinny_norm(
+        _ptr(x), x.stride(0), _ptr(w_tiled), _ptr(w_up_tiled), 0, _ptr(out), n, m, n, k,
+        _ptr(normed.ss_parts), normed.ss_parts.shape[0], ctypes.c_float(normed.eps),
+        None, 0, None, None, _stream()))
+    return out
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None,
-           tiled: torch.Tensor | None = None) -> torch.Tensor:
+           tiled: torch.Tensor | None = None, next_norm: NextNorm | None = None):
     """``x @ w.T`` for a weight ``[out, in]``; ``tiled`` is ``tile_weight(w)`` if the
-    model keeps that copy for small batches.
+    model keeps that copy for small batches.  ``x`` may be ``NormedRows``; with
+    ``next_norm`` the result may come back as ``NormedRows`` (already added into the
+    stream) instead of a tensor.
 
     float32 weights: the true 32-bit kernel (activations are widened if needed).
     bf16 weights: the hand-written kernel where it is the faster one (``skinny_pays``:
@@ -443,6 +539,17 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
     float32 output is asked for and the library cannot give it, which the hand-written
     kernel does in passes of 64 rows.
     """
+    if isinstance(x, NormedRows) or next_norm is not None:
+        # ``next_norm``: where the product can, it adds its result into the stream itself
+        # and returns ``NormedRows`` for that norm instead of the result
+        m, k = x.shape
+        if (w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and norm_folds(m, k, tiled)
+                and out_dtype in (None, torch.bfloat16)):
+            if isinstance(x, NormedRows):
+                return gemm_bf16_skinny_norm(x, tiled, tuple(w.shape))
+            return gemm_bf16_skinny_norm(x, tiled, tuple(w.shape), next_norm=next_norm)
+        if isinstance(x, NormedRows):
+            x = x.materialize()
     out_dtype = out_dtype or x.dtype
     if w.dtype == torch.float32:
         y = gemm_f32(x if x.dtype == torch.float32 else x.float(), w)

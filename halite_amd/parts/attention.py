@@ -36,6 +36,8 @@ class Attention(Mixer):
     """
 
     Params = AttentionParams
+    takes_normed_rows = True
+    folds_next_norm = True
 
     def __init__(self, params, build):
         super().__init__(params, build)
@@ -97,7 +99,7 @@ class Attention(Mixer):
         if attention_kernels.mfma_supported(self.build.dtype, self.p.head_dim, group.page_size):
             ctx.plan_attention(group.group_id, self.p.n_heads, self.p.n_kv_heads, self.p.window or 0, self.p.head_dim)
 
-    def forward(self, x, ctx, run):
+    def forward(self, x, ctx, run, then=None):
         p = self.p
         kv = run.kv
         group = ctx.group(kv.group_id)
@@ -110,7 +112,9 @@ class Attention(Mixer):
                 ctx.token_seg, group.block_table, kv.k, kv.v, group.page_size, kv.tiled,
             )
             out = ctx.attention(q, q.shape[1], kv, group, p.n_heads, p.scale, p.window or 0)
-            return ops.linear(out, self.w_out, tiled=self.t_out)
+            return ops.linear(out, self.w_out, tiled=self.t_out, next_norm=then)
+        if isinstance(x, ops.NormedRows):
+            x = x.materialize()
         if run.appends:
             qkv = ops.linear(x, self.w_qkv, tiled=self.t_qkv)
             n_kv_append = p.n_kv_heads
@@ -129,4 +133,4 @@ class Attention(Mixer):
             k_pages=kv.k, v_pages=kv.v, page_size=group.page_size, tiled=kv.tiled,
         )
         out = ctx.attention(qkv, qkv.shape[1], kv, group, p.n_heads, p.scale, p.window or 0)
-        return ops.linear(out, self.w_out, tiled=self.t_out)
+        return ops.linear(out, self.w_out, tiled=self.t_out, next_norm=then)

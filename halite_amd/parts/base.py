@@ -111,7 +111,17 @@ class Part:
 
 
 class Mixer(Part):
-    """Mixes information between the tokens of a request (attention here)."""
+    """Mixes information between the tokens of a request (attention here).
+
+    Two optional abilities, which a block uses only where both neighbours have them (so a
+    part without them never sees either): ``takes_normed_rows``, ``forward`` accepts
+    ``kernels.ops.NormedRows`` for ``x`` (rows whose norm the part's first product
+    finishes); ``folds_next_norm``, ``forward`` takes ``then=ops.NextNorm`` and may
+    return ``NormedRows`` for that norm, with its result already added into the stream,
+    instead of the result."""
+
+    takes_normed_rows: ClassVar[bool] = False
+    folds_next_norm: ClassVar[bool] = False
 
     def prepare(self, ctx: "StepContext", run: RunBinding) -> None:
         """Called for every run before the step's arrays go to the device; a mixer
@@ -122,6 +132,10 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    # as for Mixer
+    takes_normed_rows: ClassVar[bool] = False
+    folds_next_norm: ClassVar[bool] = False
+
     def forward(self, x: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
         raise NotImplementedError
 
@@ -135,8 +149,14 @@ class Norm(Part):
     ) -> torch.Tensor:
         """Normalises the float32 stream ``h`` after adding ``delta`` to it (the sum
         is written back to ``h``); with ``rows`` only those rows, and ``h`` is left
-        as it is."""
+        as it is.  ``delta`` may be what a product left for this norm
+        (``kernels.ops.NormedRows``, see ``foldable``), which is handed on as it is."""
         raise NotImplementedError
+
+    def foldable(self, h: torch.Tensor):
+        """``kernels.ops.NextNorm`` if the product before this norm may add into ``h`` and
+        prepare the norm's input itself, else None."""
+        return None
 
 
 class PositionEncoding(Part):

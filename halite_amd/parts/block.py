@@ -25,8 +25,19 @@ class PreNormBlock:
             "ff": self.ff,
         }
 
-    def forward(self, h, pending, ctx, run):
+    # The norm between two parts can be folded into the products around it where the part
+    # before it offers that and the part after it takes such rows.
+    def first_norm_for(self, h):
+        """For the block that runs before this one: what its last product may prepare."""
+        return self.mixer_norm.foldable(h) if self.mixer.takes_normed_rows else None
+
+    def forward(self, h, pending, ctx, run, next_norm=None):
         x = self.mixer_norm.forward(h, delta=pending)
-        a = self.mixer.forward(x, ctx, run)
+        then = None
+        if self.mixer.folds_next_norm and self.ff.takes_normed_rows:
+            then = self.ff_norm.foldable(h)
+        a = self.mixer.forward(x, ctx, run, then=then) if then is not None else self.mixer.forward(x, ctx, run)
         x = self.ff_norm.forward(h, delta=a)
+        if next_norm is not None and self.ff.folds_next_norm:
+            return self.ff.forward(x, ctx, then=next_norm)
         return self.ff.forward(x, ctx)

@@ -113,9 +113,15 @@ class Decoder:
         the step's tokens are in the cache afterwards."""
         h = self.embedding.forward(ctx.tokens)
         pending = None
-        for run in self.runs:
-            block = self.layers[self.spec.order[run.index].layer]
-            pending = block.forward(h, pending, ctx, run)
+        blocks = [self.layers[self.spec.order[run.index].layer] for run in self.runs]
+        for i, run in enumerate(self.runs):
+            # what the next block's first norm lets this block's last product do for it
+            ahead = blocks[i + 1] if i + 1 < len(blocks) else None
+            next_norm = ahead.first_norm_for(h) if hasattr(ahead, "first_norm_for") else None
+            if next_norm is not None:
+                pending = blocks[i].forward(h, pending, ctx, run, next_norm=next_norm)
+            else:
+                pending = blocks[i].forward(h, pending, ctx, run)
         if ctx.n_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         x = self.final_norm.forward(h, delta=pending, rows=ctx.logit_rows)

@@ -30,6 +30,8 @@ class GatedFeedForward(FeedForward):
     the multiply are float32 on the accumulators or on the product's output."""
 
     Params = GatedParams
+    takes_normed_rows = True
+    folds_next_norm = True
 
     def param_decls(self):
         f, d = self.p.intermediate_size, self.p.hidden_size
@@ -62,12 +64,17 @@ class GatedFeedForward(FeedForward):
             if self.w_out.dtype == torch.bfloat16:
                 self.t_out = ops.tile_weight(self.w_out)
 
-    def forward(self, x, ctx):
+    def forward(self, x, ctx, then=None):
         f = self.p.intermediate_size
         w = self.w_gate_up
+        if isinstance(x, ops.NormedRows):
+            if ops.norm_folds(x.shape[0], x.shape[1], self.t_gate):
+                act = ops.gemm_bf16_skinny_norm(x, self.t_gate, (f, x.shape[1]), w_up_tiled=self.t_up)
+                return ops.linear(act, self.w_out, tiled=self.t_out, next_norm=then)
+            x = x.materialize()
         if self.t_gate is not None and x.dtype == torch.bfloat16 and x.shape[0] <= ops.SKINNY_ROWS and x.shape[1] % 8 == 0:
             act = ops.gemm_bf16_skinny(x, self.t_gate, w_up=self.t_up, tiled_shape=(f, x.shape[1]))
-            return ops.linear(act, self.w_out, tiled=self.t_out)
+            return ops.linear(act, self.w_out, tiled=self.t_out, next_norm=then)
         fused = (
             w.dtype == torch.bfloat16
             and x.dtype == torch.bfloat16
@@ -79,4 +86,4 @@ class GatedFeedForward(FeedForward):
             act = ops.gemm_bf16_skinny(x, w[:f], w_up=w[f:])
         else:
             act = ops.silu_mul(ops.linear(x, w))
-        return ops.linear(act, self.w_out, tiled=self.t_out)
+        return ops.linear(act, self.w_out, tiled=self.t_out, next_norm=then)

@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+import torch
 from pydantic import BaseModel, Field, StrictInt
 
 from ..kernels import ops
@@ -26,4 +27,14 @@ class RMSNorm(Norm):
         return {"weight": ParamDecl((self.p.size,), init="ones")}
 
     def forward(self, h, delta=None, rows=None):
+        if isinstance(delta, ops.NormedRows):
+            # the product before has added its result into h and prepared these rows
+            if delta.weight is not self.weight or rows is not None:
+                raise ValueError("rows were prepared for another norm")
+            return delta
         return ops.rmsnorm(h, self.weight, self.p.eps, self.build.dtype, delta=delta, rows=rows)
+
+    def foldable(self, h):
+        if self.build.dtype != torch.bfloat16 or not h.is_cuda:
+            return None
+        return ops.NextNorm(h, self.weight, self.p.eps)

@@ -237,6 +237,58 @@ def test_qkv_rope_append_in_one_kernel(gpu, M, H, K, D, width, page, tiled):
     assert float(kp.float().abs().sum()) > 0
 
 
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("d,F,wdt", [(64, 96, "float32"), (120, 352, "bfloat16"), (4096, 1024, "bfloat16"), (1000, 200, "bfloat16")])
+def test_norm_folded_into_the_products_around_it(gpu, M, d, F, wdt):
+    """product -> add into the stream -> RMSNorm -> product (plain and gated), with the norm
+    done by the two products, against the same chain with the norm's own kernel and
+    against plain arithmetic."""
+    dt = torch.bfloat16
+    eps = 1e-5
+    a = rnd(M, F, seed=1).to(dt).to(gpu)                      # what the first product reads
+    w1 = (rnd(d, F, seed=2) * 0.3).to(dt).to(gpu)             # into the stream
+    w2 = (rnd(F, d, seed=3) * 0.3).to(dt).to(gpu)             # out of the norm (gate)
+    w3 = (rnd(F, d, seed=4) * 0.3).to(dt).to(gpu)             # out of the norm (up)
+    nw = (1.0 + 0.5 * rnd(d, seed=5)).to(DT[wdt]).to(gpu)
+    h0 = (rnd(M, d, seed=6) * 3.0).to(gpu)
+    h0[0, 3] = 40.0  # one large element: a row's scale must come from the whole row
+    t1, t2, t3 = ops.tile_weight(w1), ops.tile_weight(w2), ops.tile_weight(w3)
+
+    # the norm's own kernel between the products
+    h_ref = h0.clone()
+    delta = ops.gemm_bf16_skinny(a, t1, tiled_shape=(d, F))
+    y = ops.rmsnorm(h_ref, nw, eps, dt, delta=delta)
+    plain_out = ops.gemm_bf16_skinny(y, t2, tiled_shape=(F, d))
+    gated_out = ops.gemm_bf16_skinny(y, t2, w_up=t3, tiled_shape=(F, d))
+
+    # folded
+    h = h0.clone()
+    rows = ops.gemm_bf16_skinny_norm(a, t1, (d, F), next_norm=ops.NextNorm(h, nw, eps))
+    assert isinstance(rows, ops.NormedRows) and rows.ss_parts.shape == (-(-d // 16), 16)
+    assert torch.equal(h, h_ref)  # the same sums, rounded at the same place, added to the same stream
+    close(rows.ss_parts.sum(0)[:M], (h_ref.double() ** 2).sum(1), 1e-5, "sums of squares")
+    assert float(rows.ss_parts[:, M:].abs().sum()) == 0
+    close(rows.materialize(), y, 1.2e-2, "rows made whole")
+    got_plain = ops.gemm_bf16_skinny_norm(rows, t2, (F, d))
+    got_gated = ops.gemm_bf16_skinny_norm(rows, t2, (F, d), w_up_tiled=t3)
+    close(got_plain, plain_out, 1.5e-2, "plain product after the folded norm")
+    close(got_gated, gated_out, 2e-2, "gated product after the folded norm")
+
+    # plain arithmetic in float64 from the same stream
+    hd = h_ref.double().cpu()
+    n64 = hd * torch.rsqrt((hd ** 2).mean(1, keepdim=True) + eps) * nw.double().cpu()
+    close(got_plain, n64 @ w2.double().cpu().T, 1.5e-2, "against float64")
+    g, u = n64 @ w2.double().cpu().T, n64 @ w3.double().cpu().T
+    close(got_gated, u * g * torch.sigmoid(g), 2e-2, "gated against float64")
+    # through linear(): the same two calls, and a reader without a tiled copy gets whole rows
+    h = h0.clone()
+    rows2 = ops.linear(a, w1, tiled=t1, next_norm=ops.NextNorm(h, nw, eps))
+    assert torch.equal(rows2.x, rows.x) and torch.equal(h, h_ref)
+    assert torch.equal(ops.linear(rows2, w2, tiled=t2), got_plain)
+    close(ops.linear(rows2, w2), plain_out, 1.5e-2, "materialised rows")
+    assert isinstance(ops.linear(a, w1, next_norm=ops.NextNorm(h0.clone(), nw, eps)), torch.Tensor)
+
+
 def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use, tiled=False):
     """``segs``: list of (cached before, new tokens).  Builds one dense sequence per
     segment, pages it, and compares the rows of the new tokens with plain attention
