@@ -91,6 +91,41 @@ def test_bfloat16_run_of_a_folder_stored_in_float32(folders):
     replay.compare(rows, ref, TOL["bfloat16"])
 
 
+def test_steps_of_few_tokens_take_the_fused_kernels(folders, monkeypatch):
+    """With the tiled weight copy a bf16 step of at most 16 tokens runs rotation and append
+    inside the q, k, v product and every norm but the first and the last inside the
+    products around it; a larger step and the 32-bit path use the kernels of their own.
+    (Their results are compared with the plain implementation by the schedules above.)"""
+    from halite_amd.engine.batch import Segment
+    from halite_amd.kernels import ops
+
+    calls = {}
+    for name in ("rmsnorm", "rope_append", "qkv_rope_append", "gemm_bf16_skinny_norm"):
+        def counted(*a, _f=getattr(ops, name), _n=name, **kw):
+            calls[_n] = calls.get(_n, 0) + 1
+            return _f(*a, **kw)
+        monkeypatch.setattr(ops, name, counted)
+    folder, requests, _ = folders[("B", "bfloat16")]
+    layers = tiny.TINY_B["num_hidden_layers"]
+    toks = requests["r1"]
+    runner = make_runner(folder, "bfloat16", 128)
+    slot = runner.admit()
+    runner.step([Segment(slot, 0, toks[:20], [19])])
+    assert calls == {"rmsnorm": 2 * layers + 1, "rope_append": layers}
+    calls.clear()
+    runner.step([Segment(slot, 20, toks[20:23], [2])])
+    # per layer: o-proj (prepares the next norm), gate/up (scaled), down (prepares) = 3,
+    # less the last down-projection, whose norm is the model's final one over wanted rows
+    assert calls == {"rmsnorm": 2, "qkv_rope_append": layers, "gemm_bf16_skinny_norm": 3 * layers - 1}
+    runner.free(slot)
+    calls.clear()
+    folder32, _, _ = folders[("B", "float32")]
+    runner = make_runner(folder32, "float32", 128)
+    slot = runner.admit()
+    runner.step([Segment(slot, 0, toks[:3], [2])])
+    assert calls == {"rmsnorm": 2 * layers + 1, "rope_append": layers}
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_cuts_agree_with_each_other(folders, dtype):
     """The logits at a position do not depend on how the tokens were cut, beyond
