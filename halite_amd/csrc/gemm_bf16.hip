@@ -73,7 +73,7 @@ struct NormFusion {
   float* ss_out;
 };
 enum { SK_ROPE = 1, SK_SCALED = 2, SK_PREP = 4 };
-#define SK_MAX_PART_LOADS 4  // float4 loads of partial sums per thread, at most
+#define SK_MAX_PART_LOADS 4  // float4 loads of partial sums per thread that are asked for ahead
 
 // PL: float4 loads of partial sums per thread (SCALED), held in registers through the loop
 template <int NT, int MT, bool GATED, int U, int FLAGS = 0, int PL = 1>
@@ -84,9 +84,11 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
                                    NormFusion nf = NormFusion{}) {
   constexpr bool ROPE = (FLAGS & SK_ROPE) != 0, SCALED = (FLAGS & SK_SCALED) != 0,
                  PREP = (FLAGS & SK_PREP) != 0;
-  static_assert(!(SCALED || PREP) || MT == 1, "the folded norm serves at most 16 rows");
+  static_assert(!(SCALED || PREP || ROPE) || (MT <= 2 && NT <= 2),
+                "the extra epilogues serve at most 32 rows");
   static_assert(!PREP || (NT == 1 && !GATED && !ROPE && !SCALED), "PREP takes one plain tile");
-  __shared__ float row_sums[16][16];  // SCALED: [wave][row]; PREP: [column of the tile][row]
+  constexpr int RW = 16 * MT;  // rows of X a workgroup holds, and floats per part of the sums
+  __shared__ float row_sums[16][RW];  // SCALED: [wave][row]; PREP: [column of the tile][row]
   extern __shared__ float red[];  // [waves][sets][NT*MT][64][4]
   const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
   const int n_waves = blockDim.x / HAL_WAVE;
@@ -100,13 +102,13 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   const int s_end = s_begin + per_wave < steps ? s_begin + per_wave : steps;
 
   // SCALED: this thread's share of the partial sums is asked for before anything else, so
-  // that it has arrived long before the epilogue; float4 f holds rows 4 (f % 4) .. + 3 of
-  // part f / 4, and f % 4 == lane % 4 for every f of a thread
+  // that it has arrived long before the epilogue; with QW = RW / 4, float4 f holds rows
+  // 4 (f % QW) .. + 3 of part f / QW, and f % QW == lane % QW for every f of a thread
   // (a load past the end is clamped here and dropped where the sums are added)
   float4 my_parts[PL];
   if constexpr (SCALED) {
     const float4* pp = (const float4*)nf.ss_in;
-    const int last = nf.n_parts * 4 - 1;
+    const int last = nf.n_parts * (RW / 4) - 1;
 #pragma unroll
     for (int k = 0; k < PL; ++k) {
       const int f = tid + k * (int)blockDim.x;
@@ -227,15 +229,20 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
     float4 sum = float4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int k = 0; k < PL; ++k) {
-      if (tid + k * (int)blockDim.x < nf.n_parts * 4)
+      if (tid + k * (int)blockDim.x < nf.n_parts * (RW / 4))
         sum.x += my_parts[k].x, sum.y += my_parts[k].y, sum.z += my_parts[k].z, sum.w += my_parts[k].w;
     }
+    // more parts than the loads ahead cover (a very wide model): the rest is read here
+    for (int f = tid + PL * (int)blockDim.x; f < nf.n_parts * (RW / 4); f += blockDim.x) {
+      const float4 more = ((const float4*)nf.ss_in)[f];
+      sum.x += more.x, sum.y += more.y, sum.z += more.z, sum.w += more.w;
+    }
 #pragma unroll
-    for (int off = 4; off < HAL_WAVE; off <<= 1) {
+    for (int off = RW / 4; off < HAL_WAVE; off <<= 1) {
       sum.x += __shfl_xor(sum.x, off, HAL_WAVE), sum.y += __shfl_xor(sum.y, off, HAL_WAVE);
       sum.z += __shfl_xor(sum.z, off, HAL_WAVE), sum.w += __shfl_xor(sum.w, off, HAL_WAVE);
     }
-    if (lane < 4) *(float4*)&row_sums[wave][lane * 4] = sum;
+    if (lane < RW / 4) *(float4*)&row_sums[wave][lane * 4] = sum;
   }
   __syncthreads();
   // rsqrt(mean(h^2) + eps) of row m, as the norm's own kernel computes it
@@ -246,13 +253,14 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   };
 
   if constexpr (ROPE) {
-    static_assert(NT == 1 && MT == 1 && !GATED, "the rotating epilogue takes one tile");
-    // pair p: elements c and c + 8 of the tile, for token m; C is q alone, [M, H * D]
+    static_assert(!GATED, "the rotating epilogue is not the gated one");
+    // pair p: elements c and c + 8 of tile f, for token m; C is q alone, [M, H * D]
     const int D = rope.D, half = D / 2, tiles_per_head = D / 16;
-    for (int p = tid; p < 128; p += blockDim.x) {
-      const int c = p / 16, m = p % 16;
-      if (m >= M) continue;
-      const int idx0 = ((c / 4) * 16 + m) * 4 + c % 4, idx1 = idx0 + 128;
+    for (int p = tid; p < NT * MT * 128; p += blockDim.x) {
+      const int f = p / (MT * 128), t = (p / 128) % MT, c = (p % 128) / 16, m = t * 16 + p % 16;
+      const int tile = blockIdx.x * NT + f;
+      if (m >= M || tile * 16 >= N) continue;
+      const int idx0 = (f * MT + t) * 256 + ((c / 4) * 16 + p % 16) * 4 + c % 4, idx1 = idx0 + 128;
       float v0 = 0.f, v1 = 0.f;
       for (int w = 0; w < slots; ++w) {
         v0 += red[(size_t)w * TILE + idx0];
@@ -264,7 +272,7 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
       }
       // the product is rounded to bf16 before the rotation, as the unfused way stores it
       const float x0 = bf16_to_f32(f32_to_bf16(v0)), x1 = bf16_to_f32(f32_to_bf16(v1));
-      const int head = blockIdx.x / tiles_per_head, d0 = (blockIdx.x % tiles_per_head) * 8 + c;
+      const int head = tile / tiles_per_head, d0 = (tile % tiles_per_head) * 8 + c;
       const int d1 = d0 + half;
       const int pos = rope.positions[m];
       if (pos < 0 || pos >= rope.table_len) continue;  // checked on the host
@@ -300,9 +308,9 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   if constexpr (PREP) {
     // thread (column c of the tile, row m): h += product (rounded to bf16 first, as the
     // unfused way hands it on), the next norm's input, and h^2 for the row's sum
-    if (tid < 256) {
-      const int c = tid / 16, m = tid % 16, n = n_base + c;
-      const int idx = ((c / 4) * 16 + m) * 4 + c % 4;
+    for (int e = tid; e < MT * 256; e += blockDim.x) {
+      const int t = e / 256, c = (e % 256) / 16, m = t * 16 + e % 16, n = n_base + c;
+      const int idx = t * 256 + ((c / 4) * 16 + e % 16) * 4 + c % 4;
       float sq = 0.f;
       if (n < N && m < M) {
         float v = 0.f;
@@ -317,11 +325,11 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
       row_sums[c][m] = sq;
     }
     __syncthreads();
-    if (tid < 16) {
+    if (tid < RW) {
       float total = 0.f;
 #pragma unroll
       for (int c = 0; c < 16; ++c) total += row_sums[c][tid];
-      nf.ss_out[(size_t)blockIdx.x * 16 + tid] = total;
+      nf.ss_out[(size_t)blockIdx.x * RW + tid] = total;
     }
     return;
   }
@@ -365,14 +373,13 @@ static int launch_skinny(const bf16_t* X, int ldx, const bf16_t* W, const bf16_t
   while (slots > 1 && (size_t)slots * per_wave > 64 * 1024) slots /= 2;
   const size_t smem = (size_t)slots * per_wave;
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
-  if constexpr ((FLAGS & SK_SCALED) != 0 && PL < SK_MAX_PART_LOADS) {
-    if (nf.n_parts * 4 > PL * waves * HAL_WAVE)  // more loads per thread
+  // (two row tiles: the accumulators need the registers, and what the loads ahead do not
+  // cover is read in the epilogue)
+  if constexpr ((FLAGS & SK_SCALED) != 0 && PL < (MT == 1 ? SK_MAX_PART_LOADS : 2)) {
+    if (nf.n_parts * 4 * MT > PL * waves * HAL_WAVE)  // more loads per thread
       return launch_skinny<NT, MT, GATED, U, FLAGS, PL * 2>(X, ldx, W, W2, ldw, C, ldc, out_mode, M,
                                                             N, K, waves, stream, rope, nf);
   }
-  if ((FLAGS & SK_SCALED) && nf.n_parts * 4 > PL * waves * HAL_WAVE)
-    return hal_fail("skinny gemm: %d partial sums per row are more than %d threads take",
-                    nf.n_parts, waves * HAL_WAVE);
   hipLaunchKernelGGL((skinny_gemm_kernel<NT, MT, GATED, U, FLAGS, PL>), dim3(blocks),
                      dim3(waves * HAL_WAVE), smem, stream, X, ldx, W, W2, ldw, C, ldc, out_mode,
                      M, N, K, slots, rope, nf);
@@ -457,19 +464,20 @@ extern "C" int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const
   return hal_fail("hal_gemm_bf16_skinny: no kernel for nt=%d mt=%d", nt, mt);
 }
 
-// The same product for at most 16 rows with the RMSNorm before or after it folded in.
+// The same product for at most 32 rows with the RMSNorm before or after it folded in.
+// The sums of h^2 come in parts of 16 floats (up to 16 rows) or 32 floats (17 to 32 rows).
 // ss_in (or null): X holds bf16(w * bf16(h)) of the norm before this product and ss_in
-// [n_parts, 16] the partial sums of h^2 that the product before left; the result is scaled
+// [n_parts, 16 or 32] the partial sums of h^2 that the product before left; the result is scaled
 // by rsqrt(sum / K + eps) per row.  norm_w (or null, not with W2): C is the float32 stream
 // h [M, N]; the result is added into it, xw_out [M, N] receives bf16(norm_w * bf16(h)) and
-// ss_out [ceil(N / 16), 16] this product's partial sums of h^2 for the product after.
+// ss_out [ceil(N / 16), 16 or 32] this product's partial sums of h^2 for the product after.
 // Without norm_w the result goes to C as bf16.
 extern "C" int hal_gemm_bf16_skinny_norm(const void* X, int ldx, const void* W, const void* W2,
                                          int ldw, void* C, int ldc, int M, int N, int K,
                                          const float* ss_in, int n_parts, float eps,
                                          const void* norm_w, int norm_w_dtype, void* xw_out,
                                          float* ss_out, hipStream_t stream) {
-  HAL_REQUIRE(M >= 0 && M <= 16, "hal_gemm_bf16_skinny_norm: M=%d (at most 16 rows)", M);
+  HAL_REQUIRE(M >= 0 && M <= 32, "hal_gemm_bf16_skinny_norm: M=%d (at most 32 rows)", M);
   HAL_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "hal_gemm_bf16_skinny_norm: N=%d K=%d", N, K);
   HAL_REQUIRE(ldx >= K && (ldw >= K || ldw == 0) && ldc >= N && ldx % 8 == 0 && ldw % 8 == 0,
               "hal_gemm_bf16_skinny_norm: leading dimensions %d %d %d", ldx, ldw, ldc);
@@ -488,17 +496,28 @@ extern "C" int hal_gemm_bf16_skinny_norm(const void* X, int ldx, const void* W, 
   const bf16_t* x = (const bf16_t*)X;
   const bf16_t* w = (const bf16_t*)W;
   const bf16_t* w2 = (const bf16_t*)W2;
+  // 17 to 32 rows: two row tiles per wave, half as many steps of K in flight
+#define SK_NORM_LAUNCH(MT_, GATED_, U_, FLAGS_, W2_, MODE_)                                        \
+  return launch_skinny<1, MT_, GATED_, U_, FLAGS_>(x, ldx, w, W2_, ldw, C, ldc, MODE_, M, N, K,    \
+                                                   waves, stream, RopeEpilogue{}, nf)
+  if (M <= 16) {
+    if (w2) SK_NORM_LAUNCH(1, true, 4, SK_SCALED, w2, SK_OUT_BF16);
+    if (norm_w) SK_NORM_LAUNCH(1, false, 8, SK_PREP, nullptr, SK_OUT_F32_ADD);
+    SK_NORM_LAUNCH(1, false, 8, SK_SCALED, nullptr, SK_OUT_BF16);
+  }
+  if (norm_w) SK_NORM_LAUNCH(2, false, 4, SK_PREP, nullptr, SK_OUT_F32_ADD);
+#undef SK_NORM_LAUNCH
+  // the products that read the normed rows take two tiles of W as well (fewer, larger
+  // workgroups read X less often), as hal_gemm_bf16_skinny does at these sizes
+  const int waves2 = skinny_waves((N + 31) / 32, steps);
   if (w2)
-    return launch_skinny<1, 1, true, 4, SK_SCALED>(x, ldx, w, w2, ldw, C, ldc, SK_OUT_BF16, M, N, K,
-                                                   waves, stream, RopeEpilogue{}, nf);
-  if (norm_w)
-    return launch_skinny<1, 1, false, 8, SK_PREP>(x, ldx, w, nullptr, ldw, C, ldc, SK_OUT_F32_ADD, M,
-                                                  N, K, waves, stream, RopeEpilogue{}, nf);
-  return launch_skinny<1, 1, false, 8, SK_SCALED>(x, ldx, w, nullptr, ldw, C, ldc, SK_OUT_BF16, M, N,
-                                                  K, waves, stream, RopeEpilogue{}, nf);
+    return launch_skinny<2, 2, true, 2, SK_SCALED>(x, ldx, w, w2, ldw, C, ldc, SK_OUT_BF16, M, N, K,
+                                                   waves2, stream, RopeEpilogue{}, nf);
+  return launch_skinny<2, 2, false, 4, SK_SCALED>(x, ldx, w, nullptr, ldw, C, ldc, SK_OUT_BF16, M, N,
+                                                  K, waves2, stream, RopeEpilogue{}, nf);
 }
 
-// The packed q, k, v projection of at most 16 tokens with rotation and append in its
+// The packed q, k, v projection of at most 32 tokens with rotation and append in its
 // epilogue.  W is the projection's weight with its rows reordered (see RopeEpilogue) and
 // then laid out in tiles as for hal_gemm_bf16_skinny with ldw == 0; q_out [M, H * D]
 // receives the rotated queries; rotated keys and the values go to the pages of each
@@ -510,7 +529,7 @@ extern "C" int hal_qkv_rope_append(const void* X, int ldx, const void* W, void* 
                                    void* v_pages, int H, int K, int D, int page_size, int n_pages,
                                    int tiled, const float* ss_in, int n_parts, float eps,
                                    hipStream_t stream) {
-  HAL_REQUIRE(M >= 0 && M <= 16, "hal_qkv_rope_append: M=%d (at most 16 tokens)", M);
+  HAL_REQUIRE(M >= 0 && M <= 32, "hal_qkv_rope_append: M=%d (at most 32 tokens)", M);
   HAL_REQUIRE(!ss_in || (n_parts > 0 && eps > 0.f && ((uintptr_t)ss_in % 16) == 0),
               "hal_qkv_rope_append: partial sums of the norm before");
   HAL_REQUIRE(H > 0 && K > 0 && D > 0 && D % 16 == 0, "hal_qkv_rope_append: heads %d, %d, size %d",
@@ -532,11 +551,21 @@ extern "C" int hal_qkv_rope_append(const void* X, int ldx, const void* W, void* 
   RopeEpilogue rope{positions, token_seg, block_table, bt_stride, cos_t, sin_t, table_len,
                     (bf16_t*)k_pages, (bf16_t*)v_pages, H, K, D, page_size, n_pages, tiled};
   NormFusion nf{ss_in, n_parts, eps, nullptr, 0, nullptr, nullptr};
+#define SK_ROPE_LAUNCH(MT_, U_, FLAGS_)                                                            \
+  return launch_skinny<1, MT_, false, U_, FLAGS_>((const bf16_t*)X, ldx, (const bf16_t*)W, nullptr, \
+                                                  0, q_out, H * D, SK_OUT_BF16, M, N, K_in, waves,  \
+                                                  stream, rope, nf)
+  if (M <= 16) {
+    if (ss_in) SK_ROPE_LAUNCH(1, 8, SK_ROPE | SK_SCALED);
+    SK_ROPE_LAUNCH(1, 8, SK_ROPE);
+  }
+#undef SK_ROPE_LAUNCH
+  const int waves2 = skinny_waves((N + 31) / 32, steps);
   if (ss_in)
-    return launch_skinny<1, 1, false, 8, SK_ROPE | SK_SCALED>(
+    return launch_skinny<2, 2, false, 4, SK_ROPE | SK_SCALED>(
         (const bf16_t*)X, ldx, (const bf16_t*)W, nullptr, 0, q_out, H * D, SK_OUT_BF16, M, N, K_in,
-        waves, stream, rope, nf);
-  return launch_skinny<1, 1, false, 8, SK_ROPE>((const bf16_t*)X, ldx, (const bf16_t*)W, nullptr, 0,
-                                                q_out, H * D, SK_OUT_BF16, M, N, K_in, waves,
+        waves2, stream, rope, nf);
+  return launch_skinny<2, 2, false, 4, SK_ROPE>((const bf16_t*)X, ldx, (const bf16_t*)W, nullptr, 0,
+                                                q_out, H * D, SK_OUT_BF16, M, N, K_in, waves2,
                                                 stream, rope, nf);
 }

@@ -44,7 +44,7 @@ int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, float* C, int
 int hal_gemm_bf16_skinny(const void* X, int ldx, const void* W, const void* W2, int ldw, void* C,
                          int ldc, int out_mode, int M, int N, int K, hipStream_t stream);
 
-// The packed q, k, v projection of M <= 16 tokens with the rotation of q and k (pairs
+// The packed q, k, v projection of M <= 32 tokens with the rotation of q and k (pairs
 // (j, j + D/2), whole head) and the append of k and v to the pages in its epilogue.  W:
 // the weight's rows reordered per head to [8j .. 8j+7, D/2 + 8j .. D/2 + 8j+7] for
 // j = 0 .. D/16 - 1, then tiled as for ldw == 0 above.  q_out [M, H * D] bf16.  ss_in (or
@@ -56,8 +56,8 @@ int hal_qkv_rope_append(const void* X, int ldx, const void* W, void* q_out, int 
                         int n_pages, int tiled, const float* ss_in, int n_parts, float eps,
                         hipStream_t stream);
 
-// The product for M <= 16 rows with the RMSNorm before it (ss_in: partial sums of squares
-// [n_parts, 16] left by the product before; X holds bf16(w * bf16(h))) or after it
+// The product for M <= 32 rows with the RMSNorm before it (ss_in: partial sums of squares
+// [n_parts, 16] (32 for more than 16 rows) left by the product before; X holds bf16(w * bf16(h))) or after it
 // (norm_w: C is the float32 stream h, added into; xw_out [M, N] and ss_out [ceil(N/16), 16]
 // are left for the product after) folded in.
 int hal_gemm_bf16_skinny_norm(const void* X, int ldx, const void* W, const void* W2, int ldw,

@@ -35,9 +35,9 @@ class NextNorm:
 
 @dataclass
 class NormedRows:
-    """At most 16 rows on their way through an RMSNorm whose scaling is left to the product
+    """At most 32 rows on their way through an RMSNorm whose scaling is left to the product
     that reads them: ``x`` [rows, d] is ``bf16(weight * bf16(h))`` and ``ss_parts``
-    [parts, 16] holds partial sums of ``h^2`` per row, so the norm's output is
+    [parts, 16 or 32] holds partial sums of ``h^2`` per row, so the norm's output is
     ``x * rsqrt(ss_parts.sum(0) / d + eps)`` row by row."""
 
     x: torch.Tensor
@@ -276,7 +276,9 @@ def qkv_rope_append(
     _i32(positions, "positions"), _i32(token_seg, "token_seg"), _i32(block_table, "block_table")
     m, k = x.shape
     n = (n_heads + 2 * n_kv_heads) * head_dim
-    _need(x.dtype == torch.bfloat16 and x.stride(1) == 1 and m <= SKINNY_ROWS, "qkv_rope_append: up to 16 bf16 rows")
+    _need(x.dtype == torch.bfloat16 and x.stride(1) == 1 and m <= FUSED_ROWS, "qkv_rope_append: up to 32 bf16 rows")
+    _need(normed is None or (normed.ss_parts.shape[1] == 16 * -(-m // 16) and normed.ss_parts.is_contiguous()),
+          "qkv_rope_append: sums of squares")
     _need(head_dim % 16 == 0 and k % 8 == 0, "qkv_rope_append: head size in steps of 16, width in steps of 8")
     _need(
         w_paired_tiled.dtype == torch.bfloat16 and w_paired_tiled.is_contiguous()
@@ -399,6 +401,8 @@ def sample(
 
 SKINNY_MAX_ROWS = 64  # what the kernel takes
 SKINNY_ROWS = 16  # up to here it beats the library product
+FUSED_ROWS = 32  # what the epilogues that take other kernels' work take
+FUSED_MID_ELEMENTS = 32 * 1024 * 1024  # the largest matrix on which they pay at 17 to 32 rows
 # ... if the weights lie in its tiled order.  On row-major weights (a model too large for
 # the second copy) it wins only on small matrices or a single row: measured on Llama-3.1-70B
 # shapes at 8 and 16 rows, the library reads 4.7-5.5 TB/s where the kernel reads 3.2-4.6.
@@ -475,10 +479,14 @@ def gemm_bf16_skinny(
     return out
 
 
-def norm_folds(m: int, k: int, tiled: torch.Tensor | None) -> bool:
-    """Whether a product of ``m`` rows over ``k`` columns against a weight with a tiled
-    copy can take an RMSNorm before or after it into itself."""
-    return tiled is not None and 0 < m <= SKINNY_ROWS and k % 8 == 0
+def norm_folds(m: int, n: int, k: int, tiled: torch.Tensor | None) -> bool:
+    """Whether a product of ``m`` rows against an ``[n, k]`` weight with a tiled copy
+    takes an RMSNorm before or after it, or the rotation and the append, into itself: up
+    to 16 rows always, 17 to 32 rows on matrices that the small-batch kernel still reads
+    as fast as the library product does."""
+    if tiled is None or m <= 0 or k % 8:
+        return False
+    return m <= SKINNY_ROWS or (m <= FUSED_ROWS and n * k <= FUSED_MID_ELEMENTS)
 
 
 def gemm_bf16_skinny_norm(
@@ -500,7 +508,8 @@ def gemm_bf16_skinny_norm(
     m, k = x.shape
     n, k2 = tiled_shape
     _need(x.dtype == torch.bfloat16 and x.stride(1) == 1, "skinny gemm takes bf16 rows")
-    _need(k == k2 and norm_folds(m, k, w_tiled), "skinny gemm with a folded norm: at most 16 rows, K in steps of 8")
+    _need(k == k2 and 0 < m <= FUSED_ROWS and k % 8 == 0, "skinny gemm with a folded norm: at most 32 rows, K in steps of 8")
+    row_width = 16 * -(-m // 16)
     _need((normed is None) != (next_norm is None), "skinny gemm with a folded norm: the norm before or the one after")
     need = (-(-n // 16) * 16) * (-(-k // 32) * 32)
     for t in (w_tiled, w_up_tiled):
@@ -512,11 +521,12 @@ def gemm_bf16_skinny_norm(
         _need(h.dtype == torch.float32 and h.shape == (m, n) and h.is_contiguous(), "skinny gemm: residual stream")
         _need(nw.numel() == n and nw.dtype in (torch.float32, torch.bfloat16), "skinny gemm: norm weight")
         xw = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-        parts = torch.empty((-(-n // 16), 16), dtype=torch.float32, device=x.device)
+        parts = torch.empty((-(-n // 16), row_width), dtype=torch.float32, device=x.device)
         _check(lib, lib.hal_gemm_bf16_skinny_norm(
             _ptr(x), x.stride(0), _ptr(w_tiled), None, 0, _ptr(h), n, m, n, k, None, 0, ctypes.c_float(0.0),
             _ptr(nw), dtype_code(nw.dtype), _ptr(xw), _ptr(parts), _stream()))
         return NormedRows(xw, parts, next_norm.eps, nw)
+    _need(normed.ss_parts.shape[1] == row_width and normed.ss_parts.is_contiguous(), "skinny gemm: sums of squares")
     out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     _check(lib, lib.hal_gemm_bf16_skinny_norm(
         _ptr(x), x.stride(0), _ptr(w_tiled), _ptr(w_up_tiled), 0, _ptr(out), n, m, n, k,
@@ -543,7 +553,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
         # ``next_norm``: where the product can, it adds its result into the stream itself
         # and returns ``NormedRows`` for that norm instead of the result
         m, k = x.shape
-        if (w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and norm_folds(m, k, tiled)
+        if (w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and norm_folds(m, w.shape[0], k, tiled)
                 and out_dtype in (None, torch.bfloat16)):
             if isinstance(x, NormedRows):
                 return gemm_bf16_skinny_norm(x, tiled, tuple(w.shape))

@@ -104,8 +104,8 @@ class Attention(Mixer):
         kv = run.kv
         group = ctx.group(kv.group_id)
         n_q = p.n_heads * p.head_dim
-        if (run.appends and self.t_qkv_paired is not None and x.shape[0] <= ops.SKINNY_ROWS
-                and x.dtype == torch.bfloat16 and kv.k.dtype == torch.bfloat16):
+        if (run.appends and x.dtype == torch.bfloat16 and kv.k.dtype == torch.bfloat16
+                and ops.norm_folds(x.shape[0], self.w_qkv.shape[0], x.shape[1], self.t_qkv_paired)):
             cos, sin = self.position.tables(ctx.max_position + 1)
             q = ops.qkv_rope_append(
                 x, self.t_qkv_paired, ctx.positions, cos, sin, p.n_heads, p.n_kv_heads, p.head_dim,

@@ -67,18 +67,20 @@ class GatedFeedForward(FeedForward):
     def forward(self, x, ctx, then=None):
         f = self.p.intermediate_size
         w = self.w_gate_up
+        # The gated product with SiLU·mul in its epilogue beats the library product and a
+        # kernel for SiLU·mul up to 16 rows, and at 17 to 32 rows on matrices of up to 64 M
+        # elements (measured in captured graphs: 50 against 56 us at 14336 x 4096, 23 against
+        # 25 at 8192 x 3072, 202 against 179 at 28672 x 8192).
+        m, d = x.shape
+        small = (self.t_gate is not None and x.dtype == torch.bfloat16 and d % 8 == 0
+                 and (m <= ops.SKINNY_ROWS or (m <= ops.FUSED_ROWS and f * d <= 64 * 2**20)))
         if isinstance(x, ops.NormedRows):
-            if ops.norm_folds(x.shape[0], x.shape[1], self.t_gate):
-                act = ops.gemm_bf16_skinny_norm(x, self.t_gate, (f, x.shape[1]), w_up_tiled=self.t_up)
+            if small:
+                act = ops.gemm_bf16_skinny_norm(x, self.t_gate, (f, d), w_up_tiled=self.t_up)
                 return ops.linear(act, self.w_out, tiled=self.t_out, next_norm=then)
             x = x.materialize()
-        # the gated product with SiLU·mul in its epilogue also beats the library product and a
-        # kernel for SiLU·mul at 17 to 32 rows, on matrices of up to 64 M elements (measured in
-        # captured graphs: 50 against 56 us at 14336 x 4096, 23 against 25 at 8192 x 3072,
-        # 202 against 179 at 28672 x 8192)
-        rows_ok = x.shape[0] <= ops.SKINNY_ROWS or (x.shape[0] <= 32 and f * x.shape[1] <= 64 * 2**20)
-        if self.t_gate is not None and x.dtype == torch.bfloat16 and rows_ok and x.shape[1] % 8 == 0:
-            act = ops.gemm_bf16_skinny(x, self.t_gate, w_up=self.t_up, tiled_shape=(f, x.shape[1]))
+        if small:
+            act = ops.gemm_bf16_skinny(x, self.t_gate, w_up=self.t_up, tiled_shape=(f, d))
             return ops.linear(act, self.w_out, tiled=self.t_out, next_norm=then)
         fused = (
             w.dtype == torch.bfloat16

@@ -192,7 +192,7 @@ def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page, tiled):
     assert float(vpc.abs().sum(dim=(1, 2))[~written].sum()) == 0
 
 
-@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 32])
 @pytest.mark.parametrize("H,K,D,width,page,tiled", [
     (4, 2, 16, 64, 8, False), (6, 3, 48, 120, 16, False), (5, 1, 80, 200, 4, False),
     (8, 2, 64, 352, 32, True), (32, 8, 128, 4096, 64, True), (2, 2, 160, 96, 64, True),
@@ -229,7 +229,9 @@ def test_qkv_rope_append_in_one_kernel(gpu, M, H, K, D, width, page, tiled):
     # the same sums in the same order, rounded at the same places
     close(q, qkv[:, : H * D], 4e-3, "rotated q, fused against unfused")
     close(kp, kp2, 4e-3, "key pages")
-    assert torch.equal(vp, vp2)
+    if M <= 16:  # the same sums in the same order; beyond, the unfused product splits K otherwise
+        assert torch.equal(vp, vp2)
+    close(vp, vp2, 4e-3, "value pages")
     # and the rotation itself against the plain one, from the unrotated product
     c, s_ = cos.cpu()[positions.long()], sin.cpu()[positions.long()]
     want_q = P.rotate_half_split(plain_qkv[:, : H * D].view(M, H, D), c, s_)
@@ -237,7 +239,7 @@ def test_qkv_rope_append_in_one_kernel(gpu, M, H, K, D, width, page, tiled):
     assert float(kp.float().abs().sum()) > 0
 
 
-@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("M", [1, 7, 16, 19, 32])
 @pytest.mark.parametrize("d,F,wdt", [(64, 96, "float32"), (120, 352, "bfloat16"), (4096, 1024, "bfloat16"), (1000, 200, "bfloat16")])
 def test_norm_folded_into_the_products_around_it(gpu, M, d, F, wdt):
     """product -> add into the stream -> RMSNorm -> product (plain and gated), with the norm
@@ -264,8 +266,10 @@ def test_norm_folded_into_the_products_around_it(gpu, M, d, F, wdt):
     # folded
     h = h0.clone()
     rows = ops.gemm_bf16_skinny_norm(a, t1, (d, F), next_norm=ops.NextNorm(h, nw, eps))
-    assert isinstance(rows, ops.NormedRows) and rows.ss_parts.shape == (-(-d // 16), 16)
-    assert torch.equal(h, h_ref)  # the same sums, rounded at the same place, added to the same stream
+    assert isinstance(rows, ops.NormedRows) and rows.ss_parts.shape == (-(-d // 16), 16 * -(-M // 16))
+    if M <= 16:  # the same sums, rounded at the same place, added to the same stream
+        assert torch.equal(h, h_ref)
+    close(h, h_ref, 1e-3, "the stream")  # beyond 16 rows the unfused product splits K otherwise
     close(rows.ss_parts.sum(0)[:M], (h_ref.double() ** 2).sum(1), 1e-5, "sums of squares")
     assert float(rows.ss_parts[:, M:].abs().sum()) == 0
     close(rows.materialize(), y, 1.2e-2, "rows made whole")
@@ -283,7 +287,7 @@ def test_norm_folded_into_the_products_around_it(gpu, M, d, F, wdt):
     # through linear(): the same two calls, and a reader without a tiled copy gets whole rows
     h = h0.clone()
     rows2 = ops.linear(a, w1, tiled=t1, next_norm=ops.NextNorm(h, nw, eps))
-    assert torch.equal(rows2.x, rows.x) and torch.equal(h, h_ref)
+    assert torch.equal(rows2.x, rows.x) and float((h - h_ref).abs().max()) <= 1e-3 * float(h_ref.abs().max())
     assert torch.equal(ops.linear(rows2, w2, tiled=t2), got_plain)
     close(ops.linear(rows2, w2), plain_out, 1.5e-2, "materialised rows")
     assert isinstance(ops.linear(a, w1, next_norm=ops.NextNorm(h0.clone(), nw, eps)), torch.Tensor)

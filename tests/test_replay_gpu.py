@@ -92,7 +92,7 @@ def test_bfloat16_run_of_a_folder_stored_in_float32(folders):
 
 
 def test_steps_of_few_tokens_take_the_fused_kernels(folders, monkeypatch):
-    """With the tiled weight copy a bf16 step of at most 16 tokens runs rotation and append
+    """With the tiled weight copy a bf16 step of at most 32 tokens runs rotation and append
     inside the q, k, v product and every norm but the first and the last inside the
     products around it; a larger step and the 32-bit path use the kernels of their own.
     (Their results are compared with the plain implementation by the schedules above.)"""
@@ -107,16 +107,20 @@ def test_steps_of_few_tokens_take_the_fused_kernels(folders, monkeypatch):
         monkeypatch.setattr(ops, name, counted)
     folder, requests, _ = folders[("B", "bfloat16")]
     layers = tiny.TINY_B["num_hidden_layers"]
-    toks = requests["r1"]
+    toks = requests["r2"]
     runner = make_runner(folder, "bfloat16", 128)
     slot = runner.admit()
-    runner.step([Segment(slot, 0, toks[:20], [19])])
+    runner.step([Segment(slot, 0, toks[:40], [39])])
     assert calls == {"rmsnorm": 2 * layers + 1, "rope_append": layers}
-    calls.clear()
-    runner.step([Segment(slot, 20, toks[20:23], [2])])
     # per layer: o-proj (prepares the next norm), gate/up (scaled), down (prepares) = 3,
     # less the last down-projection, whose norm is the model's final one over wanted rows
-    assert calls == {"rmsnorm": 2, "qkv_rope_append": layers, "gemm_bf16_skinny_norm": 3 * layers - 1}
+    fused = {"rmsnorm": 2, "qkv_rope_append": layers, "gemm_bf16_skinny_norm": 3 * layers - 1}
+    calls.clear()
+    runner.step([Segment(slot, 40, toks[40:60], [19])])  # 17 to 32 tokens: two row tiles per wave
+    assert calls == fused
+    calls.clear()
+    runner.step([Segment(slot, 60, toks[60:63], [2])])
+    assert calls == fused
     runner.free(slot)
     calls.clear()
     folder32, _, _ = folders[("B", "float32")]
