@@ -14,6 +14,8 @@ class PreNormBlock:
     norm (or to the model's final norm) instead of adding it itself.
     """
 
+    takes_next_norm = True  # forward() accepts next_norm=
+
     def __init__(self, mixer_norm, mixer, ff_norm, ff):
         self.mixer_norm, self.mixer, self.ff_norm, self.ff = mixer_norm, mixer, ff_norm, ff
 

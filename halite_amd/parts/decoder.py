@@ -116,8 +116,12 @@ class Decoder:
         blocks = [self.layers[self.spec.order[run.index].layer] for run in self.runs]
         for i, run in enumerate(self.runs):
             # what the next block's first norm lets this block's last product do for it
+            # (both are optional abilities of an arrangement: `takes_next_norm` of the one that
+            # runs now, `first_norm_for` of the one that runs next)
             ahead = blocks[i + 1] if i + 1 < len(blocks) else None
-            next_norm = ahead.first_norm_for(h) if hasattr(ahead, "first_norm_for") else None
+            next_norm = None
+            if getattr(blocks[i], "takes_next_norm", False) and hasattr(ahead, "first_norm_for"):
+                next_norm = ahead.first_norm_for(h)
             if next_norm is not None:
                 pending = blocks[i].forward(h, pending, ctx, run, next_norm=next_norm)
             else:

@@ -14,7 +14,7 @@ from halite_amd.config import LayerRun, LayerSpec, ModelConfig, ModelSpec, PartS
 from halite_amd.engine.batch import Segment
 from halite_amd.engine.runner import ModelRunner
 from halite_amd.parts import MIXERS, BuildContext, Decoder, Mixer, ParamDecl, StateNeed
-from halite_amd.parts.base import FEED_FORWARDS, NORMS, POSITIONS, FeedForward, PositionEncoding
+from halite_amd.parts.base import FEED_FORWARDS, NORMS, POSITIONS, FeedForward, PositionEncoding, register_arrangement
 from halite_amd.weights import fill_random
 
 pytestmark = pytest.mark.gpu
@@ -400,3 +400,45 @@ def test_toy_routing_and_other_position_encodings(gpu, dtype):
     mixers = {"a": att_with(rope_a), "b": att_with(rope_b), "pos": add_position}
     ref = {rid: plain_model(runner.model, toks, mixers, {"b": plain_routed}) for rid, toks in requests.items()}
     replay_all(runner, requests, ref, TOL[dtype], 97)
+
+
+# -- an arrangement that knows nothing of the norms folded into products ----------------
+
+
+
+@register_arrangement("pre_norm_plain_test")
+class PlainPreNorm:
+    """The same arithmetic as ``pre_norm`` through the plain interface: four parts, tensors
+    in, a tensor out, no word about the block before or after."""
+
+    def __init__(self, mixer_norm, mixer, ff_norm, ff):
+        self.mixer_norm, self.mixer, self.ff_norm, self.ff = mixer_norm, mixer, ff_norm, ff
+
+    def parts(self):
+        return {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "ff_norm": self.ff_norm, "ff": self.ff}
+
+    def forward(self, h, pending, ctx, run):
+        x = self.mixer_norm.forward(h, delta=pending)
+        assert isinstance(x, torch.Tensor) and (pending is None or isinstance(pending, torch.Tensor))
+        a = self.mixer.forward(x, ctx, run)
+        x = self.ff_norm.forward(h, delta=a)
+        assert isinstance(a, torch.Tensor) and isinstance(x, torch.Tensor)
+        return self.ff.forward(x, ctx)
+
+
+def test_a_plain_arrangement_between_blocks_that_fold_their_norms(gpu):
+    """``pre_norm`` blocks fold their norms into the products around them where both sides can;
+    a block with the plain interface in between is handed tensors only, and the model gives
+    what the plain implementation gives."""
+    rope_p = dict(rotary_dim=16, theta=10000.0, interleaved=False)
+    spec = toy_spec({"a": attention_spec(), "b": attention_spec(heads=2, kv=1), "c": attention_spec(kv=4)},
+                    [LayerRun(layer="a"), LayerRun(layer="b"), LayerRun(layer="c"), LayerRun(layer="a")])
+    spec.layers["b"].arrangement = "pre_norm_plain_test"
+    runner = make_runner(gpu, spec, "bfloat16")
+
+    def att(part, x, positions, i, run, memo):
+        return plain_attention_layer(part, x, positions, rope_p)[0]
+
+    requests = {f"r{i}": [int(t) % 97 for t in tiny.random_tokens(tiny.TINY_A, n, 60 + i)] for i, n in enumerate([50, 3, 35])}
+    ref = {rid: plain_model(runner.model, toks, {"a": att, "b": att, "c": att}) for rid, toks in requests.items()}
+    replay_all(runner, requests, ref, TOL["bfloat16"], 97)
