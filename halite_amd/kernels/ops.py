@@ -483,10 +483,14 @@ def norm_folds(m: int, n: int, k: int, tiled: torch.Tensor | None) -> bool:
     """Whether a product of ``m`` rows against an ``[n, k]`` weight with a tiled copy
     takes an RMSNorm before or after it, or the rotation and the append, into itself: up
     to 16 rows always, 17 to 32 rows on matrices that the small-batch kernel still reads
-    as fast as the library product does."""
+    as fast as the library product does (not too large, rows not much longer than there
+    are rows)."""
     if tiled is None or m <= 0 or k % 8:
         return False
-    return m <= SKINNY_ROWS or (m <= FUSED_ROWS and n * k <= FUSED_MID_ELEMENTS)
+    # (in captured graphs at 24 to 32 rows: o-proj 4096 x 4096 14-15 us against 18 for the
+    # library product and a norm kernel; down 4096 x 14336 36-41 against 33-35, and
+    # 3072 x 8192 22-25 against 21-22: two row tiles read the long rows of X twice as often)
+    return m <= SKINNY_ROWS or (m <= FUSED_ROWS and n * k <= FUSED_MID_ELEMENTS and k <= 2 * n)
 
 
 def gemm_bf16_skinny_norm(

@@ -287,9 +287,14 @@ def test_norm_folded_into_the_products_around_it(gpu, M, d, F, wdt):
     # through linear(): the same two calls, and a reader without a tiled copy gets whole rows
     h = h0.clone()
     rows2 = ops.linear(a, w1, tiled=t1, next_norm=ops.NextNorm(h, nw, eps))
-    assert torch.equal(rows2.x, rows.x) and float((h - h_ref).abs().max()) <= 1e-3 * float(h_ref.abs().max())
-    assert torch.equal(ops.linear(rows2, w2, tiled=t2), got_plain)
-    close(ops.linear(rows2, w2), plain_out, 1.5e-2, "materialised rows")
+    if ops.norm_folds(M, d, F, t1):
+        assert torch.equal(rows2.x, rows.x) and float((h - h_ref).abs().max()) <= 1e-3 * float(h_ref.abs().max())
+    else:  # beyond 16 rows linear() folds only where that is the faster way; the result is then as ever
+        assert isinstance(rows2, torch.Tensor) and torch.equal(h, h0)
+        close(rows2, delta, 4e-3, "the product alone")
+    if ops.norm_folds(M, F, d, t2):
+        assert torch.equal(ops.linear(rows, w2, tiled=t2), got_plain)
+    close(ops.linear(rows, w2), plain_out, 1.5e-2, "materialised rows")
     assert isinstance(ops.linear(a, w1, next_norm=ops.NextNorm(h0.clone(), nw, eps)), torch.Tensor)
 
 

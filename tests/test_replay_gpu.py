@@ -117,7 +117,9 @@ def test_steps_of_few_tokens_take_the_fused_kernels(folders, monkeypatch):
     fused = {"rmsnorm": 2, "qkv_rope_append": layers, "gemm_bf16_skinny_norm": 3 * layers - 1}
     calls.clear()
     runner.step([Segment(slot, 40, toks[40:60], [19])])  # 17 to 32 tokens: two row tiles per wave
-    assert calls == fused
+    # ... where that is the faster way: not for the down-projection, whose rows are long, so
+    # the norm after it is a kernel
+    assert calls == {"rmsnorm": 2 + layers - 1, "qkv_rope_append": layers, "gemm_bf16_skinny_norm": 2 * layers}
     calls.clear()
     runner.step([Segment(slot, 60, toks[60:63], [2])])
     assert calls == fused
