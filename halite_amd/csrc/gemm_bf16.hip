@@ -18,13 +18,15 @@
 // two elements of a rotation pair lie half a head apart; the weight's rows are reordered
 // for this epilogue so that a tile of 16 rows holds eight pairs.
 //
-// With at most 16 rows the RMSNorm between two products (src/halite/nn/normalization.py:
+// With at most 32 rows the RMSNorm between two products (src/halite/nn/normalization.py:
 // 43-57, src/halite/transformers/block.py:56-74) needs no kernel of its own.  The product
 // before it (PREP) adds its result into the float32 residual stream h, writes
 // bf16(w * bf16(h)) for the norm's weight w, and leaves one sum of h^2 per row and
 // workgroup; the product after it (SCALED) adds those sums up in a fixed order and
 // multiplies its float32 accumulators by rsqrt(mean(h^2) + eps), which is the same number
 // up to the place of one bf16 rounding (the norm's kernel rounds h * rstd, this way rounds h).
+// Up to 16 rows always, 17 to 32 rows (two row tiles per wave) where the host finds it the
+// faster way.
 #include "hal_common.h"
 #include "hal_api.h"
 #include <stdlib.h>
@@ -58,15 +60,16 @@ struct RopeEpilogue {
   int H, K, D, page_size, n_pages, tiled;
 };
 
-// The norm folded into the products around it (at most 16 rows).
+// The norm folded into the products around it (at most 32 rows; RW below is 16 for up to
+// 16 rows of X and 32 beyond, the same in the product before the norm and the one after).
 struct NormFusion {
-  // SCALED: X holds bf16(w * bf16(h)); sums of h^2, [n_parts][16], one row of 16 per
+  // SCALED: X holds bf16(w * bf16(h)); sums of h^2, [n_parts][RW], one part per
   // workgroup of the product before; the norm's eps (its size is this product's K)
   const float* ss_in;
   int n_parts;
   float eps;
   // PREP: C is h (float32, added into); the next norm's weight [N], where bf16(w * bf16(h))
-  // goes ([M, N] bf16) and where this workgroup's sums of h^2 go ([workgroups][16])
+  // goes ([M, N] bf16) and where this workgroup's sums of h^2 go ([workgroups][RW])
   const void* norm_w;
   int norm_w_dtype;
   bf16_t* xw_out;
