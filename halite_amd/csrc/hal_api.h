@@ -74,6 +74,12 @@ int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temp
 int hal_sample_greedy(const float* logits, int ld, int n_rows, int V, float* parts,
                       int* out_token, float* out_logprob, hipStream_t stream);
 
+// Rows without filters, greedy or drawn from the whole temperature-scaled distribution; each
+// row is spread over 32 blocks.  `parts`: room for n_rows * 32 * 4 floats.
+int hal_sample_unfiltered(const float* logits, int ld, int n_rows, int V, const float* temperature,
+                          const int* top_k, const uint64_t* seeds, const int* draw_index,
+                          float* parts, int* out_token, float* out_logprob, hipStream_t stream);
+
 int hal_attention_mfma_head_dim();
 int hal_attention_mfma_rows_per_big_item();
 // merge_parts: the most partial results that any merge item joins, or 0 if not known (the

@@ -357,26 +357,45 @@ extern "C" int hal_sample(const float* logits, int ld, int n_rows, int V, const 
   return 0;
 }
 
-// ---- all rows greedy: the row is spread over GREEDY_PARTS blocks --------------------------
-// Stage one: a block takes a contiguous share of a row and leaves its maximum, the first
-// index of that maximum and the sum of exp(x - maximum); stage two joins a row's shares in
-// order (ties go to the lower index, as everywhere).
-#define GREEDY_PARTS 32
-#define GREEDY_THREADS 256
+// ---- no row has a filter: the row is spread over ROW_PARTS blocks ---------------------------
+// Greedy rows and rows that draw from the whole temperature-scaled distribution need the
+// row's maximum, the sum of exp(z - maximum) and, for a draw, one walk to the token at which
+// the cumulative probability passes u: no thresholds.  Stage one: a block takes a contiguous
+// share of a row and leaves its maximum, the first index of that maximum and the sum of
+// exp(z - maximum), z = logit / temperature (the logit itself for a greedy row).  Stage two
+// joins a row's shares in order (ties go to the lower index, as everywhere); for a draw it
+// finds the share in which the running sum passes u * total and walks that share, a quarter
+// per wave, as the one-block kernel walks the row.  Same generator, same rule, same
+// log-probability as there; sums are added in another order, so a draw within rounding of a
+// token's edge may fall to its neighbour.
+#define ROW_PARTS 32
+#define PART_THREADS 256
 
-__global__ void __launch_bounds__(GREEDY_THREADS)
-greedy_part_kernel(const float* __restrict__ logits, int ld, int V, float* __restrict__ parts) {
-  __shared__ ArgMax amax_s[GREEDY_THREADS / HAL_WAVE];
+__device__ __forceinline__ int part_share(int V) { return ((V + ROW_PARTS - 1) / ROW_PARTS + 3) / 4 * 4; }
+// a row is greedy if it has no temperature array (all rows greedy), a temperature of 0 or top_k 1
+__device__ __forceinline__ float row_scale_of(const float* temperature, const int* top_k, int row) {
+  if (!temperature) return 0.f;
+  const float T = temperature[row];
+  return (T == 0.f || (top_k && top_k[row] == 1)) ? 0.f : T;
+}
+
+__global__ void __launch_bounds__(PART_THREADS)
+row_part_kernel(const float* __restrict__ logits, int ld, int V,
+                const float* __restrict__ temperature, const int* __restrict__ top_k,
+                float* __restrict__ parts) {
+  __shared__ ArgMax amax_s[PART_THREADS / HAL_WAVE];
   __shared__ float red[16];
   const int row = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
   const int lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
-  const int share = ((V + GREEDY_PARTS - 1) / GREEDY_PARTS + 3) / 4 * 4;
+  const int share = part_share(V);
   const int begin = part * share;
   const int end = begin + share < V ? begin + share : V;
   const float* x = logits + (size_t)row * ld;
+  const float T = row_scale_of(temperature, top_k, row);
+  const float inv_scale = T == 0.f ? 1.f : T;
   ArgMax am = {-INFINITY, 0x7fffffff};
-  for (int i = begin + tid; i < end; i += GREEDY_THREADS) {
-    const float z = clean_logit(x[i]);
+  for (int i = begin + tid; i < end; i += PART_THREADS) {
+    const float z = clean_logit(x[i]) / inv_scale;
     if (z > am.v) am.v = z, am.i = i;  // a thread's indices rise: the first maximum stays
   }
 #pragma unroll
@@ -389,26 +408,31 @@ greedy_part_kernel(const float* __restrict__ logits, int ld, int V, float* __res
   if (lane == 0) amax_s[wave] = am;
   __syncthreads();
   am = amax_s[0];
-  for (int w = 1; w < GREEDY_THREADS / HAL_WAVE; ++w) am = argmax_merge(am, amax_s[w]);
+  for (int w = 1; w < PART_THREADS / HAL_WAVE; ++w) am = argmax_merge(am, amax_s[w]);
   float sum = 0.f;
-  for (int i = begin + tid; i < end; i += GREEDY_THREADS) sum += expf(clean_logit(x[i]) - am.v);
+  for (int i = begin + tid; i < end; i += PART_THREADS) sum += expf(clean_logit(x[i]) / inv_scale - am.v);
   sum = block_sum(sum, red);
   if (tid == 0) {
-    float* p = parts + ((size_t)row * GREEDY_PARTS + part) * 4;
+    float* p = parts + ((size_t)row * ROW_PARTS + part) * 4;
     p[0] = am.v;
     p[1] = __int_as_float(am.i);
     p[2] = begin < end ? sum : 0.f;
   }
 }
 
-__global__ void __launch_bounds__(HAL_WAVE)
-greedy_join_kernel(const float* __restrict__ parts, int* __restrict__ out_token,
-                   float* __restrict__ out_logprob) {
-  const int row = blockIdx.x, lane = threadIdx.x;
+__global__ void __launch_bounds__(PART_THREADS)
+row_join_kernel(const float* __restrict__ logits, int ld, int V, const float* __restrict__ parts,
+                const float* __restrict__ temperature, const int* __restrict__ top_k,
+                const uint64_t* __restrict__ seeds, const int* __restrict__ draw_index,
+                int* __restrict__ out_token, float* __restrict__ out_logprob) {
+  __shared__ float quarter_mass[PART_THREADS / HAL_WAVE];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
+  // every wave joins the shares for itself (32 values)
   ArgMax am = {-INFINITY, 0x7fffffff};
   float sum = 0.f;
-  if (lane < GREEDY_PARTS) {
-    const float* p = parts + ((size_t)row * GREEDY_PARTS + lane) * 4;
+  if (lane < ROW_PARTS) {
+    const float* p = parts + ((size_t)row * ROW_PARTS + lane) * 4;
     am.v = p[0], am.i = __float_as_int(p[1]), sum = p[2];
   }
   ArgMax best = am;
@@ -419,12 +443,108 @@ greedy_join_kernel(const float* __restrict__ parts, int* __restrict__ out_token,
     o.i = __shfl_xor(best.i, off, HAL_WAVE);
     best = argmax_merge(best, o);
   }
-  const float scaled = (am.v == -INFINITY) ? 0.f : sum * expf(am.v - best.v);
+  const float m = best.v;
+  const float scaled = (am.v == -INFINITY) ? 0.f : sum * expf(am.v - m);
   const float total = wave_sum(scaled);
-  if (lane == 0) {
-    out_token[row] = best.i;
-    out_logprob[row] = -logf(total);
+  const float T = row_scale_of(temperature, top_k, row);
+  if (T == 0.f) {  // greedy
+    if (tid == 0) {
+      out_token[row] = best.i;
+      out_logprob[row] = -logf(total);
+    }
+    return;
   }
+  // the share in which the running sum (shares in order) passes the target
+  const float target = uniform_draw(seeds[row], (uint32_t)draw_index[row]) * total;
+  float incl = scaled;
+#pragma unroll
+  for (int off = 1; off < HAL_WAVE; off <<= 1) {
+    const float up = __shfl_up(incl, off, HAL_WAVE);
+    if (lane >= off) incl += up;
+  }
+  const unsigned long long some = __builtin_amdgcn_ballot_w64(scaled > 0.f);
+  const unsigned long long hit = __builtin_amdgcn_ballot_w64(scaled > 0.f && incl > target);
+  // rounding may leave the target at the very end: the last share that holds anything
+  const int part = hit ? __builtin_ctzll(hit) : 63 - __builtin_clzll(some);
+  const float before_part = __shfl(incl - scaled, part, HAL_WAVE);
+
+  // the share is walked as the one-block kernel walks a row: a quarter per wave
+  const float* x = logits + (size_t)row * ld;
+  const int share = part_share(V);
+  const int p_begin = part * share, p_end = p_begin + share < V ? p_begin + share : V;
+  constexpr int n_waves = PART_THREADS / HAL_WAVE;
+  const int run_len = ((p_end - p_begin + n_waves - 1) / n_waves + HAL_WAVE - 1) / HAL_WAVE * HAL_WAVE;
+  const int begin = p_begin + wave * run_len;
+  const int end = begin + run_len < p_end ? begin + run_len : p_end;
+  auto mass_of = [&](int i, float& z) {
+    if (i >= end) return 0.f;
+    z = clean_logit(x[i]) / T;
+    return expf(z - m);
+  };
+  float mine = 0.f, zz;
+  for (int i = begin + lane; i < end; i += HAL_WAVE) mine += mass_of(i, zz);
+  const float wave_mass = wave_sum(mine);
+  if (lane == 0) quarter_mass[wave] = wave_mass;
+  __syncthreads();
+  float before = before_part;
+  int pick = -1, last = -1;
+  for (int w = 0; w < n_waves; ++w) {
+    if (quarter_mass[w] > 0.f) last = w;
+    if (pick < 0 && quarter_mass[w] > 0.f && before + quarter_mass[w] > target) pick = w;
+    if (pick < 0) before += quarter_mass[w];
+  }
+  if (pick < 0) {  // rounding again: the last quarter that holds anything, from its start
+    pick = last;
+    before = before_part;
+    for (int w = 0; w < pick; ++w) before += quarter_mass[w];
+  }
+  if (wave != pick) return;
+  float run = before;
+  int tok = -1, last_kept = -1;
+  float z_tok = 0.f, z_last = 0.f;
+  for (int i0 = begin; i0 < end && tok < 0; i0 += HAL_WAVE) {
+    float z = 0.f;
+    const float e = mass_of(i0 + lane, z);
+    float inc = e;
+#pragma unroll
+    for (int off = 1; off < HAL_WAVE; off <<= 1) {
+      const float up = __shfl_up(inc, off, HAL_WAVE);
+      if (lane >= off) inc += up;
+    }
+    const unsigned long long kept_lanes = __builtin_amdgcn_ballot_w64(e > 0.f);
+    const unsigned long long found = __builtin_amdgcn_ballot_w64(e > 0.f && run + inc > target);
+    if (kept_lanes) {
+      const int hi = 63 - __builtin_clzll(kept_lanes);
+      last_kept = i0 + hi;
+      z_last = __shfl(z, hi, HAL_WAVE);
+    }
+    if (found) {
+      const int lo = __builtin_ctzll(found);
+      tok = i0 + lo;
+      z_tok = __shfl(z, lo, HAL_WAVE);
+    }
+    run += __shfl(inc, HAL_WAVE - 1, HAL_WAVE);
+  }
+  if (tok < 0) {
+    tok = last_kept;
+    z_tok = z_last;
+  }
+  if (lane == 0) {
+    out_token[row] = tok;
+    out_logprob[row] = z_tok - m - logf(total);
+  }
+}
+
+static int launch_row_parts(const float* logits, int ld, int n_rows, int V, const float* temperature,
+                            const int* top_k, const uint64_t* seeds, const int* draw_index,
+                            float* parts, int* out_token, float* out_logprob, hipStream_t stream) {
+  hipLaunchKernelGGL(row_part_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0, stream, logits,
+                     ld, V, temperature, top_k, parts);
+  HAL_LAUNCH_CHECK();
+  hipLaunchKernelGGL(row_join_kernel, dim3(n_rows), dim3(PART_THREADS), 0, stream, logits, ld, V,
+                     parts, temperature, top_k, seeds, draw_index, out_token, out_logprob);
+  HAL_LAUNCH_CHECK();
+  return 0;
 }
 
 // Greedy decoding of every row: first index of the maximum and its log-probability under
@@ -436,11 +556,23 @@ extern "C" int hal_sample_greedy(const float* logits, int ld, int n_rows, int V,
   HAL_REQUIRE(n_rows <= 65535, "hal_sample_greedy: %d rows exceed the grid limit", n_rows);
   if (n_rows == 0) return 0;
   HAL_REQUIRE(parts != nullptr, "hal_sample_greedy: no room for the partial results");
-  hipLaunchKernelGGL(greedy_part_kernel, dim3(GREEDY_PARTS, n_rows), dim3(GREEDY_THREADS), 0, stream,
-                     logits, ld, V, parts);
-  HAL_LAUNCH_CHECK();
-  hipLaunchKernelGGL(greedy_join_kernel, dim3(n_rows), dim3(HAL_WAVE), 0, stream, parts, out_token,
-                     out_logprob);
-  HAL_LAUNCH_CHECK();
-  return 0;
+  return launch_row_parts(logits, ld, n_rows, V, nullptr, nullptr, nullptr, nullptr, parts, out_token,
+                          out_logprob, stream);
+}
+
+// Rows without filters (no top-k beyond 1, no top-p, no min-p): greedy rows (temperature 0
+// or top_k 1) and draws from the whole temperature-scaled distribution, as hal_sample gives
+// them.  `parts` has room for n_rows * 32 * 4 floats.
+extern "C" int hal_sample_unfiltered(const float* logits, int ld, int n_rows, int V,
+                                     const float* temperature, const int* top_k,
+                                     const uint64_t* seeds, const int* draw_index, float* parts,
+                                     int* out_token, float* out_logprob, hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "hal_sample_unfiltered: bad sizes rows=%d V=%d ld=%d",
+              n_rows, V, ld);
+  HAL_REQUIRE(n_rows <= 65535, "hal_sample_unfiltered: %d rows exceed the grid limit", n_rows);
+  if (n_rows == 0) return 0;
+  HAL_REQUIRE(parts && temperature && top_k && seeds && draw_index,
+              "hal_sample_unfiltered: arguments missing");
+  return launch_row_parts(logits, ld, n_rows, V, temperature, top_k, seeds, draw_index, parts,
+                          out_token, out_logprob, stream);
 }

@@ -366,10 +366,13 @@ def sample(
     draw_index: torch.Tensor,
     all_greedy: bool = False,
     key_scratch: bool = True,
+    unfiltered: bool = False,
 ):
     """Next token and log-probability of every row of float32 ``logits``.
     ``all_greedy`` promises that no row samples (``temperature`` 0 or ``top_k`` 1 in
-    every row): the rows are then spread over many blocks.  Otherwise, with
+    every row), ``unfiltered`` that every row is greedy or draws from its whole
+    distribution (no top-k, top-p or min-p): the rows are then spread over many blocks,
+    in two launches.  Otherwise, with
     ``key_scratch``, the kernel gets room for one 32-bit key per logit, which its passes
     over a row read instead of deriving it again."""
     lib = library.core_library()
@@ -387,6 +390,12 @@ def sample(
     if all_greedy and logits.is_contiguous():  # every row spread over many blocks
         parts = torch.empty((n, 32, 4), dtype=torch.float32, device=logits.device)
         _check(lib, lib.hal_sample_greedy(_ptr(logits), vocab, n, vocab, _ptr(parts), _ptr(tokens), _ptr(logprobs), _stream()))
+        return tokens, logprobs
+    if unfiltered and logits.is_contiguous():
+        parts = torch.empty((n, 32, 4), dtype=torch.float32, device=logits.device)
+        _check(lib, lib.hal_sample_unfiltered(
+            _ptr(logits), vocab, n, vocab, _ptr(temperature), _ptr(top_k), _ptr(seeds), _ptr(draw_index),
+            _ptr(parts), _ptr(tokens), _ptr(logprobs), _stream()))
         return tokens, logprobs
     keys = torch.empty((n, vocab), dtype=torch.int32, device=logits.device) if key_scratch and not all_greedy else None
     _check(

@@ -80,5 +80,7 @@ class Sampler:
         fd = dev[2 * n : 5 * n].view(torch.float32).view(3, n)
         idv = dev[5 * n : 7 * n].view(2, n)
         sd = dev[: 2 * n].view(torch.int64)
+        vocab = logits.shape[1]
+        unfiltered = all(p.greedy or (not 0 < p.top_k < vocab and p.top_p >= 1.0 and p.min_p <= 0.0) for p in params)
         return ops.sample(logits.contiguous(), fd[0], idv[0], fd[1], fd[2], sd, idv[1],
-                          all_greedy=all(p.greedy for p in params))
+                          all_greedy=all(p.greedy for p in params), unfiltered=unfiltered)

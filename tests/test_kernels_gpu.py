@@ -596,6 +596,35 @@ def test_sample_large_vocabulary(gpu, vocab):
         assert agree > 0.8 * n
 
 
+@pytest.mark.parametrize("vocab", [331, 1000, 50257, 128256])
+def test_sample_unfiltered_rows_over_many_blocks(gpu, vocab):
+    """Rows without filters (greedy ones among them) spread over many blocks: the tokens and
+    log-probabilities of the plain sampler, and of the one-block kernel wherever the draw is
+    not within rounding of a token's edge."""
+    n = 48
+    base = rnd(1, vocab, seed=85, scale=3.0)[0]
+    base[vocab // 5] = float("nan")
+    clean = torch.where(torch.isnan(base), torch.full_like(base, -1e5), base)
+    logits = base[None].repeat(n, 1)
+    temps = torch.tensor([0.0 if i % 6 == 5 else (0.7 if i % 2 else 1.3) for i in range(n)])
+    top_k = torch.tensor([1 if i % 12 == 0 else (-1 if i % 3 else vocab) for i in range(n)], dtype=torch.int32)
+    f = lambda v, dt: torch.full((n,), v, dtype=dt, device=gpu)
+    args = (logits.to(gpu), temps.to(gpu), top_k.to(gpu), f(1.0, torch.float32), f(0.0, torch.float32),
+            f(9, torch.int64), torch.arange(n, dtype=torch.int32, device=gpu))
+    tok, lp = ops.sample(*args, unfiltered=True)
+    tok1, lp1 = ops.sample(*args)
+    agree = 0
+    for i in range(n):
+        greedy = float(temps[i]) == 0.0 or int(top_k[i]) == 1
+        params = {"temperature": 0.0 if greedy else float(temps[i]), "seed": 9}
+        t, logprob, margin = P.sample_token(clean, params, i)
+        if greedy or margin > 2e-5:
+            assert int(tok[i]) == t == int(tok1[i]), f"row {i}: many blocks {int(tok[i])}, one block {int(tok1[i])}, plain {t}"
+            assert abs(float(lp[i]) - logprob) < 2e-4 and abs(float(lp[i]) - float(lp1[i])) < 2e-4
+            agree += 1
+    assert agree > 0.6 * n  # with 128 k tokens many a draw lies within rounding of an edge
+
+
 def test_sample_rows_are_independent(gpu):
     logits = rnd(8, 331, seed=82, scale=2.0)
     temp = torch.tensor([0.0, 1.0, 0.5, 2.0, 1.0, 0.0, 1.0, 0.7])
