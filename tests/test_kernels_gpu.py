@@ -90,6 +90,10 @@ def test_silu_mul_and_residual_add(gpu, dtype):
     odd = rnd(7, 2 * 353, seed=16, scale=3.0).to(dt)  # a width that is no multiple of 4
     g, u = odd[:, :353].float(), odd[:, 353:].float()
     close(ops.silu_mul(odd.to(gpu)), u * g * torch.sigmoid(g), 1e-6 if dtype == "float32" else 5e-3)
+    for rows, F in ((7, 348), (301, 1000), (2048, 1432)):  # multiples of 4 only and of 8; many rows
+        big = rnd(rows, 2 * F, seed=17, scale=3.0).to(dt)
+        g, u = big[:, :F].float(), big[:, F:].float()
+        close(ops.silu_mul(big.to(gpu)), u * g * torch.sigmoid(g), 1e-6 if dtype == "float32" else 5e-3)
     h, d = rnd(5, 77, seed=7), rnd(5, 77, seed=8).to(dt)
     close(ops.residual_add(h.to(gpu).clone(), d.to(gpu)), h + d.float(), 1e-7)
 
