@@ -79,6 +79,13 @@ def test_rmsnorm(gpu, dtype, d):
     if dtype == "bfloat16":
         out = ops.rmsnorm(h.to(gpu).clone(), w.float().to(gpu), eps, dt)
         close(out, P.rms_norm(h, w.float(), eps), tol, "norm, 32-bit weight")
+    # many rows (a prompt): smaller blocks, several vectors per thread
+    many, dm = rnd(300, d, seed=6, scale=2.0), rnd(300, d, seed=7).to(dt)
+    xm = many + dm.float()
+    want = P.rms_norm(xm.to(dt), w, eps) if dtype == "float32" else (w.float() * (xm * torch.rsqrt(xm.pow(2).mean(-1, keepdim=True) + eps)).to(dt).float())
+    hg = many.to(gpu).clone()
+    close(ops.rmsnorm(hg, w.to(gpu), eps, dt, delta=dm.to(gpu)), want, tol, "norm of many rows")
+    close(hg, xm, 1e-7, "stream of many rows after add")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
