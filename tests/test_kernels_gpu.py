@@ -251,7 +251,8 @@ def test_qkv_rope_append_in_one_kernel(gpu, M, H, K, D, width, page, tiled):
 
 
 @pytest.mark.parametrize("M", [1, 7, 16, 19, 32])
-@pytest.mark.parametrize("d,F,wdt", [(64, 96, "float32"), (120, 352, "bfloat16"), (4096, 1024, "bfloat16"), (1000, 200, "bfloat16")])
+@pytest.mark.parametrize("d,F,wdt", [(64, 96, "float32"), (120, 352, "bfloat16"), (4096, 1024, "bfloat16"), (1000, 200, "bfloat16"),
+                                     (8192, 512, "bfloat16")])  # the last: more partial sums than a thread asks for ahead
 def test_norm_folded_into_the_products_around_it(gpu, M, d, F, wdt):
     """product -> add into the stream -> RMSNorm -> product (plain and gated), with the norm
     done by the two products, against the same chain with the norm's own kernel and
