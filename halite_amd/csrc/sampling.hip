@@ -535,6 +535,286 @@ row_join_kernel(const float* __restrict__ logits, int ld, int V, const float* __
   }
 }
 
+// ---- rows with filters, spread over many blocks -----------------------------------------
+// The one-block kernel above spends most of its time in the first histogram: a row's keys
+// crowd into a few dozen of the 2,048 bins, and a block's atomics on one bin wait for each
+// other.  Here a row's keys are split over ROW_PARTS blocks for every pass; a block builds
+// its histogram in LDS and adds the bins it has filled to the row's histogram in memory
+// (integers: the order does not matter), and a one-block kernel per row walks that histogram
+// exactly as the kernel above walks its own.  Thresholds are therefore the same keys as
+// there; the drawn token may differ where the draw is within rounding of a token's edge,
+// since the kept masses are added in another order.  Not served: top-k, top-p and min-p all
+// at once, where top-p refers to what top-k kept (two searches one after the other).
+struct FiltRow {
+  float m, total;  // maximum of z and sum of exp(z - m) over the row
+  int best;        // first index of the maximum
+  int flags;       // 1: greedy, 2: top-k is searched, 4: top-p is searched
+  uint32_t prefix[2];
+  uint32_t key_min;
+  uint32_t unused;
+  unsigned long long above[2], target[2];
+};
+static_assert(sizeof(FiltRow) == 64, "FiltRow is 16 words");
+enum { FILT_GREEDY = 1, FILT_K = 2, FILT_P = 4 };
+
+__device__ __forceinline__ int level_shift(int level) { return level == 0 ? 21 : (level == 1 ? 10 : 0); }
+__device__ __forceinline__ int level_up(int level) { return level == 0 ? 32 : (level == 1 ? 21 : 10); }
+
+__global__ void __launch_bounds__(HAL_WAVE)
+filt_join_kernel(const float* __restrict__ parts, const float* __restrict__ temperature,
+                 const int* __restrict__ top_k, const float* __restrict__ top_p, int V,
+                 FiltRow* __restrict__ rows) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  ArgMax am = {-INFINITY, 0x7fffffff};
+  float sum = 0.f;
+  if (lane < ROW_PARTS) {
+    const float* p = parts + ((size_t)row * ROW_PARTS + lane) * 4;
+    am.v = p[0], am.i = __float_as_int(p[1]), sum = p[2];
+  }
+  ArgMax best = am;
+#pragma unroll
+  for (int off = HAL_WAVE / 2; off > 0; off >>= 1) {
+    ArgMax o;
+    o.v = __shfl_xor(best.v, off, HAL_WAVE);
+    o.i = __shfl_xor(best.i, off, HAL_WAVE);
+    best = argmax_merge(best, o);
+  }
+  const float scaled = (am.v == -INFINITY) ? 0.f : sum * expf(am.v - best.v);
+  const float total = wave_sum(scaled);
+  if (lane != 0) return;
+  const bool greedy = row_scale_of(temperature, top_k, row) == 0.f;
+  const int k = top_k[row];
+  FiltRow r;
+  r.m = best.v, r.total = total, r.best = best.i;
+  r.flags = greedy ? FILT_GREEDY : ((k > 0 && k < V ? FILT_K : 0) | (top_p[row] < 1.f ? FILT_P : 0));
+  r.prefix[0] = r.prefix[1] = 0u, r.key_min = 0u, r.unused = 0u;
+  r.above[0] = r.above[1] = 0ull;
+  r.target[0] = (unsigned long long)(k > 0 ? k : 0), r.target[1] = ~0ull;  // top_p of the whole mass, set at level 0
+  rows[row] = r;
+}
+
+// One level of the search: the histogram of a share of the row, added to the row's.
+__global__ void __launch_bounds__(PART_THREADS)
+filt_hist_kernel(const float* __restrict__ logits, int ld, int V,
+                 const float* __restrict__ temperature, const FiltRow* __restrict__ rows, int level,
+                 unsigned long long* __restrict__ hist) {  // [rows][2][SAMPLE_BINS]
+  __shared__ uint32_t count_s[SAMPLE_BINS];
+  __shared__ unsigned long long mass_s[SAMPLE_BINS];
+  const int row = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
+  const FiltRow r = rows[row];
+  const bool on_k = (r.flags & FILT_K) != 0, on_p = (r.flags & FILT_P) != 0;
+  if (!on_k && !on_p) return;
+  for (int b = tid; b < SAMPLE_BINS; b += PART_THREADS) count_s[b] = 0u, mass_s[b] = 0ull;
+  __syncthreads();
+  const int share = part_share(V);
+  const int begin = part * share, end = begin + share < V ? begin + share : V;
+  const float* x = logits + (size_t)row * ld;
+  const float T = temperature[row];
+  const int shift = level_shift(level), up = level_up(level);
+  for (int i = begin + tid; i < end; i += PART_THREADS) {
+    const uint32_t key = sort_key(clean_logit(x[i]) / T);
+    const uint32_t high = level == 0 ? 0u : key >> up;
+    const uint32_t bin = (key >> shift) & (SAMPLE_BINS - 1) & ((1u << (up - shift)) - 1u);
+    if (on_k && high == r.prefix[0]) atomicAdd(&count_s[bin], 1u);
+    if (on_p && high == r.prefix[1])
+      atomicAdd(&mass_s[bin], (unsigned long long)(expf(key_value(key) - r.m) * 1099511627776.0f));
+  }
+  __syncthreads();
+  unsigned long long* h = hist + (size_t)row * 2 * SAMPLE_BINS;
+  for (int b = tid; b < SAMPLE_BINS; b += PART_THREADS) {
+    if (count_s[b]) atomicAdd(&h[b], (unsigned long long)count_s[b]);
+    if (mass_s[b]) atomicAdd(&h[SAMPLE_BINS + b], mass_s[b]);
+  }
+}
+
+// The walk over the row's histogram of one level (as in sample_kernel); leaves the
+// histogram cleared for the next level, and after the last level the smallest kept key.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+filt_find_kernel(FiltRow* __restrict__ rows, unsigned long long* __restrict__ hist,
+                 const float* __restrict__ top_p, int level) {
+  __shared__ unsigned long long scan_tmp[SAMPLE_THREADS / HAL_WAVE];
+  __shared__ unsigned long long whole_mass;
+  __shared__ unsigned long long found_above[2];
+  __shared__ uint32_t found_bin[2];
+  __shared__ int found_any[2];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  FiltRow r = rows[row];
+  const bool on[2] = {(r.flags & FILT_K) != 0, (r.flags & FILT_P) != 0};
+  if (!on[0] && !on[1]) return;
+  unsigned long long* h = hist + (size_t)row * 2 * SAMPLE_BINS;
+  const int shift = level_shift(level), up = level_up(level);
+  if (level == 0 && on[1]) {
+    // the whole mass, as the histogram has it: the reference of top-p
+    unsigned long long all = h[SAMPLE_BINS + 2 * tid] + h[SAMPLE_BINS + 2 * tid + 1];
+    all += block_suffix_u64(all, scan_tmp);
+    if (tid == 0) whole_mass = all;
+    __syncthreads();
+    r.target[1] = (unsigned long long)((double)top_p[row] * (double)whole_mass);
+  }
+#pragma unroll
+  for (int sidx = 0; sidx < 2; ++sidx) {
+    if (!on[sidx]) continue;
+    // bins in descending order: thread t has bins 2t+1 and 2t
+    const unsigned long long h1 = h[sidx * SAMPLE_BINS + 2 * tid + 1], h0 = h[sidx * SAMPLE_BINS + 2 * tid];
+    const unsigned long long higher = r.above[sidx] + block_suffix_u64(h1 + h0, scan_tmp);
+    if (tid == 0) found_bin[sidx] = 0u, found_above[sidx] = r.above[sidx], found_any[sidx] = 0;
+    __syncthreads();
+    if (higher < r.target[sidx] && higher + h1 >= r.target[sidx]) {
+      found_bin[sidx] = 2 * tid + 1, found_above[sidx] = higher, found_any[sidx] = 1;
+    } else if (higher + h1 < r.target[sidx] && higher + h1 + h0 >= r.target[sidx]) {
+      found_bin[sidx] = 2 * tid, found_above[sidx] = higher + h1, found_any[sidx] = 1;
+    }
+    __syncthreads();
+    // a target of zero, or one beyond the whole sum, is met by no bin: the first keeps the
+    // largest key only, the second every key
+    if (!found_any[sidx]) {
+      if (r.target[sidx] == 0ull) {
+        int top = -1;
+        if (h1 != 0ull) top = 2 * tid + 1; else if (h0 != 0ull) top = 2 * tid;
+        if (top >= 0) atomicMax(&found_bin[sidx], (uint32_t)top);
+      }
+      __syncthreads();
+    }
+    r.prefix[sidx] = (r.prefix[sidx] << (up - shift)) | found_bin[sidx];
+    r.above[sidx] = found_above[sidx];
+    __syncthreads();
+  }
+  // cleared for the next level (every thread has read its bins)
+  h[2 * tid] = h[2 * tid + 1] = 0ull;
+  h[SAMPLE_BINS + 2 * tid] = h[SAMPLE_BINS + 2 * tid + 1] = 0ull;
+  if (tid == 0) {
+    if (level == 2) {
+      r.key_min = on[0] ? r.prefix[0] : 0u;
+      if (on[1] && r.prefix[1] > r.key_min) r.key_min = r.prefix[1];
+    }
+    rows[row] = r;
+  }
+}
+
+__device__ __forceinline__ float kept_mass_at(const float* x, int i, float T, const FiltRow& r, float mp,
+                                              float& z) {
+  const uint32_t key = sort_key(clean_logit(x[i]) / T);
+  if (key < r.key_min) return 0.f;
+  z = key_value(key);
+  const float e = expf(z - r.m);
+  return e >= mp ? e : 0.f;
+}
+
+// The kept mass of every share of a row.
+__global__ void __launch_bounds__(PART_THREADS)
+filt_mass_kernel(const float* __restrict__ logits, int ld, int V,
+                 const float* __restrict__ temperature, const float* __restrict__ min_p,
+                 const FiltRow* __restrict__ rows, float* __restrict__ kept) {  // [rows][ROW_PARTS]
+  __shared__ float red[16];
+  const int row = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
+  const FiltRow r = rows[row];
+  if (r.flags & FILT_GREEDY) return;
+  const int share = part_share(V);
+  const int begin = part * share, end = begin + share < V ? begin + share : V;
+  const float* x = logits + (size_t)row * ld;
+  const float T = temperature[row], mp = min_p[row];
+  float mine = 0.f, z;
+  for (int i = begin + tid; i < end; i += PART_THREADS) mine += kept_mass_at(x, i, T, r, mp, z);
+  mine = block_sum(mine, red);
+  if (tid == 0) kept[(size_t)row * ROW_PARTS + part] = mine;
+}
+
+// The draw: the share in which the running kept mass passes u * (kept mass), then the walk
+// through that share, a quarter per wave.
+__global__ void __launch_bounds__(PART_THREADS)
+filt_pick_kernel(const float* __restrict__ logits, int ld, int V,
+                 const float* __restrict__ temperature, const float* __restrict__ min_p,
+                 const FiltRow* __restrict__ rows, const float* __restrict__ kept,
+                 const uint64_t* __restrict__ seeds, const int* __restrict__ draw_index,
+                 int* __restrict__ out_token, float* __restrict__ out_logprob) {
+  __shared__ float quarter_mass[PART_THREADS / HAL_WAVE];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
+  const FiltRow r = rows[row];
+  if (r.flags & FILT_GREEDY) {
+    if (tid == 0) {
+      out_token[row] = r.best;
+      out_logprob[row] = -logf(r.total);
+    }
+    return;
+  }
+  const float mass = lane < ROW_PARTS ? kept[(size_t)row * ROW_PARTS + lane] : 0.f;
+  float incl = mass;
+#pragma unroll
+  for (int off = 1; off < HAL_WAVE; off <<= 1) {
+    const float up = __shfl_up(incl, off, HAL_WAVE);
+    if (lane >= off) incl += up;
+  }
+  const float kept_mass = __shfl(incl, HAL_WAVE - 1, HAL_WAVE);
+  const float target = uniform_draw(seeds[row], (uint32_t)draw_index[row]) * kept_mass;
+  const unsigned long long some = __builtin_amdgcn_ballot_w64(mass > 0.f);
+  const unsigned long long hit = __builtin_amdgcn_ballot_w64(mass > 0.f && incl > target);
+  // (the largest key is always kept, so some share holds something)
+  const int part = hit ? __builtin_ctzll(hit) : (some ? 63 - __builtin_clzll(some) : 0);
+  const float before_part = __shfl(incl - mass, part, HAL_WAVE);
+
+  const float* x = logits + (size_t)row * ld;
+  const float T = temperature[row], mp = min_p[row];
+  const int share = part_share(V);
+  const int p_begin = part * share, p_end = p_begin + share < V ? p_begin + share : V;
+  constexpr int n_waves = PART_THREADS / HAL_WAVE;
+  const int run_len = ((p_end - p_begin + n_waves - 1) / n_waves + HAL_WAVE - 1) / HAL_WAVE * HAL_WAVE;
+  const int begin = p_begin + wave * run_len;
+  const int end = begin + run_len < p_end ? begin + run_len : p_end;
+  float mine = 0.f, zz = 0.f;
+  for (int i = begin + lane; i < end; i += HAL_WAVE) mine += kept_mass_at(x, i, T, r, mp, zz);
+  const float wave_mass = wave_sum(mine);
+  if (lane == 0) quarter_mass[wave] = wave_mass;
+  __syncthreads();
+  float before = before_part;
+  int pick = -1, last = -1;
+  for (int w = 0; w < n_waves; ++w) {
+    if (quarter_mass[w] > 0.f) last = w;
+    if (pick < 0 && quarter_mass[w] > 0.f && before + quarter_mass[w] > target) pick = w;
+    if (pick < 0) before += quarter_mass[w];
+  }
+  if (pick < 0) {  // rounding left the target at the very end: the last quarter that holds anything
+    pick = last < 0 ? 0 : last;
+    before = before_part;
+    for (int w = 0; w < pick; ++w) before += quarter_mass[w];
+  }
+  if (wave != pick) return;
+  float run = before;
+  int tok = -1, last_kept = -1;
+  float z_tok = 0.f, z_last = 0.f;
+  for (int i0 = begin; i0 < end && tok < 0; i0 += HAL_WAVE) {
+    float z = 0.f;
+    const float e = i0 + lane < end ? kept_mass_at(x, i0 + lane, T, r, mp, z) : 0.f;
+    float inc = e;
+#pragma unroll
+    for (int off = 1; off < HAL_WAVE; off <<= 1) {
+      const float up = __shfl_up(inc, off, HAL_WAVE);
+      if (lane >= off) inc += up;
+    }
+    const unsigned long long kept_lanes = __builtin_amdgcn_ballot_w64(e > 0.f);
+    const unsigned long long found = __builtin_amdgcn_ballot_w64(e > 0.f && run + inc > target);
+    if (kept_lanes) {
+      const int hi = 63 - __builtin_clzll(kept_lanes);
+      last_kept = i0 + hi;
+      z_last = __shfl(z, hi, HAL_WAVE);
+    }
+    if (found) {
+      const int lo = __builtin_ctzll(found);
+      tok = i0 + lo;
+      z_tok = __shfl(z, lo, HAL_WAVE);
+    }
+    run += __shfl(inc, HAL_WAVE - 1, HAL_WAVE);
+  }
+  if (tok < 0) {
+    tok = last_kept >= 0 ? last_kept : r.best;
+    z_tok = last_kept >= 0 ? z_last : r.m;
+  }
+  if (lane == 0) {
+    out_token[row] = tok;
+    out_logprob[row] = z_tok - r.m - logf(r.total);
+  }
+}
+
 static int launch_row_parts(const float* logits, int ld, int n_rows, int V, const float* temperature,
                             const int* top_k, const uint64_t* seeds, const int* draw_index,
                             float* parts, int* out_token, float* out_logprob, hipStream_t stream) {
@@ -575,4 +855,41 @@ extern "C" int hal_sample_unfiltered(const float* logits, int ld, int n_rows, in
               "hal_sample_unfiltered: arguments missing");
   return launch_row_parts(logits, ld, n_rows, V, temperature, top_k, seeds, draw_index, parts,
                           out_token, out_logprob, stream);
+}
+
+// Rows with filters (and greedy or unfiltered ones among them), every row spread over 32
+// blocks in every pass.  Not for a row with top-k, top-p and min-p all at once (hal_sample
+// serves that).  Room: `parts` n_rows * 32 * 4 floats, `kept` n_rows * 32 floats, `state`
+// n_rows * 16 words, `hist` n_rows * 2 * 2048 64-bit words, which must be zero (and are
+// left zero).
+extern "C" int hal_sample_spread(const float* logits, int ld, int n_rows, int V,
+                                 const float* temperature, const int* top_k, const float* top_p,
+                                 const float* min_p, const uint64_t* seeds, const int* draw_index,
+                                 float* parts, float* kept, void* state, void* hist,
+                                 int* out_token, float* out_logprob, hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "hal_sample_spread: bad sizes rows=%d V=%d ld=%d",
+              n_rows, V, ld);
+  HAL_REQUIRE(n_rows <= 65535, "hal_sample_spread: %d rows exceed the grid limit", n_rows);
+  if (n_rows == 0) return 0;
+  HAL_REQUIRE(temperature && top_k && top_p && min_p && seeds && draw_index && parts && kept &&
+                  state && hist && ((uintptr_t)state % 8) == 0 && ((uintptr_t)hist % 8) == 0,
+              "hal_sample_spread: arguments missing");
+  FiltRow* rows = (FiltRow*)state;
+  unsigned long long* h = (unsigned long long*)hist;
+  hipLaunchKernelGGL(row_part_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0, stream, logits,
+                     ld, V, temperature, top_k, parts);
+  hipLaunchKernelGGL(filt_join_kernel, dim3(n_rows), dim3(HAL_WAVE), 0, stream, parts, temperature,
+                     top_k, top_p, V, rows);
+  for (int level = 0; level < 3; ++level) {
+    hipLaunchKernelGGL(filt_hist_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0, stream,
+                       logits, ld, V, temperature, rows, level, h);
+    hipLaunchKernelGGL(filt_find_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, rows, h,
+                       top_p, level);
+  }
+  hipLaunchKernelGGL(filt_mass_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0, stream, logits,
+                     ld, V, temperature, min_p, rows, kept);
+  hipLaunchKernelGGL(filt_pick_kernel, dim3(n_rows), dim3(PART_THREADS), 0, stream, logits, ld, V,
+                     temperature, min_p, rows, kept, seeds, draw_index, out_token, out_logprob);
+  HAL_LAUNCH_CHECK();
+  return 0;
 }

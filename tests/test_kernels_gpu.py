@@ -526,13 +526,14 @@ def test_linear_dispatch(gpu):
     assert ops.linear(x, w.to(gpu)).dtype == torch.bfloat16
 
 
-def _sample(gpu, logits, **kw):
+def _sample(gpu, logits, spread=False, **kw):
     n = logits.shape[0]
     f = lambda v, dt: torch.full((n,), v, dtype=dt, device=gpu) if not torch.is_tensor(v) else v.to(gpu)
     return ops.sample(
         logits.to(gpu), f(kw.get("temperature", 1.0), torch.float32), f(kw.get("top_k", -1), torch.int32),
         f(kw.get("top_p", 1.0), torch.float32), f(kw.get("min_p", 0.0), torch.float32),
         f(kw.get("seed", 7), torch.int64), kw.get("draw", torch.arange(n, dtype=torch.int32)).to(gpu),
+        spread=spread,
     )
 
 
@@ -563,7 +564,14 @@ def test_sample_matches_the_plain_sampler(gpu, kw):
     vocab, n = 1000, 400
     base = rnd(1, vocab, seed=81, scale=2.5)[0]
     logits = base[None].repeat(n, 1)
-    tok, lp = _sample(gpu, logits, seed=11, **kw)
+    both_ways = [_sample(gpu, logits, seed=11, **kw)]
+    if not ("top_k" in kw and "top_p" in kw and "min_p" in kw):  # the rows spread over many blocks
+        both_ways.append(_sample(gpu, logits, seed=11, spread=True, **kw))
+    for tok, lp in both_ways:
+        _compare_with_plain(base, kw, tok, lp, n)
+
+
+def _compare_with_plain(base, kw, tok, lp, n):
     params = {"temperature": 1.0, "seed": 11, **kw}
     probs = P.filtered_probabilities(base, params["temperature"], params.get("top_k", -1), params.get("top_p", 1.0), params.get("min_p", 0.0))
     agree = 0
@@ -597,15 +605,19 @@ def test_sample_large_vocabulary(gpu, vocab):
             torch.arange(n, dtype=torch.int32, device=gpu), key_scratch=False,  # the keys are derived again in every pass
         )
         assert torch.equal(tok, tok_again)
-        agree = 0
-        for i in range(n):
-            t, logprob, margin = P.sample_token(clean, params, i)
-            assert probs[int(tok[i])] > 0, f"{kw}: a filtered token was sampled"
-            if margin > 2e-5:
-                assert int(tok[i]) == t, f"{kw} draw {i}: kernel {int(tok[i])}, plain {t}"
-                assert abs(float(lp[i]) - logprob) < 2e-4
-                agree += 1
-        assert agree > 0.8 * n
+        ways = [(tok, lp)]
+        if not ("top_k" in kw and "top_p" in kw and "min_p" in kw):  # the rows spread over many blocks
+            ways.append(_sample(gpu, logits, seed=5, spread=True, **kw))
+        for tok, lp in ways:
+            agree = 0
+            for i in range(n):
+                t, logprob, margin = P.sample_token(clean, params, i)
+                assert probs[int(tok[i])] > 0, f"{kw}: a filtered token was sampled"
+                if margin > 2e-5:
+                    assert int(tok[i]) == t, f"{kw} draw {i}: kernel {int(tok[i])}, plain {t}"
+                    assert abs(float(lp[i]) - logprob) < 2e-4
+                    agree += 1
+            assert agree > 0.8 * n
 
 
 @pytest.mark.parametrize("vocab", [331, 1000, 50257, 128256])
