@@ -82,7 +82,7 @@ int hal_sample_unfiltered(const float* logits, int ld, int n_rows, int V, const 
 
 // Rows with filters spread over 32 blocks a pass (not top-k, top-p and min-p all at once in
 // one row).  parts: n_rows * 32 * 4 floats; kept: n_rows * 32 floats; state: n_rows * 16
-// words; hist: n_rows * 2 * 2048 64-bit words, zero on entry and on return.
+// words; hist: n_rows * 2 * 2048 64-bit words.
 int hal_sample_spread(const float* logits, int ld, int n_rows, int V, const float* temperature,
                       const int* top_k, const float* top_p, const float* min_p,
                       const uint64_t* seeds, const int* draw_index, float* parts, float* kept,

@@ -563,8 +563,10 @@ __device__ __forceinline__ int level_up(int level) { return level == 0 ? 32 : (l
 __global__ void __launch_bounds__(HAL_WAVE)
 filt_join_kernel(const float* __restrict__ parts, const float* __restrict__ temperature,
                  const int* __restrict__ top_k, const float* __restrict__ top_p, int V,
-                 FiltRow* __restrict__ rows) {
+                 FiltRow* __restrict__ rows, unsigned long long* __restrict__ hist) {
   const int row = blockIdx.x, lane = threadIdx.x;
+  // the row's histogram starts at zero (the searches leave it so, but the room may be new)
+  for (int b = lane; b < 2 * SAMPLE_BINS; b += HAL_WAVE) hist[(size_t)row * 2 * SAMPLE_BINS + b] = 0ull;
   ArgMax am = {-INFINITY, 0x7fffffff};
   float sum = 0.f;
   if (lane < ROW_PARTS) {
@@ -860,8 +862,7 @@ extern "C" int hal_sample_unfiltered(const float* logits, int ld, int n_rows, in
 // Rows with filters (and greedy or unfiltered ones among them), every row spread over 32
 // blocks in every pass.  Not for a row with top-k, top-p and min-p all at once (hal_sample
 // serves that).  Room: `parts` n_rows * 32 * 4 floats, `kept` n_rows * 32 floats, `state`
-// n_rows * 16 words, `hist` n_rows * 2 * 2048 64-bit words, which must be zero (and are
-// left zero).
+// n_rows * 16 words, `hist` n_rows * 2 * 2048 64-bit words.
 extern "C" int hal_sample_spread(const float* logits, int ld, int n_rows, int V,
                                  const float* temperature, const int* top_k, const float* top_p,
                                  const float* min_p, const uint64_t* seeds, const int* draw_index,
@@ -879,7 +880,7 @@ extern "C" int hal_sample_spread(const float* logits, int ld, int n_rows, int V,
   hipLaunchKernelGGL(row_part_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0, stream, logits,
                      ld, V, temperature, top_k, parts);
   hipLaunchKernelGGL(filt_join_kernel, dim3(n_rows), dim3(HAL_WAVE), 0, stream, parts, temperature,
-                     top_k, top_p, V, rows);
+                     top_k, top_p, V, rows, h);
   for (int level = 0; level < 3; ++level) {
     hipLaunchKernelGGL(filt_hist_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0, stream,
                        logits, ld, V, temperature, rows, level, h);

@@ -404,7 +404,7 @@ def sample(
         parts = torch.empty((n, 32, 4), dtype=torch.float32, device=dev)
         kept = torch.empty((n, 32), dtype=torch.float32, device=dev)
         state = torch.empty((n, 16), dtype=torch.int32, device=dev)
-        hist = torch.zeros((n, 2, 2048), dtype=torch.int64, device=dev)
+        hist = torch.empty((n, 2, 2048), dtype=torch.int64, device=dev)
         _check(lib, lib.hal_sample_spread(
             _ptr(logits), vocab, n, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(min_p),
             _ptr(seeds), _ptr(draw_index), _ptr(parts), _ptr(kept), _ptr(state), _ptr(hist),
