@@ -57,9 +57,9 @@ int hal_qkv_rope_append(const void* X, int ldx, const void* W, void* q_out, int 
                         hipStream_t stream);
 
 // The product for M <= 32 rows with the RMSNorm before it (ss_in: partial sums of squares
-// [n_parts, 16] (32 for more than 16 rows) left by the product before; X holds bf16(w * bf16(h))) or after it
-// (norm_w: C is the float32 stream h, added into; xw_out [M, N] and ss_out [ceil(N/16), 16]
-// are left for the product after) folded in.
+// [n_parts, 16] (32 for more than 16 rows) left by the product before; X holds
+// bf16(w * bf16(h))) or after it (norm_w: C is the float32 stream h, added into; xw_out [M, N]
+// and ss_out [ceil(N/16), 16 or 32] are left for the product after) folded in.
 int hal_gemm_bf16_skinny_norm(const void* X, int ldx, const void* W, const void* W2, int ldw,
                               void* C, int ldc, int M, int N, int K, const float* ss_in,
                               int n_parts, float eps, const void* norm_w, int norm_w_dtype,
@@ -70,7 +70,7 @@ int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temp
                const int* draw_index, int* out_token, float* out_logprob, uint32_t* key_rows,
                hipStream_t stream);
 
-// ---- the head-size-specific library (attention_mfma.hip) ---------------------------------
+// Greedy decoding of every row, each row spread over 32 blocks.  `parts`: n_rows * 32 * 4 floats.
 int hal_sample_greedy(const float* logits, int ld, int n_rows, int V, float* parts,
                       int* out_token, float* out_logprob, hipStream_t stream);
 
@@ -89,6 +89,7 @@ int hal_sample_spread(const float* logits, int ld, int n_rows, int V, const floa
                       void* state, void* hist, int* out_token, float* out_logprob,
                       hipStream_t stream);
 
+// ---- the head-size-specific library (attention_mfma.hip) ---------------------------------
 int hal_attention_mfma_head_dim();
 int hal_attention_mfma_rows_per_big_item();
 // merge_parts: the most partial results that any merge item joins, or 0 if not known (the
