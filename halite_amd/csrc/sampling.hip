@@ -155,7 +155,7 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
 
   if (greedy) {
     if (tid == 0) {
-      out_token[row] = am.i;
+      out_token[row] = am.i < V ? am.i : 0;  // (a row of nothing but -inf has no maximum)
       out_logprob[row] = -logf(total);  // z_max - m - log(total)
     }
     return;
@@ -304,6 +304,7 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
   __syncthreads();
   int pick = chosen_thread;
   if (pick == 0x7fffffff) pick = last_thread;  // rounding left the target at the very end
+  if (pick < 0) pick = 0;                      // nothing is kept anywhere: token 0 below
   if (wave != pick) return;
   float run = before;
   int tok = -1, last_kept = -1;
@@ -332,8 +333,8 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
     run += __shfl(incl, HAL_WAVE - 1, HAL_WAVE);
   }
   if (tok < 0) {
-    tok = last_kept;
-    z_tok = z_last;
+    tok = last_kept >= 0 ? last_kept : (am.i < V ? am.i : 0);
+    z_tok = last_kept >= 0 ? z_last : m;
   }
   if (lane == 0) {
     out_token[row] = tok;
@@ -449,7 +450,7 @@ row_join_kernel(const float* __restrict__ logits, int ld, int V, const float* __
   const float T = row_scale_of(temperature, top_k, row);
   if (T == 0.f) {  // greedy
     if (tid == 0) {
-      out_token[row] = best.i;
+      out_token[row] = best.i < V ? best.i : 0;
       out_logprob[row] = -logf(total);
     }
     return;
@@ -465,7 +466,8 @@ row_join_kernel(const float* __restrict__ logits, int ld, int V, const float* __
   const unsigned long long some = __builtin_amdgcn_ballot_w64(scaled > 0.f);
   const unsigned long long hit = __builtin_amdgcn_ballot_w64(scaled > 0.f && incl > target);
   // rounding may leave the target at the very end: the last share that holds anything
-  const int part = hit ? __builtin_ctzll(hit) : 63 - __builtin_clzll(some);
+  // (a row of nothing but -inf holds nothing anywhere: share 0 then, and token 0 below)
+  const int part = hit ? __builtin_ctzll(hit) : (some ? 63 - __builtin_clzll(some) : 0);
   const float before_part = __shfl(incl - scaled, part, HAL_WAVE);
 
   // the share is walked as the one-block kernel walks a row: a quarter per wave
@@ -494,7 +496,7 @@ row_join_kernel(const float* __restrict__ logits, int ld, int V, const float* __
     if (pick < 0) before += quarter_mass[w];
   }
   if (pick < 0) {  // rounding again: the last quarter that holds anything, from its start
-    pick = last;
+    pick = last < 0 ? 0 : last;
     before = before_part;
     for (int w = 0; w < pick; ++w) before += quarter_mass[w];
   }
@@ -526,8 +528,8 @@ row_join_kernel(const float* __restrict__ logits, int ld, int V, const float* __
     run += __shfl(inc, HAL_WAVE - 1, HAL_WAVE);
   }
   if (tok < 0) {
-    tok = last_kept;
-    z_tok = z_last;
+    tok = last_kept >= 0 ? last_kept : (best.i < V ? best.i : 0);
+    z_tok = last_kept >= 0 ? z_last : m;
   }
   if (lane == 0) {
     out_token[row] = tok;
@@ -735,7 +737,7 @@ filt_pick_kernel(const float* __restrict__ logits, int ld, int V,
   const FiltRow r = rows[row];
   if (r.flags & FILT_GREEDY) {
     if (tid == 0) {
-      out_token[row] = r.best;
+      out_token[row] = r.best < V ? r.best : 0;
       out_logprob[row] = -logf(r.total);
     }
     return;
@@ -808,7 +810,7 @@ filt_pick_kernel(const float* __restrict__ logits, int ld, int V,
     run += __shfl(inc, HAL_WAVE - 1, HAL_WAVE);
   }
   if (tok < 0) {
-    tok = last_kept >= 0 ? last_kept : r.best;
+    tok = last_kept >= 0 ? last_kept : (r.best < V ? r.best : 0);
     z_tok = last_kept >= 0 ? z_last : r.m;
   }
   if (lane == 0) {

@@ -649,6 +649,28 @@ def test_sample_unfiltered_rows_over_many_blocks(gpu, vocab):
     assert agree > 0.6 * n  # with 128 k tokens many a draw lies within rounding of an edge
 
 
+def test_sample_rows_that_hold_nothing(gpu):
+    """A row of nothing but -inf (no distribution at all) and a row of nothing but NaN
+    (uniform, by the NaN rule): every way of sampling still returns a token of the vocabulary."""
+    vocab = 1000
+    logits = torch.full((4, vocab), float("-inf"))
+    logits[1] = float("nan")
+    logits[2] = rnd(1, vocab, seed=3)[0]
+    logits[3, 1:] = float("-inf")
+    logits[3, 0] = 0.5
+    for kw in ({"temperature": 0.0}, {}, {"top_k": 5}, {"top_p": 0.5}, {"min_p": 0.2}):
+        for spread in (False, True):
+            tok, _ = _sample(gpu, logits, spread=spread, **kw)
+            assert all(0 <= int(t) < vocab for t in tok), (kw, spread, tok.tolist())
+            assert int(tok[3]) == 0
+        n = logits.shape[0]
+        f = lambda v, dt: torch.full((n,), v, dtype=dt, device=gpu)
+        tok, _ = ops.sample(logits.to(gpu), f(kw.get("temperature", 1.0), torch.float32), f(-1, torch.int32),
+                            f(1.0, torch.float32), f(0.0, torch.float32), f(7, torch.int64), f(0, torch.int32),
+                            unfiltered=True, all_greedy=kw.get("temperature") == 0.0)
+        assert all(0 <= int(t) < vocab for t in tok) and int(tok[3]) == 0
+
+
 def test_sample_rows_are_independent(gpu):
     logits = rnd(8, 331, seed=82, scale=2.0)
     temp = torch.tensor([0.0, 1.0, 0.5, 2.0, 1.0, 0.0, 1.0, 0.7])
