@@ -425,6 +425,7 @@ SKINNY_MAX_ROWS = 64  # what the kernel takes
 SKINNY_ROWS = 16  # up to here it beats the library product
 FUSED_ROWS = 32  # what the epilogues that take other kernels' work take
 FUSED_MID_ELEMENTS = 32 * 1024 * 1024  # the largest matrix on which they pay at 17 to 32 rows
+GATED_MID_ELEMENTS = 64 * 1024 * 1024  # the same for the gated product with SiLU*mul (each of its two matrices)
 # ... if the weights lie in its tiled order.  On row-major weights (a model too large for
 # the second copy) it wins only on small matrices or a single row: measured on Llama-3.1-70B
 # shapes at 8 and 16 rows, the library reads 4.7-5.5 TB/s where the kernel reads 3.2-4.6.

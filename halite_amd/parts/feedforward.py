@@ -73,7 +73,7 @@ class GatedFeedForward(FeedForward):
         # 25 at 8192 x 3072, 202 against 179 at 28672 x 8192).
         m, d = x.shape
         small = (self.t_gate is not None and x.dtype == torch.bfloat16 and d % 8 == 0
-                 and (m <= ops.SKINNY_ROWS or (m <= ops.FUSED_ROWS and f * d <= 64 * 2**20)))
+                 and (m <= ops.SKINNY_ROWS or (m <= ops.FUSED_ROWS and f * d <= ops.GATED_MID_ELEMENTS)))
         if isinstance(x, ops.NormedRows):
             if small:
                 act = ops.gemm_bf16_skinny_norm(x, self.t_gate, (f, d), w_up_tiled=self.t_up)
