@@ -80,13 +80,13 @@ int hal_sample_unfiltered(const float* logits, int ld, int n_rows, int V, const 
                           const int* top_k, const uint64_t* seeds, const int* draw_index,
                           float* parts, int* out_token, float* out_logprob, hipStream_t stream);
 
-// Rows with filters spread over 32 blocks a pass (not top-k, top-p and min-p all at once in
-// one row).  parts: n_rows * 32 * 4 floats; kept: n_rows * 32 floats; state: n_rows * 16
-// words; hist: n_rows * 2 * 2048 64-bit words.
+// Rows with filters spread over 32 blocks a pass.  any_late: some row has top-k, top-p and
+// min-p all at once (searched twice).  parts: n_rows * 32 * 4 floats; kept: n_rows * 32
+// floats; state: n_rows * 20 words; hist: n_rows * 2 * 2048 64-bit words.
 int hal_sample_spread(const float* logits, int ld, int n_rows, int V, const float* temperature,
                       const int* top_k, const float* top_p, const float* min_p,
                       const uint64_t* seeds, const int* draw_index, float* parts, float* kept,
-                      void* state, void* hist, int* out_token, float* out_logprob,
+                      void* state, void* hist, int any_late, int* out_token, float* out_logprob,
                       hipStream_t stream);
 
 // ---- the head-size-specific library (attention_mfma.hip) ---------------------------------

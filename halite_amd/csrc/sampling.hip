@@ -545,27 +545,32 @@ row_join_kernel(const float* __restrict__ logits, int ld, int V, const float* __
 // (integers: the order does not matter), and a one-block kernel per row walks that histogram
 // exactly as the kernel above walks its own.  Thresholds are therefore the same keys as
 // there; the drawn token may differ where the draw is within rounding of a token's edge,
-// since the kept masses are added in another order.  Not served: top-k, top-p and min-p all
-// at once, where top-p refers to what top-k kept (two searches one after the other).
+// since the kept masses are added in another order.  A row with top-k, top-p and min-p all
+// at once, where top-p refers to what top-k kept, is searched twice: top-k first, then (the
+// `late` passes) the mass that top-k kept and top-p within it.
 struct FiltRow {
   float m, total;  // maximum of z and sum of exp(z - m) over the row
   int best;        // first index of the maximum
-  int flags;       // 1: greedy, 2: top-k is searched, 4: top-p is searched
+  int flags;       // FILT_*
   uint32_t prefix[2];
   uint32_t key_min;
   uint32_t unused;
   unsigned long long above[2], target[2];
+  unsigned long long kept_by_k;  // late rows: the mass of the keys that top-k kept
+  unsigned long long unused2;
 };
-static_assert(sizeof(FiltRow) == 64, "FiltRow is 16 words");
-enum { FILT_GREEDY = 1, FILT_K = 2, FILT_P = 4 };
+static_assert(sizeof(FiltRow) == 80, "FiltRow is 20 words");
+// greedy; top-k is searched; top-p is searched beside it; top-p is searched after it (late)
+enum { FILT_GREEDY = 1, FILT_K = 2, FILT_P = 4, FILT_P_LATE = 8 };
 
 __device__ __forceinline__ int level_shift(int level) { return level == 0 ? 21 : (level == 1 ? 10 : 0); }
 __device__ __forceinline__ int level_up(int level) { return level == 0 ? 32 : (level == 1 ? 21 : 10); }
 
 __global__ void __launch_bounds__(HAL_WAVE)
 filt_join_kernel(const float* __restrict__ parts, const float* __restrict__ temperature,
-                 const int* __restrict__ top_k, const float* __restrict__ top_p, int V,
-                 FiltRow* __restrict__ rows, unsigned long long* __restrict__ hist) {
+                 const int* __restrict__ top_k, const float* __restrict__ top_p,
+                 const float* __restrict__ min_p, int V, FiltRow* __restrict__ rows,
+                 unsigned long long* __restrict__ hist) {
   const int row = blockIdx.x, lane = threadIdx.x;
   // the row's histogram starts at zero (the searches leave it so, but the room may be new)
   for (int b = lane; b < 2 * SAMPLE_BINS; b += HAL_WAVE) hist[(size_t)row * 2 * SAMPLE_BINS + b] = 0ull;
@@ -590,8 +595,11 @@ filt_join_kernel(const float* __restrict__ parts, const float* __restrict__ temp
   const int k = top_k[row];
   FiltRow r;
   r.m = best.v, r.total = total, r.best = best.i;
-  r.flags = greedy ? FILT_GREEDY : ((k > 0 && k < V ? FILT_K : 0) | (top_p[row] < 1.f ? FILT_P : 0));
-  r.prefix[0] = r.prefix[1] = 0u, r.key_min = 0u, r.unused = 0u;
+  const bool want_k = k > 0 && k < V, want_p = top_p[row] < 1.f;
+  // with min_p the reference renormalises after top-k, so top-p refers to what top-k kept
+  const bool late = want_k && want_p && min_p[row] > 0.f;
+  r.flags = greedy ? FILT_GREEDY : ((want_k ? FILT_K : 0) | (want_p ? (late ? FILT_P_LATE : FILT_P) : 0));
+  r.prefix[0] = r.prefix[1] = 0u, r.key_min = 0u, r.unused = 0u, r.kept_by_k = 0ull, r.unused2 = 0ull;
   r.above[0] = r.above[1] = 0ull;
   r.target[0] = (unsigned long long)(k > 0 ? k : 0), r.target[1] = ~0ull;  // top_p of the whole mass, set at level 0
   rows[row] = r;
@@ -601,12 +609,13 @@ filt_join_kernel(const float* __restrict__ parts, const float* __restrict__ temp
 __global__ void __launch_bounds__(PART_THREADS)
 filt_hist_kernel(const float* __restrict__ logits, int ld, int V,
                  const float* __restrict__ temperature, const FiltRow* __restrict__ rows, int level,
-                 unsigned long long* __restrict__ hist) {  // [rows][2][SAMPLE_BINS]
+                 int late, unsigned long long* __restrict__ hist) {  // [rows][2][SAMPLE_BINS]
   __shared__ uint32_t count_s[SAMPLE_BINS];
   __shared__ unsigned long long mass_s[SAMPLE_BINS];
   const int row = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
   const FiltRow r = rows[row];
-  const bool on_k = (r.flags & FILT_K) != 0, on_p = (r.flags & FILT_P) != 0;
+  const bool on_k = !late && (r.flags & FILT_K) != 0;
+  const bool on_p = (r.flags & (late ? FILT_P_LATE : FILT_P)) != 0;
   if (!on_k && !on_p) return;
   for (int b = tid; b < SAMPLE_BINS; b += PART_THREADS) count_s[b] = 0u, mass_s[b] = 0ull;
   __syncthreads();
@@ -635,7 +644,7 @@ filt_hist_kernel(const float* __restrict__ logits, int ld, int V,
 // histogram cleared for the next level, and after the last level the smallest kept key.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 filt_find_kernel(FiltRow* __restrict__ rows, unsigned long long* __restrict__ hist,
-                 const float* __restrict__ top_p, int level) {
+                 const float* __restrict__ top_p, int level, int late) {
   __shared__ unsigned long long scan_tmp[SAMPLE_THREADS / HAL_WAVE];
   __shared__ unsigned long long whole_mass;
   __shared__ unsigned long long found_above[2];
@@ -643,11 +652,14 @@ filt_find_kernel(FiltRow* __restrict__ rows, unsigned long long* __restrict__ hi
   __shared__ int found_any[2];
   const int row = blockIdx.x, tid = threadIdx.x;
   FiltRow r = rows[row];
-  const bool on[2] = {(r.flags & FILT_K) != 0, (r.flags & FILT_P) != 0};
+  const bool on[2] = {!late && (r.flags & FILT_K) != 0, (r.flags & (late ? FILT_P_LATE : FILT_P)) != 0};
   if (!on[0] && !on[1]) return;
   unsigned long long* h = hist + (size_t)row * 2 * SAMPLE_BINS;
   const int shift = level_shift(level), up = level_up(level);
-  if (level == 0 && on[1]) {
+  if (level == 0 && late) {
+    // top-p of what top-k kept
+    r.target[1] = (unsigned long long)((double)top_p[row] * (double)r.kept_by_k);
+  } else if (level == 0 && on[1]) {
     // the whole mass, as the histogram has it: the reference of top-p
     unsigned long long all = h[SAMPLE_BINS + 2 * tid] + h[SAMPLE_BINS + 2 * tid + 1];
     all += block_suffix_u64(all, scan_tmp);
@@ -688,10 +700,43 @@ filt_find_kernel(FiltRow* __restrict__ rows, unsigned long long* __restrict__ hi
   h[SAMPLE_BINS + 2 * tid] = h[SAMPLE_BINS + 2 * tid + 1] = 0ull;
   if (tid == 0) {
     if (level == 2) {
-      r.key_min = on[0] ? r.prefix[0] : 0u;
+      if (!late) r.key_min = on[0] ? r.prefix[0] : 0u;
       if (on[1] && r.prefix[1] > r.key_min) r.key_min = r.prefix[1];
     }
     rows[row] = r;
+  }
+}
+
+// Late rows: the mass of the keys that top-k kept, as the histograms count it (integers).
+__global__ void __launch_bounds__(PART_THREADS)
+filt_kept_by_k_kernel(const float* __restrict__ logits, int ld, int V,
+                      const float* __restrict__ temperature, FiltRow* __restrict__ rows) {
+  __shared__ unsigned long long tmp[PART_THREADS / HAL_WAVE];
+  const int row = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
+  const FiltRow r = rows[row];
+  if (!(r.flags & FILT_P_LATE)) return;
+  const int share = part_share(V);
+  const int begin = part * share, end = begin + share < V ? begin + share : V;
+  const float* x = logits + (size_t)row * ld;
+  const float T = temperature[row];
+  unsigned long long mine = 0ull;
+  for (int i = begin + tid; i < end; i += PART_THREADS) {
+    const uint32_t key = sort_key(clean_logit(x[i]) / T);
+    if (key >= r.key_min) mine += (unsigned long long)(expf(key_value(key) - r.m) * 1099511627776.0f);
+  }
+#pragma unroll
+  for (int off = HAL_WAVE / 2; off > 0; off >>= 1) {
+    const uint32_t lo = __shfl_xor((uint32_t)mine, off, HAL_WAVE);
+    const uint32_t hi = __shfl_xor((uint32_t)(mine >> 32), off, HAL_WAVE);
+    mine += ((unsigned long long)hi << 32) | lo;
+  }
+  if (lane == 0) tmp[wave] = mine;
+  __syncthreads();
+  if (tid == 0) {
+    unsigned long long all = 0ull;
+    for (int w = 0; w < PART_THREADS / HAL_WAVE; ++w) all += tmp[w];
+    if (all) atomicAdd(&rows[row].kept_by_k, all);
   }
 }
 
@@ -862,13 +907,14 @@ extern "C" int hal_sample_unfiltered(const float* logits, int ld, int n_rows, in
 }
 
 // Rows with filters (and greedy or unfiltered ones among them), every row spread over 32
-// blocks in every pass.  Not for a row with top-k, top-p and min-p all at once (hal_sample
-// serves that).  Room: `parts` n_rows * 32 * 4 floats, `kept` n_rows * 32 floats, `state`
-// n_rows * 16 words, `hist` n_rows * 2 * 2048 64-bit words.
+// blocks in every pass.  `any_late`: some row has top-k, top-p and min-p all at once (its
+// second search costs seven launches more; a wrong 0 leaves such a row without top-p).
+// Room: `parts` n_rows * 32 * 4 floats, `kept` n_rows * 32 floats, `state` n_rows * 20
+// words, `hist` n_rows * 2 * 2048 64-bit words.
 extern "C" int hal_sample_spread(const float* logits, int ld, int n_rows, int V,
                                  const float* temperature, const int* top_k, const float* top_p,
                                  const float* min_p, const uint64_t* seeds, const int* draw_index,
-                                 float* parts, float* kept, void* state, void* hist,
+                                 float* parts, float* kept, void* state, void* hist, int any_late,
                                  int* out_token, float* out_logprob, hipStream_t stream) {
   HAL_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "hal_sample_spread: bad sizes rows=%d V=%d ld=%d",
               n_rows, V, ld);
@@ -882,12 +928,18 @@ extern "C" int hal_sample_spread(const float* logits, int ld, int n_rows, int V,
   hipLaunchKernelGGL(row_part_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0, stream, logits,
                      ld, V, temperature, top_k, parts);
   hipLaunchKernelGGL(filt_join_kernel, dim3(n_rows), dim3(HAL_WAVE), 0, stream, parts, temperature,
-                     top_k, top_p, V, rows, h);
-  for (int level = 0; level < 3; ++level) {
-    hipLaunchKernelGGL(filt_hist_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0, stream,
-                       logits, ld, V, temperature, rows, level, h);
-    hipLaunchKernelGGL(filt_find_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, rows, h,
-                       top_p, level);
+                     top_k, top_p, min_p, V, rows, h);
+  // the searches; then, if some row has top-k, top-p and min-p all at once, its second search
+  for (int late = 0; late <= (any_late ? 1 : 0); ++late) {
+    if (late)
+      hipLaunchKernelGGL(filt_kept_by_k_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0,
+                         stream, logits, ld, V, temperature, rows);
+    for (int level = 0; level < 3; ++level) {
+      hipLaunchKernelGGL(filt_hist_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0, stream,
+                         logits, ld, V, temperature, rows, level, late, h);
+      hipLaunchKernelGGL(filt_find_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, rows, h,
+                         top_p, level, late);
+    }
   }
   hipLaunchKernelGGL(filt_mass_kernel, dim3(ROW_PARTS, n_rows), dim3(PART_THREADS), 0, stream, logits,
                      ld, V, temperature, min_p, rows, kept);

@@ -368,13 +368,15 @@ def sample(
     key_scratch: bool = True,
     unfiltered: bool = False,
     spread: bool = False,
+    late: bool = True,
 ):
     """Next token and log-probability of every row of float32 ``logits``.
     ``all_greedy`` promises that no row samples (``temperature`` 0 or ``top_k`` 1 in
     every row), ``unfiltered`` that every row is greedy or draws from its whole
     distribution (no top-k, top-p or min-p): the rows are then spread over many blocks,
-    in two launches.  ``spread`` promises that no row has top-k, top-p and min-p all at
-    once: every pass over a row is then shared by 32 blocks (ten launches).  Otherwise, with
+    in two launches.  ``spread``: every pass over a row is shared by 32 blocks (ten
+    launches; seven more unless ``late`` is false, which promises that no row has top-k,
+    top-p and min-p all at once).  Otherwise, with
     ``key_scratch``, the kernel gets room for one 32-bit key per logit, which its passes
     over a row read instead of deriving it again."""
     lib = library.core_library()
@@ -403,12 +405,12 @@ def sample(
         dev = logits.device
         parts = torch.empty((n, 32, 4), dtype=torch.float32, device=dev)
         kept = torch.empty((n, 32), dtype=torch.float32, device=dev)
-        state = torch.empty((n, 16), dtype=torch.int32, device=dev)
+        state = torch.empty((n, 20), dtype=torch.int32, device=dev)
         hist = torch.empty((n, 2, 2048), dtype=torch.int64, device=dev)
         _check(lib, lib.hal_sample_spread(
             _ptr(logits), vocab, n, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(min_p),
             _ptr(seeds), _ptr(draw_index), _ptr(parts), _ptr(kept), _ptr(state), _ptr(hist),
-            _ptr(tokens), _ptr(logprobs), _stream()))
+            1 if late else 0, _ptr(tokens), _ptr(logprobs), _stream()))
         return tokens, logprobs
     keys = torch.empty((n, vocab), dtype=torch.int32, device=logits.device) if key_scratch and not all_greedy else None
     _check(

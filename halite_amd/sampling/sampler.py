@@ -83,7 +83,7 @@ class Sampler:
         vocab = logits.shape[1]
         unfiltered = all(p.greedy or (not 0 < p.top_k < vocab and p.top_p >= 1.0 and p.min_p <= 0.0) for p in params)
         # top-k, top-p and min-p all at once in one row: top-p then refers to what top-k kept,
-        # two searches one after the other, which only the one-block kernel does
-        spread = not any(not p.greedy and 0 < p.top_k < vocab and p.top_p < 1.0 and p.min_p > 0.0 for p in params)
+        # two searches one after the other
+        late = any(not p.greedy and 0 < p.top_k < vocab and p.top_p < 1.0 and p.min_p > 0.0 for p in params)
         return ops.sample(logits.contiguous(), fd[0], idv[0], fd[1], fd[2], sd, idv[1],
-                          all_greedy=all(p.greedy for p in params), unfiltered=unfiltered, spread=spread)
+                          all_greedy=all(p.greedy for p in params), unfiltered=unfiltered, spread=True, late=late)

@@ -564,9 +564,8 @@ def test_sample_matches_the_plain_sampler(gpu, kw):
     vocab, n = 1000, 400
     base = rnd(1, vocab, seed=81, scale=2.5)[0]
     logits = base[None].repeat(n, 1)
-    both_ways = [_sample(gpu, logits, seed=11, **kw)]
-    if not ("top_k" in kw and "top_p" in kw and "min_p" in kw):  # the rows spread over many blocks
-        both_ways.append(_sample(gpu, logits, seed=11, spread=True, **kw))
+    # one block per row, and the rows spread over many blocks
+    both_ways = [_sample(gpu, logits, seed=11, **kw), _sample(gpu, logits, seed=11, spread=True, **kw)]
     for tok, lp in both_ways:
         _compare_with_plain(base, kw, tok, lp, n)
 
@@ -605,9 +604,7 @@ def test_sample_large_vocabulary(gpu, vocab):
             torch.arange(n, dtype=torch.int32, device=gpu), key_scratch=False,  # the keys are derived again in every pass
         )
         assert torch.equal(tok, tok_again)
-        ways = [(tok, lp)]
-        if not ("top_k" in kw and "top_p" in kw and "min_p" in kw):  # the rows spread over many blocks
-            ways.append(_sample(gpu, logits, seed=5, spread=True, **kw))
+        ways = [(tok, lp), _sample(gpu, logits, seed=5, spread=True, **kw)]  # and spread over many blocks
         for tok, lp in ways:
             agree = 0
             for i in range(n):
