@@ -208,6 +208,8 @@ def main() -> int:
                     help="run the prompt of the prefill measurement in portions of this many tokens (0: whole)")
     ap.add_argument("--steps-ahead", type=int, default=1, choices=[0, 1],
                     help="scheduler workloads: launch decode steps before the tokens of the step before are read")
+    ap.add_argument("--sampling", default="greedy", choices=["greedy", "temperature", "top_p", "top_k", "all"],
+                    help="how the decode steps sample (the contract's line is greedy)")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b"],
                     help="decode8b: the headline line; the others run requests through the scheduler")
     args = ap.parse_args()
@@ -263,7 +265,10 @@ def main() -> int:
                 pos += n
             tok, _ = sampler.forward(logits, [greedy], [0], [0])
             last.append(int(tok[0]))
-        params, seeds, draws = [greedy] * batch, [0] * batch, [0] * batch
+        how = {"greedy": greedy, "temperature": SamplingParams(temperature=0.8),
+               "top_p": SamplingParams(temperature=0.8, top_p=0.9), "top_k": SamplingParams(temperature=0.8, top_k=50),
+               "all": SamplingParams(temperature=0.8, top_k=50, top_p=0.9, min_p=0.05)}[args.sampling]
+        params, seeds, draws = [how] * batch, list(range(batch)), [0] * batch
 
         def one_step(tokens):
             segs = [Segment(s, runner.cache.length(s), [t], [0]) for s, t in zip(slots, tokens)]
@@ -353,6 +358,7 @@ def main() -> int:
             "prefill_tokens": args.prefill_tokens,
             "page_size": runner.cache.page_size,
             "hip_graph": not args.no_graph,
+            "sampling": args.sampling,
             "parallelism": "single GPU",
         },
         "roofline": {
