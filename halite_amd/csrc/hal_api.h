@@ -74,6 +74,18 @@ int hal_sample(const float* logits, int ld, int n_rows, int V, const float* temp
 int hal_sample_greedy(const float* logits, int ld, int n_rows, int V, float* parts,
                       int* out_token, float* out_logprob, hipStream_t stream);
 
+// hal_sample_greedy without any allocation.  This entry point has no counterpart in the
+// reference.  It is for callers that cannot allocate device memory: code under HIP graph
+// capture, tight serving loops, harnesses that forbid hipMalloc.  The partial results go
+// to an array that the library holds on every GPU it runs on (512 KiB, there until the
+// process ends) instead of to `parts`; at most hal_sample_greedy_static_max_rows() (1024)
+// rows, more are refused.  It calls no hipMalloc, hipFree or allocating routine.  All calls
+// on one GPU share that array: calls that may overlap there (other streams, other host
+// threads) race; calls on one stream do not.
+int hal_sample_greedy_static_max_rows();
+int hal_sample_greedy_static(const float* logits, int ld, int n_rows, int V, int* out_token,
+                             float* out_logprob, hipStream_t stream);
+
 // Rows without filters, greedy or drawn from the whole temperature-scaled distribution; each
 // row is spread over 32 blocks.  `parts`: room for n_rows * 32 * 4 floats.
 int hal_sample_unfiltered(const float* logits, int ld, int n_rows, int V, const float* temperature,

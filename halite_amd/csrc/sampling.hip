@@ -10,6 +10,7 @@
 // NaN logits count as -1e5.  src/halite/transformers/infer/engine/sampler.py:17-60
 #include "hal_common.h"
 #include "hal_api.h"
+#include <mutex>
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_BINS 2048  // two per thread
@@ -885,6 +886,58 @@ extern "C" int hal_sample_greedy(const float* logits, int ld, int n_rows, int V,
   HAL_REQUIRE(n_rows <= 65535, "hal_sample_greedy: %d rows exceed the grid limit", n_rows);
   if (n_rows == 0) return 0;
   HAL_REQUIRE(parts != nullptr, "hal_sample_greedy: no room for the partial results");
+  return launch_row_parts(logits, ld, n_rows, V, nullptr, nullptr, nullptr, nullptr, parts, out_token,
+                          out_logprob, stream);
+}
+
+// ---- greedy decoding without any allocation ---------------------------------------------
+// The partial results of hal_sample_greedy in memory that the library itself holds: one
+// array per GPU, there from the moment the library is loaded until the process ends.
+#define STATIC_GREEDY_ROWS 1024
+static __device__ __align__(256) float scratch[STATIC_GREEDY_ROWS * ROW_PARTS * 4];  // 512 KiB
+
+#define STATIC_MAX_DEVICES 64
+static float* g_scratch_of_device[STATIC_MAX_DEVICES];  // the array's address on each GPU
+static std::mutex g_scratch_lock;
+
+// The address of this GPU's copy of `scratch`.  The array's name means nothing to host
+// code; the address is asked for once per device, with that device current.
+static int scratch_of_current_device(float** out) {
+  int dev = -1;
+  HAL_CHECK_HIP(hipGetDevice(&dev));
+  HAL_REQUIRE(dev >= 0 && dev < STATIC_MAX_DEVICES, "hal_sample_greedy_static: device %d of at most %d",
+              dev, STATIC_MAX_DEVICES);
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (g_scratch_of_device[dev] == nullptr) {
+    float* ptr = nullptr;
+    HAL_CHECK_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+    HAL_REQUIRE(ptr != nullptr, "hal_sample_greedy_static: the scratch array has no address on device %d", dev);
+    g_scratch_of_device[dev] = ptr;
+  }
+  *out = g_scratch_of_device[dev];
+  return 0;
+}
+
+extern "C" int hal_sample_greedy_static_max_rows() { return STATIC_GREEDY_ROWS; }
+
+// hal_sample_greedy for callers that cannot allocate: the partial results go to the
+// library's own array on the current GPU instead of to `parts`.  Calls no hipMalloc, no
+// hipFree and no routine that allocates; launches the same two kernels.  Nothing in the
+// array has to start at zero: the first kernel writes every word that the second reads (32
+// shares of every row), so what an earlier call left does no harm.  All calls on a GPU
+// share the array: two calls whose kernels may overlap (different streams, different host
+// threads) race; calls on one stream follow each other and are safe.
+extern "C" int hal_sample_greedy_static(const float* logits, int ld, int n_rows, int V,
+                                        int* out_token, float* out_logprob, hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "hal_sample_greedy_static: bad sizes rows=%d V=%d ld=%d",
+              n_rows, V, ld);
+  HAL_REQUIRE(n_rows <= STATIC_GREEDY_ROWS,
+              "hal_sample_greedy_static: %d rows, the scratch array holds the partial results of at most %d",
+              n_rows, STATIC_GREEDY_ROWS);
+  if (n_rows == 0) return 0;
+  HAL_REQUIRE(logits && out_token && out_logprob, "hal_sample_greedy_static: arguments missing");
+  float* parts = nullptr;
+  if (int rc = scratch_of_current_device(&parts)) return rc;
   return launch_row_parts(logits, ld, n_rows, V, nullptr, nullptr, nullptr, nullptr, parts, out_token,
                           out_logprob, stream);
 }
