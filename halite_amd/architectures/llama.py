@@ -21,10 +21,16 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
         max_positions=cfg.max_position_embeddings,
     )
     if cfg.rope_scaling is not None:
-        rope["scaling"] = cfg.rope_scaling.model_dump()
+        sc = cfg.rope_scaling  # "llama3" is the only type the configuration lets through
+        rope["scaling"] = dict(
+            kind="banded",
+            factor=sc.factor,
+            low_freq_factor=sc.low_freq_factor,
+            high_freq_factor=sc.high_freq_factor,
+            original_context_len=sc.original_max_position_embeddings,
+        )
     norm = PartSpec(kind="rmsnorm", size=cfg.hidden_size, eps=cfg.rms_norm_eps)
-    layer = LayerSpec(
-        arrangement="pre_norm",
+    layer = LayerSpec(arrangement="pre_norm", parts=dict(
         mixer_norm=norm,
         mixer=PartSpec(
             kind="attention",
@@ -45,7 +51,7 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
             intermediate_size=cfg.intermediate_size,
             activation=cfg.hidden_act,
         ),
-    )
+    ))
     names = [str(i) for i in range(cfg.num_hidden_layers)]
     return ModelSpec(
         architecture="LlamaForCausalLM",

@@ -11,6 +11,8 @@ reserved one is free and every slot is free.
 
 from __future__ import annotations
 
+import sys
+
 import numpy as np
 import torch
 
@@ -88,14 +90,24 @@ class CacheManager:
         return (self.num_pages - 1) * self.page_size
 
     def free_pages(self) -> int:
-        """Free pages of the tightest group."""
-        return min((g.pool.available for g in self.groups), default=0)
+        """Free pages of the tightest group; a model without paged layers has no page to
+        run out of, which the largest integer stands for."""
+        return min((g.pool.available for g in self.groups), default=sys.maxsize)
 
     def layer_pages(self, run: int) -> LayerPages | None:
         return self._pages.get(run)
 
     def state_of_run(self, run: int) -> dict[str, torch.Tensor]:
         return self.state.tensors.get(run, {})
+
+    def release_storage(self) -> None:
+        """Drops the device memory of pages and state rows (the bookkeeping stays); the
+        manager serves no step afterwards."""
+        for g in self.groups:
+            g.storage = None
+        for pages in self._pages.values():
+            pages.k = pages.v = None
+        self.state.tensors = {}
 
     # -- requests -----------------------------------------------------------------
     def admit(self) -> int:

@@ -161,6 +161,13 @@ class CacheGroup:
         self.pool.free(held)
         return len(held)
 
+    def tokens_held_at_most(self, n_tokens: float) -> float:
+        """Cache tokens of this group that ``n_tokens`` tokens of one request take at
+        most: all of them, or what a window spans (whole pages, and the one being left)."""
+        if self.need.window is None:
+            return n_tokens
+        return min(n_tokens, (-(-self.need.window // self.page_size) + 1) * self.page_size)
+
     def pages_per_token_span(self, n_tokens: int) -> int:
         """Upper bound of the pages a request of ``n_tokens`` holds at once."""
         if self.need.window is None:

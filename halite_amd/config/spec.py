@@ -30,14 +30,27 @@ class PartSpec(BaseModel):
 
 
 class LayerSpec(BaseModel):
-    """A block: which arrangement and which four parts
-    (src/halite/transformers/block.py:10-85)."""
+    """A block: which arrangement, and the parts that the arrangement asks for, by the
+    names it gives them (src/halite/transformers/block.py:10-85 takes its norms, its
+    attention and its feed-forward as arguments in the same way).  Which names exist, and
+    which of them may be left out, is the arrangement's to say: ``pre_norm`` has
+    ``mixer_norm``, ``mixer``, ``ff_norm`` and ``ff``.  A name the arrangement does not
+    know is an error when the model is built, never dropped."""
+
+    model_config = ConfigDict(extra="forbid")
 
     arrangement: str = "pre_norm"
-    mixer_norm: PartSpec
-    mixer: PartSpec
-    ff_norm: PartSpec
-    ff: PartSpec
+    parts: dict[str, PartSpec]
+
+    @model_validator(mode="before")
+    @classmethod
+    def _parts_as_keywords(cls, data):
+        """``LayerSpec(mixer=..., ff=...)`` stands for ``LayerSpec(parts={"mixer": ..., "ff": ...})``."""
+        if isinstance(data, dict) and "parts" not in data:
+            data = dict(data)
+            head = {"arrangement": data.pop("arrangement")} if "arrangement" in data else {}
+            data = {**head, "parts": data}
+        return data
 
 
 class LayerRun(BaseModel):

@@ -275,6 +275,38 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   }
 }
 
+// ---- the scaling that an RMSNorm left to its reader ----------------------------------------
+// A product has written x = bf16(w * bf16(h)) and, per row, partial sums of h^2 (ss
+// [n_parts][row_width]); the norm's output is x * rsqrt(sum / d + eps).  Readers that
+// cannot scale their own result get the rows from here.  One block per row; the partial
+// sums are added in a fixed order (thread by thread, then lanes, then waves).
+__global__ void __launch_bounds__(256)
+scale_normed_rows_kernel(const bf16_t* __restrict__ x, int ldx, const float* __restrict__ ss,
+                         int n_parts, int row_width, float eps, bf16_t* __restrict__ out, int d) {
+  __shared__ float red[16];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  float sum = 0.f;
+  for (int p = tid; p < n_parts; p += 256) sum += ss[(size_t)p * row_width + row];
+  sum = block_sum(sum, red);
+  const float rstd = rsqrtf(sum / (float)d + eps);
+  for (int c = tid; c < d; c += 256)
+    out[(size_t)row * d + c] = f32_to_bf16(bf16_to_f32(x[(size_t)row * ldx + c]) * rstd);
+}
+
+extern "C" int hal_scale_normed_rows(const void* x, int ldx, const float* ss, int n_parts,
+                                     int row_width, float eps, void* out, int m, int d,
+                                     hipStream_t stream) {
+  HAL_REQUIRE(m >= 0 && d > 0 && ldx >= d && n_parts > 0 && eps > 0.f,
+              "hal_scale_normed_rows: bad sizes m=%d d=%d ldx=%d parts=%d", m, d, ldx, n_parts);
+  HAL_REQUIRE(m <= row_width, "hal_scale_normed_rows: %d rows, sums of squares for %d", m, row_width);
+  if (m == 0) return 0;
+  HAL_REQUIRE(x && ss && out, "hal_scale_normed_rows: arguments missing");
+  hipLaunchKernelGGL(scale_normed_rows_kernel, dim3(m), dim3(256), 0, stream, (const bf16_t*)x, ldx, ss,
+                     n_parts, row_width, eps, (bf16_t*)out, d);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
 // four elements per access; F is a multiple of 4
 template <typename T>
 __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_tokens,

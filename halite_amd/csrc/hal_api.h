@@ -24,6 +24,12 @@ int hal_residual_add(float* h, const void* delta, int dtype, long long n, hipStr
 
 int hal_silu_mul(const void* gu, void* out, int dtype, int n_tokens, int F, hipStream_t stream);
 
+// out [m, d] = bf16(x * rsqrt(sum_p ss[p][row] / d + eps)): the rows of an RMSNorm whose
+// scaling was left to the reader (x = bf16(w * bf16(h)), ss [n_parts, row_width] partial
+// sums of h^2), for a reader that does not scale by itself.
+int hal_scale_normed_rows(const void* x, int ldx, const float* ss, int n_parts, int row_width,
+                          float eps, void* out, int m, int d, hipStream_t stream);
+
 int hal_rope_append(void* qkv, int dtype, int row_stride, const int* positions,
                     const int* token_seg, const int* block_table, int bt_stride,
                     const float* cos_t, const float* sin_t, int table_len, void* k_pages,

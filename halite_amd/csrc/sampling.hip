@@ -110,7 +110,7 @@ sample_kernel(const float* __restrict__ logits, int ld, int V,
       part = part * expf(am.v - z) + 1.f;  // am.v = -inf gives part * 0
       am.v = z;
       am.i = i;
-    } else {
+    } else if (z != -INFINITY) {  // (-inf adds nothing; with am.v still -inf it would add NaN)
       part += expf(z - am.v);
     }
   };

@@ -185,7 +185,7 @@ class StepContext:
     # The plans of the attention kernel are part of the same upload, so they are
     # declared before the first device access.
     def plan_attention(self, group_id: int, n_heads: int, n_kv_heads: int, window: int,
-                       head_dim: int = 128, late=False) -> None:
+                       head_dim: int, late=False) -> None:
         key = (group_id, n_heads // n_kv_heads, window)
         if key in self._plan_host:
             return

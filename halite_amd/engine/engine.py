@@ -82,11 +82,16 @@ class InferenceEngine:
             if getattr(tokenizer, "eos_id", None) is not None:
                 stop.add(tokenizer.eos_id)
             stop.update(getattr(tokenizer, "additional_stop_token_ids", None) or ())
-        self.scheduler = Scheduler(
-            model_runner.cache, self.server_config, self._run_step, model_runner.context_len, stop,
-            vocab_size=model_runner.vocab_size, tokenizer=tokenizer,
-        )
+        self._stop_token_ids = stop
+        self._new_scheduler()
         self.initialized = True
+
+    def _new_scheduler(self):
+        r = self.model_runner
+        self.scheduler = Scheduler(
+            r.cache, self.server_config, self._run_step, r.context_len, self._stop_token_ids,
+            vocab_size=r.vocab_size, tokenizer=self.tokenizer,
+        )
 
     @classmethod
     def from_pretrained(cls, folder: str, server_config: ServerConfig | None = None,
@@ -221,6 +226,8 @@ class InferenceEngine:
         return SamplingParams(**(p or {}))
 
     def infer_batch(self, requests) -> list[InferenceResult]:
+        if not self.initialized:
+            raise RuntimeError("the engine was cleaned up; initialize() it and load weights first")
         requests = self.build_batch_request(requests)
         if not requests:
             return []
@@ -267,10 +274,15 @@ class InferenceEngine:
         return self.scheduler.stats
 
     def initialize(self, capture_graphs: bool = False):
-        """``capture_graphs``: record the decode graphs of every batch size now (the
-        reference does so in its ``initialize``, engine.py:33-41) instead of at the first
-        step of each size."""
-        if capture_graphs:
+        """After ``cleanup``: the cache pool and empty weight tensors are allocated again,
+        and ``load_state_dict`` has to bring the weights before requests are served (the
+        reference's engine is used the same way between the steps of a trainer,
+        engine.py:33-52).  ``capture_graphs``: record the decode graphs of every batch
+        size now (engine.py:33-41 does so) instead of at the first step of each size."""
+        if self.model_runner.released:
+            self.model_runner.restore()
+            self._new_scheduler()
+        if capture_graphs and self.model_runner.has_weights:
             self.model_runner.capture_graphs()
         self.initialized = True
 
@@ -280,5 +292,9 @@ class InferenceEngine:
         self.model_runner.load_state_dict(state_dict)
 
     def cleanup(self):
+        """Frees the cache pool, the captured graphs and the weights (engine.py:43-46 of
+        the reference), so that something else can have the GPU's memory."""
+        self.scheduler.abort_all()
         self.scheduler.initialize()
+        self.model_runner.release()
         self.initialized = False

@@ -94,6 +94,8 @@ class ModelRunner:
         kv_heads = [n.n_kv_heads for n in needs.values()] or [1]
         self._min_kv_heads = min(kv_heads)
         self.graph_replays = 0
+        self.released = False
+        self.has_weights = True  # the model comes filled; restore() gives one that is not
 
     def _size_pool(self, needs, page_size, dtype) -> int:
         tokens = self.server_config.kv_cache_num_tokens
@@ -157,9 +159,49 @@ class ModelRunner:
         dropped."""
         from ..weights import load_state_dict
 
+        if self.released:
+            raise RuntimeError("the runner was released; restore() it before weights are loaded")
         load_state_dict(self.model, self.arch.weight_map(self.config), tensors)
         self._graphs.clear()
         self._ahead = None
+        self.has_weights = True
+
+    def release(self) -> None:
+        """Gives the device memory back: captured graphs, the cache pool and the state
+        rows, the weights and their tiled copies, the position tables (the reference's
+        engine frees its pools and moves the model to the meta device so that a trainer
+        can have the GPU, src/halite/transformers/infer/engine/engine.py:43-46;
+        model_runner.py:241-252).  ``restore`` makes the runner usable again."""
+        if self.released:
+            return
+        if not self.cache.idle():
+            raise RuntimeError("requests are still live; free them before the runner is released")
+        self._graphs.clear()
+        self._ahead = self._token_feed = self._staging = None
+        for run in self.model.runs:
+            run.kv, run.state = None, {}
+        self.cache.release_storage()
+        holders = list(self.model.named_parts().values()) + list(self.model.positions.values())
+        for part in holders:
+            for name, value in list(vars(part).items()):
+                if isinstance(value, torch.Tensor):
+                    setattr(part, name, None)
+        self.released, self.has_weights = True, False
+        gc.collect()
+        if self.device.type == "cuda":
+            torch.cuda.empty_cache()
+
+    def restore(self) -> None:
+        """After ``release``: a cache pool of the configured size again, and the model's
+        tensors allocated but not filled; ``load_state_dict`` brings the weights."""
+        if not self.released:
+            return
+        spec, dtype, tiled = self.model.spec, self.model.dtype, self.model.build.tiled_weights
+        arch, config = getattr(self, "arch", None), getattr(self, "config", None)
+        self.__init__(Decoder(spec, dtype, self.device, tiled), self.server_config, self.model_config)
+        self.has_weights = False
+        if arch is not None:
+            self.arch, self.config = arch, config
 
     # -- requests -------------------------------------------------------------------
     def admit(self) -> int:
@@ -227,6 +269,8 @@ class ModelRunner:
         the host has not read yet).  Every segment then has one token, and
         ``segments[i].tokens[0]`` is not a token id but the row of ``token_feed`` that
         holds it."""
+        if self.released or not self.has_weights:
+            raise RuntimeError("the runner has no weights on the device (released, or restored and not loaded)")
         if not segments:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         if token_feed is not None and any(s.tokens.size != 1 for s in segments):

@@ -193,7 +193,9 @@ class Scheduler:
                 f"request {req.id!r}: prompt {len(req.input_ids)} + max_new_tokens "
                 f"{p.max_new_tokens} exceeds the context length {self.context_len}"
             )
-        if self._pages_for(longest) > min(g.pool.capacity for g in self.cache.groups):
+        # every group of pages must be able to hold the request when it is alone; a model
+        # without paged layers has no such limit
+        if any(g.pages_per_token_span(longest) > g.pool.capacity for g in self.cache.groups):
             raise ValueError(
                 f"request {req.id!r}: {longest} tokens can never fit the cache pool of "
                 f"{self.cache.token_capacity} tokens"
@@ -213,9 +215,6 @@ class Scheduler:
         self.waiting.clear()
         self.running = []
         self.new_token_ratio = self.init_new_token_ratio
-
-    def _pages_for(self, n_tokens: int) -> int:
-        return max(g.pages_per_token_span(n_tokens) for g in self.cache.groups)
 
     # -- one step ---------------------------------------------------------------------
     def _fits(self, spans) -> bool:
@@ -247,6 +246,12 @@ class Scheduler:
         self.waiting.appendleft(req)
         self.stats.retractions += 1
 
+    def _decoded_ahead(self, r: Request) -> int:
+        """The length of a decoding request ``retract_decode_steps`` tokens on (or at its end,
+        if that comes first)."""
+        end = min(len(r.input_ids) + r.sampling_params.max_new_tokens, self.context_len)
+        return max(r.n_cached + 1, min(r.n_cached + self.conf.retract_decode_steps, end))
+
     def _retraction_victim(self, candidates: list[Request]) -> Request:
         # batch.py:468-476: sorted by (generated, -prompt) descending, popped from the end
         return min(candidates, key=lambda r: (len(r.output_ids), -len(r.input_ids)))
@@ -268,13 +273,21 @@ class Scheduler:
         # 1. one token for every decoding request; make room by retraction
         decoding = [r for r in self.running if r.decoding]
         retracted_any = False
-        while decoding and not self._fits([(r.slot, r.n_cached + 1) for r in decoding]):
-            if len(self.running) == 1:
-                raise RuntimeError("No space left for only one request")
-            victim = self._retraction_victim(self.running)
-            self._retract(victim)
-            retracted_any = True
-            decoding = [r for r in decoding if r is not victim]
+        if decoding and not self._fits([(r.slot, r.n_cached + 1) for r in decoding]):
+            # batch.py:468-527: requests give way until those that stay can all decode
+            # ``retract_decode_steps`` more tokens, not just this one, so that the next steps
+            # do not retract again (every retraction runs a whole prompt anew)
+            while True:
+                if len(self.running) == 1:
+                    if not self._fits([(r.slot, r.n_cached + 1) for r in decoding]):
+                        raise RuntimeError("No space left for only one request")
+                    break
+                victim = self._retraction_victim(self.running)
+                self._retract(victim)
+                retracted_any = True
+                decoding = [r for r in decoding if r is not victim]
+                if self._fits([(r.slot, self._decoded_ahead(r)) for r in decoding]):
+                    break
         if retracted_any:
             self.new_token_ratio = self._ratio_after_retraction()
         elif decoding:
@@ -301,18 +314,28 @@ class Scheduler:
 
         # 3. admission, first come first served (scheduler.py:211-265)
         if not retracted_any and self.waiting and budget > 0:
-            free_tokens = self.cache.free_pages() * self.cache.page_size
-            remaining_total = free_tokens - sum(
-                min(r.sampling_params.max_new_tokens - len(r.output_ids), CLIP_MAX_NEW_TOKENS)
-                * self.new_token_ratio
-                + (r.remaining if not r.decoding else 0)
-                for r in self.running
-            )
+            # One budget of cache tokens per group of pages (the reference has one pool):
+            # what is free, less what the running requests are expected to take.  A group
+            # with a window never holds more of a request than the window spans.  Without
+            # any group (no paged layer) only the slots limit admission.
+            groups = self.cache.groups
+            remaining_total = [
+                g.pool.available * g.page_size
+                - sum(
+                    g.tokens_held_at_most(
+                        min(r.sampling_params.max_new_tokens - len(r.output_ids), CLIP_MAX_NEW_TOKENS)
+                        * self.new_token_ratio
+                        + (r.remaining if not r.decoding else 0)
+                    )
+                    for r in self.running
+                )
+                for g in groups
+            ]
             while self.waiting and budget > 0 and self.cache.slots.available > 0:
                 r = self.waiting[0]
                 new_tokens = min(r.sampling_params.max_new_tokens - len(r.output_ids), CLIP_MAX_NEW_TOKENS)
-                need = r.n_total + new_tokens
-                if need > remaining_total and self.running:
+                need = [g.tokens_held_at_most(r.n_total + new_tokens) for g in groups]
+                if any(n > left for n, left in zip(need, remaining_total)) and self.running:
                     break  # AddRequestResult.NO_TOKEN
                 r.slot = self.cache.admit()
                 r.n_cached = 0
@@ -323,7 +346,7 @@ class Scheduler:
                     break
                 self.waiting.popleft()
                 self.running.append(r)
-                remaining_total -= need
+                remaining_total = [left - n for left, n in zip(remaining_total, need)]
                 entries.append((r, k))
                 spans.append((r.slot, r.n_cached + k))
                 budget -= k

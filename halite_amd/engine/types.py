@@ -13,7 +13,9 @@ class InferenceRequest(NamedTuple):
 
 
 class InferenceResult:
-    """One entry per sample of the request (``n`` of them)."""
+    """One entry per sample of the request (``n`` of them).  The class restates the
+    reference's result type (infer/types.py:15-64: the same fields, ``validate_lengths``
+    and ``to_dict``), so that code written against that engine reads results unchanged."""
 
     def __init__(self, id, input_ids=None, output_ids=None, output_logprobs=None,
                  finish_reason=None, num_cached_prompt_tokens=None):

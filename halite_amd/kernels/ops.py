@@ -55,9 +55,16 @@ class NormedRows:
 
     def materialize(self) -> torch.Tensor:
         """The norm's output as a tensor, for a reader that does not scale by itself."""
-        m, d = self.x.shape
-        rstd = torch.rsqrt(self.ss_parts.sum(0)[:m] / d + self.eps)
-        return (self.x.float() * rstd[:, None]).to(self.x.dtype)
+        lib = library.core_library()
+        x, ss = self.x, self.ss_parts
+        _dev(ss)
+        _need(x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1, "normed rows are bf16 rows")
+        _need(ss.dtype == torch.float32 and ss.dim() == 2, "sums of squares are float32 [parts, rows]")
+        m, d = x.shape
+        out = torch.empty((m, d), dtype=torch.bfloat16, device=x.device)
+        _check(lib, lib.hal_scale_normed_rows(
+            _ptr(x), x.stride(0), _ptr(ss), ss.shape[0], ss.shape[1], ctypes.c_float(self.eps), _ptr(out), m, d, _stream()))
+        return out
 
 
 def dtype_code(dtype: torch.dtype) -> int:

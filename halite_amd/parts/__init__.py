@@ -7,6 +7,7 @@ from .base import (
     MIXERS,
     NORMS,
     POSITIONS,
+    Arrangement,
     BuildContext,
     Embedding,
     FeedForward,
@@ -17,6 +18,7 @@ from .base import (
     ParamDecl,
     Part,
     PositionEncoding,
+    RotaryPositionEncoding,
     RunBinding,
     StateNeed,
     register_arrangement,
@@ -25,7 +27,7 @@ from .decoder import Decoder
 
 __all__ = [
     "ARRANGEMENTS", "EMBEDDINGS", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITIONS",
-    "BuildContext", "Decoder", "Embedding", "FeedForward", "Head", "Mixer", "Norm",
-    "PagedKVNeed", "ParamDecl", "Part", "PositionEncoding", "RunBinding", "StateNeed",
+    "Arrangement", "BuildContext", "Decoder", "Embedding", "FeedForward", "Head", "Mixer", "Norm",
+    "PagedKVNeed", "ParamDecl", "Part", "PositionEncoding", "RotaryPositionEncoding", "RunBinding", "StateNeed",
     "register_arrangement",
 ]

@@ -8,7 +8,7 @@ from pydantic import BaseModel, Field, StrictInt, model_validator
 
 from ..kernels import attention as attention_kernels
 from ..kernels import ops
-from .base import MIXERS, Mixer, PagedKVNeed, ParamDecl
+from .base import MIXERS, Mixer, PagedKVNeed, ParamDecl, RotaryPositionEncoding
 
 
 class AttentionParams(BaseModel):
@@ -46,8 +46,13 @@ class Attention(Mixer):
             if params.position not in build.positions:
                 raise ValueError(f"attention names position encoding {params.position!r}, which the model does not define")
             self.position = build.positions[params.position]
-            if self.position.p.head_dim != params.head_dim:
-                raise ValueError("position encoding and attention disagree on head_dim")
+            if not isinstance(self.position, RotaryPositionEncoding):
+                raise ValueError(
+                    f"attention rotates queries and keys; position encoding {params.position!r} "
+                    f"({type(self.position).__name__}) is not a RotaryPositionEncoding"
+                )
+            if self.position.rotary_dim > params.head_dim:
+                raise ValueError("the position encoding rotates more elements than a head has")
 
     def param_decls(self):
         p = self.p

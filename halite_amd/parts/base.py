@@ -160,7 +160,27 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    pass
+    """Says where a token is.  What a position encoding offers is for the mixers that name it
+    to use; the one contract the framework's own mixers know is ``RotaryPositionEncoding``."""
+
+
+class RotaryPositionEncoding(PositionEncoding):
+    """A position encoding that is applied by rotating pairs of the first ``rotary_dim``
+    elements of every query and key head: pairs ``(j, j + rotary_dim/2)``, or neighbours
+    ``(2j, 2j + 1)`` if ``interleaved``."""
+
+    @property
+    def rotary_dim(self) -> int:
+        raise NotImplementedError
+
+    @property
+    def interleaved(self) -> bool:
+        raise NotImplementedError
+
+    def tables(self, n_positions: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+        """float32 ``(cos, sin)``, each ``[at least n_positions, rotary_dim / 2]``, on the
+        device; row ``p`` holds the angles of position ``p``."""
+        raise NotImplementedError
 
 
 class Embedding(Part):
@@ -204,7 +224,47 @@ NORMS = Registry("norm")
 POSITIONS = Registry("position encoding")
 EMBEDDINGS = Registry("embedding")
 HEADS = Registry("head")
-ARRANGEMENTS: dict[str, type] = {}
+class Arrangement:
+    """The order in which a layer's parts act on the residual stream.
+
+    ``roles``: name of a part -> the registry its kind is looked up in; ``optional``:
+    names that a layer may leave out (the arrangement then finds ``None`` under them).
+    ``forward(h, pending, ctx, run)`` gets the float32 stream ``h`` [tokens, width], a
+    delta ``pending`` that the block before has not added yet (or ``None``), the step and
+    the run's binding; it adds into ``h`` what it adds and returns the delta it leaves to
+    whoever comes next (or ``None``).  Every arrangement has a part named ``mixer``."""
+
+    roles: ClassVar[dict[str, "Registry"]] = {}
+    optional: ClassVar[tuple[str, ...]] = ()
+
+    def __init__(self, parts: dict[str, Part | None]):
+        self._parts = dict(parts)
+        self.mixer = parts["mixer"]
+
+    def parts(self) -> dict[str, Part]:
+        """The parts that exist, by name (their tensors are ``layers.<layer>.<name>.*``)."""
+        return {name: part for name, part in self._parts.items() if part is not None}
+
+    def forward(self, h, pending, ctx, run):
+        raise NotImplementedError
+
+    @classmethod
+    def build(cls, kind: str, specs: dict[str, PartSpec], build: BuildContext) -> "Arrangement":
+        if "mixer" not in cls.roles:
+            raise ConfigError(f"arrangement {kind!r} declares no part named 'mixer'")
+        unknown = sorted(set(specs) - set(cls.roles))
+        missing = sorted(set(cls.roles) - set(specs) - set(cls.optional))
+        if unknown or missing:
+            raise ConfigError(
+                f"arrangement {kind!r} is made of {sorted(cls.roles)}"
+                + (f"; it has no part named {unknown}" if unknown else "")
+                + (f"; the layer leaves out {missing}" if missing else "")
+            )
+        return cls({name: (reg.build(specs[name], build) if name in specs else None)
+                    for name, reg in cls.roles.items()})
+
+
+ARRANGEMENTS: dict[str, type[Arrangement]] = {}
 
 
 def register_arrangement(kind: str):

@@ -1,12 +1,20 @@
-"""How the parts of a layer are arranged (src/halite/transformers/block.py:10-85)."""
+"""How the parts of a layer are arranged (src/halite/transformers/block.py:10-85).
+
+An arrangement says which parts it is made of, by name and by kind of part
+(``roles``), which of them may be left out (``optional``), and how a step's tokens
+go through them.  The builder makes the parts that the layer's description names,
+refuses names that the arrangement does not have, and hands the arrangement a dict.
+One part of every arrangement is its ``mixer``: the part that may own a cache and
+per-request state, which the step function binds to every run of the layer.
+"""
 
 from __future__ import annotations
 
-from .base import register_arrangement
+from .base import FEED_FORWARDS, MIXERS, NORMS, Arrangement, register_arrangement
 
 
 @register_arrangement("pre_norm")
-class PreNormBlock:
+class PreNormBlock(Arrangement):
     """``h = h + mixer(norm(h)); h = h + ff(norm(h))`` (block.py:56-74).
 
     The residual stream ``h`` is float32.  Each add is done by the norm that
@@ -14,18 +22,12 @@ class PreNormBlock:
     norm (or to the model's final norm) instead of adding it itself.
     """
 
+    roles = {"mixer_norm": NORMS, "mixer": MIXERS, "ff_norm": NORMS, "ff": FEED_FORWARDS}
     takes_next_norm = True  # forward() accepts next_norm=
 
-    def __init__(self, mixer_norm, mixer, ff_norm, ff):
-        self.mixer_norm, self.mixer, self.ff_norm, self.ff = mixer_norm, mixer, ff_norm, ff
-
-    def parts(self):
-        return {
-            "mixer_norm": self.mixer_norm,
-            "mixer": self.mixer,
-            "ff_norm": self.ff_norm,
-            "ff": self.ff,
-        }
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.mixer_norm, self.ff_norm, self.ff = parts["mixer_norm"], parts["ff_norm"], parts["ff"]
 
     # The norm between two parts can be folded into the products around it where the part
     # before it offers that and the part after it takes such rows.

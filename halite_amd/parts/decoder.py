@@ -16,9 +16,7 @@ from ..config.spec import ModelSpec
 from .base import (
     ARRANGEMENTS,
     EMBEDDINGS,
-    FEED_FORWARDS,
     HEADS,
-    MIXERS,
     NORMS,
     POSITIONS,
     BuildContext,
@@ -58,12 +56,7 @@ class Decoder:
             if lspec.arrangement not in ARRANGEMENTS:
                 known = ", ".join(sorted(ARRANGEMENTS))
                 raise ConfigError(f"unknown arrangement {lspec.arrangement!r}; known: {known}")
-            self.layers[name] = ARRANGEMENTS[lspec.arrangement](
-                NORMS.build(lspec.mixer_norm, build),
-                MIXERS.build(lspec.mixer, build),
-                NORMS.build(lspec.ff_norm, build),
-                FEED_FORWARDS.build(lspec.ff, build),
-            )
+            self.layers[name] = ARRANGEMENTS[lspec.arrangement].build(lspec.arrangement, lspec.parts, build)
         self.final_norm = NORMS.build(spec.final_norm, build)
         self.head = HEADS.build(spec.head, build)
         self.runs = [

@@ -6,10 +6,32 @@ from __future__ import annotations
 import math
 
 import torch
-from pydantic import BaseModel, Field, StrictBool, StrictInt, model_validator
+from typing import Literal
 
-from ..config.model import Llama3RopeScaling
-from .base import POSITIONS, PositionEncoding
+from pydantic import BaseModel, ConfigDict, Field, StrictBool, StrictInt, model_validator
+
+from .base import POSITIONS, RotaryPositionEncoding
+
+
+class BandedFrequencyScaling(BaseModel):
+    """The frequency scaling of position.py:242-284, in the part's own terms: wavelengths
+    longer than ``original_context_len / low_freq_factor`` are stretched by ``factor``,
+    those shorter than ``original_context_len / high_freq_factor`` are kept, the band
+    between is blended.  An architecture's description translates its own keys into these."""
+
+    model_config = ConfigDict(extra="forbid")
+
+    kind: Literal["banded"]
+    factor: float = Field(gt=0)
+    low_freq_factor: float
+    high_freq_factor: float
+    original_context_len: StrictInt = Field(gt=0)
+
+    @model_validator(mode="after")
+    def _check(self):
+        if self.high_freq_factor == self.low_freq_factor:
+            raise ValueError("frequency scaling: high_freq_factor equals low_freq_factor")
+        return self
 
 
 class RopeParams(BaseModel):
@@ -18,7 +40,7 @@ class RopeParams(BaseModel):
     theta: float = Field(gt=0)
     interleaved: StrictBool = False
     max_positions: StrictInt = Field(gt=0)
-    scaling: Llama3RopeScaling | None = None
+    scaling: BandedFrequencyScaling | None = None
 
     @model_validator(mode="after")
     def _check(self):
@@ -38,11 +60,11 @@ def rope_inverse_frequencies(p: RopeParams) -> torch.Tensor:
     s = p.scaling
     if s is None:
         return inv_freq
-    long_wavelen = s.original_max_position_embeddings / s.low_freq_factor
-    short_wavelen = s.original_max_position_embeddings / s.high_freq_factor
+    long_wavelen = s.original_context_len / s.low_freq_factor
+    short_wavelen = s.original_context_len / s.high_freq_factor
     wavelen = 2 * math.pi / inv_freq
     stretched = torch.where(wavelen > long_wavelen, inv_freq / s.factor, inv_freq)
-    blend = (s.original_max_position_embeddings / wavelen - s.low_freq_factor) / (
+    blend = (s.original_context_len / wavelen - s.low_freq_factor) / (
         s.high_freq_factor - s.low_freq_factor
     )
     blended = (1 - blend) * stretched / s.factor + blend * stretched
@@ -51,7 +73,7 @@ def rope_inverse_frequencies(p: RopeParams) -> torch.Tensor:
 
 
 @POSITIONS.register("rope")
-class Rope(PositionEncoding):
+class Rope(RotaryPositionEncoding):
     """Holds the float32 ``cos``/``sin`` table ``[positions, rotary_dim/2]`` on the
     device (position.py:140-167: outer product of float32 positions and
     frequencies).  The rotation itself happens in the kernel that also appends

@@ -133,7 +133,8 @@ def _fill(model: Decoder, weight_table: dict[str, str], files, folder: str) -> N
         passed_over = {k for k, v in weight_table.items() if v is None}
         unexpected = sorted(have - known - passed_over)
         if missing or unexpected or wrong_shape or wrong_dtype:
-            raise WeightError(folder, missing, unexpected, wrong_shape, wrong_dtype)
+            raise WeightError(folder, missing, unexpected, wrong_shape, wrong_dtype,
+                              other=getattr(files, "notes", ()))
 
         parts = {id(s.part): s.part for s in slots}
         views = {}

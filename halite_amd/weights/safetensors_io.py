@@ -106,7 +106,9 @@ class ModelFiles:
         index = os.path.join(folder, "model.safetensors.index.json")
         self.files: list[SafetensorsFile] = []
         self.where: dict[str, SafetensorsFile] = {}
+        self.notes: list[str] = []  # where the index and the shards disagree
         problems = []
+        shard_of = {}
         if os.path.isfile(single):
             paths = [single]
         elif os.path.isfile(index):
@@ -123,11 +125,16 @@ class ModelFiles:
             raise SafetensorsError(f"{folder}: no model.safetensors and no model.safetensors.index.json")
         if problems:
             raise SafetensorsError(f"{folder}: " + "; ".join(problems))
+        by_file = {}
         for p in paths:
             sf = SafetensorsFile(p)
             self.files.append(sf)
+            by_file[os.path.basename(p)] = sf
             for name in sf.names():
                 self.where[name] = sf
+        for name, shard in shard_of.items():
+            if name not in by_file[shard].names():
+                self.notes.append(f"the index lists {name} in {shard}, which does not hold it")
 
     def names(self):
         return list(self.where)

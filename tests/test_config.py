@@ -106,7 +106,8 @@ def test_spec_is_data():
     arch, cfg = parse_config(tiny.TINY_B)
     spec = arch.to_spec(cfg)
     assert [r.layer for r in spec.order] == ["0", "1", "2"]
-    att = spec.layers["1"].mixer
+    assert sorted(spec.layers["1"].parts) == ["ff", "ff_norm", "mixer", "mixer_norm"]
+    att = spec.layers["1"].parts["mixer"]
     assert att.kind == "attention" and att.params()["n_kv_heads"] == 1 and att.params()["head_dim"] == 32
     assert abs(att.params()["scale"] - 32**-0.5) < 1e-12
     assert spec.positions["rope"].params()["scaling"]["factor"] == 8.0
@@ -122,6 +123,37 @@ def test_spec_is_data():
     bad["order"][0]["layer"] = "nope"
     with pytest.raises(ValueError, match="unknown layer"):
         ModelSpec(**bad)
+
+
+def test_a_layer_names_the_parts_its_arrangement_has():
+    import torch
+
+    from halite_amd.config.registry import ConfigError
+    from halite_amd.parts import Decoder
+
+    arch, cfg = parse_config(tiny.TINY_A)
+    spec = arch.to_spec(cfg)
+    Decoder(spec, torch.float32, "cpu")  # builds
+    norm = spec.layers["0"].parts["ff_norm"]
+    # a part that the arrangement does not have is refused, not dropped
+    extra = spec.model_copy(deep=True)
+    extra.layers["1"].parts["post_norm"] = norm
+    with pytest.raises(ConfigError, match=r"no part named \['post_norm'\]"):
+        Decoder(extra, torch.float32, "cpu")
+    # and so is a layer that leaves one out
+    short = spec.model_copy(deep=True)
+    del short.layers["0"].parts["ff_norm"]
+    with pytest.raises(ConfigError, match=r"leaves out \['ff_norm'\]"):
+        Decoder(short, torch.float32, "cpu")
+    other = spec.model_copy(deep=True)
+    other.layers["0"].arrangement = "post_norm"
+    with pytest.raises(ConfigError, match="unknown arrangement 'post_norm'; known: pre_norm"):
+        Decoder(other, torch.float32, "cpu")
+    # the keyword form and the dict form are the same description
+    from halite_amd.config import LayerSpec
+
+    parts = spec.layers["0"].parts
+    assert LayerSpec(**parts) == LayerSpec(arrangement="pre_norm", parts=parts) == spec.layers["0"]
 
 
 def test_weight_map_names():

@@ -125,7 +125,10 @@ def test_portions_retraction_and_page_reuse_keep_the_tokens(models):
         ModelConfig(dtype="float32"),
     )
     got = tight.infer_batch([(i, p, params) for i, p in enumerate(prompts)])
-    assert tight.stats.retractions > 0
+    # requests are thrown out, but with headroom: a handful of times, not once a step
+    assert 0 < tight.stats.retractions <= 8, tight.stats.retractions
+    rerun = tight.stats.prefill_tokens - sum(len(p) for p in prompts)
+    assert rerun <= 4 * sum(len(p) + 40 for p in prompts) // 3
     assert max(tight.stats.tokens_per_step) <= 24
     assert [r.output_ids[0] for r in got] == want
     assert tight.model_runner.cache.idle()
@@ -195,6 +198,38 @@ def test_new_weights_for_a_running_engine(models, tmp_path):
     with pytest.raises(WeightError, match="model.norm.weight") as err:
         engine.load_state_dict(broken)
     assert "extra.weight" in str(err.value)
+
+
+def test_cleanup_gives_the_memory_back_and_initialize_brings_the_engine_back(models):
+    """``cleanup`` frees pool, graphs and weights (a second engine of the same size fits in
+    what came back); ``initialize`` and ``load_state_dict`` make the first one serve again,
+    with the same tokens."""
+    folder, pc, pw = models[("B", "bfloat16")]
+    server = ServerConfig(kv_cache_num_tokens=65536, use_cudagraph=True)
+    prompt = tiny.random_tokens(tiny.TINY_B, 20, 7)
+    params = {"max_new_tokens": 12, "temperature": 0.0}
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    engine = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="bfloat16"))
+    before = engine.infer_batch([(prompt, params)])[0].output_ids[0]
+    held = torch.cuda.memory_allocated() - base
+    pool = engine.model_runner.cache.groups[0].storage
+    assert held >= pool.numel() * pool.element_size() > 20e6
+    del pool
+    engine.cleanup()
+    left = torch.cuda.memory_allocated() - base
+    assert left < 0.02 * held, f"{left} of {held} bytes are still held after cleanup"
+    with pytest.raises(RuntimeError, match="cleaned up"):
+        engine.infer_batch([(prompt, params)])
+    other = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="bfloat16"))
+    assert other.infer_batch([(prompt, params)])[0].output_ids[0] == before
+    other.cleanup()
+    engine.initialize()
+    with pytest.raises(RuntimeError, match="no weights"):
+        engine.infer_batch([(prompt, params)])
+    engine.load_state_dict(pw)
+    assert engine.infer_batch([(prompt, params)])[0].output_ids[0] == before
+    assert engine.model_runner.graph_replays > 0
 
 
 def test_command_line(models, tmp_path):

@@ -285,6 +285,9 @@ def test_norm_folded_into_the_products_around_it(gpu, M, d, F, wdt):
     close(rows.ss_parts.sum(0)[:M], (h_ref.double() ** 2).sum(1), 1e-5, "sums of squares")
     assert float(rows.ss_parts[:, M:].abs().sum()) == 0
     close(rows.materialize(), y, 1.2e-2, "rows made whole")
+    scaled = rows.x.float() * torch.rsqrt(rows.ss_parts.double().sum(0)[:M] / d + eps).float()[:, None]
+    off = (rows.materialize().float() - scaled.to(dt).float()).abs() / scaled.abs().clamp_min(1e-6)
+    assert float(off.max()) <= 2 ** -7, "rows made whole: more than one bf16 step from x * rstd"
     got_plain = ops.gemm_bf16_skinny_norm(rows, t2, (F, d))
     got_gated = ops.gemm_bf16_skinny_norm(rows, t2, (F, d), w_up_tiled=t3)
     close(got_plain, plain_out, 1.5e-2, "plain product after the folded norm")
@@ -666,6 +669,30 @@ def test_sample_rows_that_hold_nothing(gpu):
                             f(1.0, torch.float32), f(0.0, torch.float32), f(7, torch.int64), f(0, torch.int32),
                             unfiltered=True, all_greedy=kw.get("temperature") == 0.0)
         assert all(0 <= int(t) < vocab for t in tok) and int(tok[3]) == 0
+
+
+def test_sample_logprob_of_a_row_that_starts_with_minus_infinity(gpu):
+    """-inf logits seen before any finite one (a thread's first logit is -inf, a later one
+    of the same thread is finite): the sum of the exponentials stays finite and the
+    log-probability is the plain softmax's, in the one-block kernel and in the spread ones."""
+    vocab = 6000
+    logits = torch.full((3, vocab), float("-inf"))
+    logits[0, 4096] = 1.0  # thread 0 sees index 0 (-inf) first, then this one
+    logits[0, 5000] = 2.0
+    logits[1, :7] = float("-inf")
+    logits[1, 7:] = rnd(1, vocab - 7, seed=9)[0]
+    logits[2] = rnd(1, vocab, seed=10)[0]
+    logits[2, ::2] = float("-inf")
+    ref = torch.log_softmax(logits.double(), dim=-1)
+    for kw in ({"temperature": 0.0}, {}, {"top_k": 50}):
+        for spread in (False, True):
+            tok, lp = (t.cpu() for t in _sample(gpu, logits, spread=spread, **kw))
+            assert torch.isfinite(lp).all(), (kw, spread, lp.tolist())
+            if kw.get("temperature") == 0.0:
+                assert tok.tolist() == ref.argmax(-1).tolist()
+            if "top_k" not in kw:
+                want = ref.gather(1, tok.long()[:, None])[:, 0]
+                assert torch.allclose(lp.double(), want, atol=1e-4), (kw, spread)
 
 
 def test_sample_rows_are_independent(gpu):

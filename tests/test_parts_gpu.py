@@ -14,7 +14,7 @@ from halite_amd.config import LayerRun, LayerSpec, ModelConfig, ModelSpec, PartS
 from halite_amd.engine.batch import Segment
 from halite_amd.engine.runner import ModelRunner
 from halite_amd.parts import MIXERS, BuildContext, Decoder, Mixer, ParamDecl, StateNeed
-from halite_amd.parts.base import FEED_FORWARDS, NORMS, POSITIONS, FeedForward, PositionEncoding, register_arrangement
+from halite_amd.parts.base import FEED_FORWARDS, NORMS, POSITIONS, Arrangement, FeedForward, PositionEncoding, register_arrangement
 from halite_amd.weights import fill_random
 
 pytestmark = pytest.mark.gpu
@@ -151,12 +151,44 @@ def plain_model(model, ids, mixers: dict, ffs: dict | None = None):
     memo = {}
     for i, run in enumerate(spec.order):
         blk = model.layers[run.layer]
-        x = P.rms_norm(h, blk.mixer_norm.weight.float().cpu(), blk.mixer_norm.p.eps)
+        parts = blk.parts()
+        if isinstance(blk, SandwichBlock):
+            h = plain_sandwich(parts, h, lambda x: mixers[run.layer](blk.mixer, x, positions, i, run, memo))
+            continue
+        x = P.rms_norm(h, parts["mixer_norm"].weight.float().cpu(), parts["mixer_norm"].p.eps)
         h = h + mixers[run.layer](blk.mixer, x, positions, i, run, memo)
-        x = P.rms_norm(h, blk.ff_norm.weight.float().cpu(), blk.ff_norm.p.eps)
-        h = h + (ffs or {}).get(run.layer, plain_gated)(blk.ff, x)
+        x = P.rms_norm(h, parts["ff_norm"].weight.float().cpu(), parts["ff_norm"].p.eps)
+        h = h + (ffs or {}).get(run.layer, plain_gated)(parts["ff"], x)
     h = P.rms_norm(h, model.final_norm.weight.float().cpu(), model.final_norm.p.eps)
     return P.output_head(h, model.embedding.weight.float().cpu())
+
+
+@register_arrangement("toy_sandwich")
+class SandwichBlock(Arrangement):
+    """Norms on both sides of the mixer, and a feed-forward that a layer may leave out:
+    ``h += post_norm(mixer(pre_norm(h)))`` and then, if there is one, ``h += ff(ff_norm(h))``.
+    Another set of parts than ``pre_norm`` has, under names of its own."""
+
+    roles = {"pre_norm": NORMS, "mixer": MIXERS, "post_norm": NORMS, "ff_norm": NORMS, "ff": FEED_FORWARDS}
+    optional = ("ff_norm", "ff")
+
+    def forward(self, h, pending, ctx, run):
+        p = self.parts()
+        x = p["pre_norm"].forward(h, delta=pending)
+        a = p["mixer"].forward(x, ctx, run)
+        a = p["post_norm"].forward(a.float())  # a norm of the mixer's output, not of the stream
+        if "ff" not in p:
+            return a
+        x = p["ff_norm"].forward(h, delta=a)
+        return p["ff"].forward(x, ctx)
+
+
+def plain_sandwich(parts, h, mixer):
+    norm = lambda name, x: P.rms_norm(x, parts[name].weight.float().cpu(), parts[name].p.eps)  # noqa: E731
+    h = h + norm("post_norm", mixer(norm("pre_norm", h)))
+    if "ff" in parts:
+        h = h + plain_gated(parts["ff"], norm("ff_norm", h))
+    return h
 
 
 def replay_all(runner, requests, ref, tol, vocab):
@@ -386,7 +418,8 @@ def test_toy_routing_and_other_position_encodings(gpu, dtype):
         ffs={"b": PartSpec(kind="toy_routed", hidden_size=64, n_experts=3, expert_size=40)},
     )
     runner = make_runner(gpu, spec, dtype)
-    assert isinstance(runner.model.layers["b"].ff, ToyRouted) and not isinstance(runner.model.layers["a"].ff, ToyRouted)
+    assert isinstance(runner.model.layers["b"].parts()["ff"], ToyRouted)
+    assert not isinstance(runner.model.layers["a"].parts()["ff"], ToyRouted)
 
     def att_with(rope_p):
         return lambda part, x, positions, i, run, memo: plain_attention_layer(part, x, positions, rope_p)[0]
@@ -407,23 +440,20 @@ def test_toy_routing_and_other_position_encodings(gpu, dtype):
 
 
 @register_arrangement("pre_norm_plain_test")
-class PlainPreNorm:
+class PlainPreNorm(Arrangement):
     """The same arithmetic as ``pre_norm`` through the plain interface: four parts, tensors
     in, a tensor out, no word about the block before or after."""
 
-    def __init__(self, mixer_norm, mixer, ff_norm, ff):
-        self.mixer_norm, self.mixer, self.ff_norm, self.ff = mixer_norm, mixer, ff_norm, ff
-
-    def parts(self):
-        return {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "ff_norm": self.ff_norm, "ff": self.ff}
+    roles = {"mixer_norm": NORMS, "mixer": MIXERS, "ff_norm": NORMS, "ff": FEED_FORWARDS}
 
     def forward(self, h, pending, ctx, run):
-        x = self.mixer_norm.forward(h, delta=pending)
+        p = self.parts()
+        x = p["mixer_norm"].forward(h, delta=pending)
         assert isinstance(x, torch.Tensor) and (pending is None or isinstance(pending, torch.Tensor))
-        a = self.mixer.forward(x, ctx, run)
-        x = self.ff_norm.forward(h, delta=a)
+        a = p["mixer"].forward(x, ctx, run)
+        x = p["ff_norm"].forward(h, delta=a)
         assert isinstance(a, torch.Tensor) and isinstance(x, torch.Tensor)
-        return self.ff.forward(x, ctx)
+        return p["ff"].forward(x, ctx)
 
 
 def test_a_plain_arrangement_between_blocks_that_fold_their_norms(gpu):
@@ -442,3 +472,108 @@ def test_a_plain_arrangement_between_blocks_that_fold_their_norms(gpu):
     requests = {f"r{i}": [int(t) % 97 for t in tiny.random_tokens(tiny.TINY_A, n, 60 + i)] for i, n in enumerate([50, 3, 35])}
     ref = {rid: plain_model(runner.model, toks, {"a": att, "b": att, "c": att}) for rid, toks in requests.items()}
     replay_all(runner, requests, ref, TOL["bfloat16"], 97)
+
+
+# -- another set of parts in a block ----------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_an_arrangement_with_other_parts_is_registered_from_here(gpu, dtype):
+    """A block with norms before and after its mixer, once with and once without a
+    feed-forward, between two ``pre_norm`` blocks: described as data, built and stepped
+    with no change to the framework."""
+    rope_p = dict(rotary_dim=16, theta=10000.0, interleaved=False)
+    spec = toy_spec({"a": attention_spec(), "s": attention_spec(heads=2, kv=1), "t": attention_spec(kv=4)},
+                    [LayerRun(layer="a"), LayerRun(layer="s"), LayerRun(layer="t"), LayerRun(layer="a")])
+    norm = spec.final_norm
+    spec.layers["s"] = LayerSpec(arrangement="toy_sandwich", parts=dict(
+        pre_norm=norm, mixer=spec.layers["s"].parts["mixer"], post_norm=norm, ff_norm=norm, ff=spec.layers["s"].parts["ff"]))
+    spec.layers["t"] = LayerSpec(arrangement="toy_sandwich", parts=dict(
+        pre_norm=norm, mixer=spec.layers["t"].parts["mixer"], post_norm=norm))
+    spec = ModelSpec(**spec.model_dump())  # the description is data
+    runner = make_runner(gpu, spec, dtype)
+    assert sorted(runner.model.layers["t"].parts()) == ["mixer", "post_norm", "pre_norm"]
+    names = {s.path for s in runner.model.param_slots()}
+    assert "layers.s.post_norm.weight" in names and "layers.t.ff.linear_out.weight" not in names
+
+    def att(part, x, positions, i, run, memo):
+        return plain_attention_layer(part, x, positions, rope_p)[0]
+
+    requests = {f"r{i}": [int(t) % 97 for t in tiny.random_tokens(tiny.TINY_A, n, 70 + i)] for i, n in enumerate([50, 3, 35])}
+    ref = {rid: plain_model(runner.model, toks, {"a": att, "s": att, "t": att}) for rid, toks in requests.items()}
+    replay_all(runner, requests, ref, TOL[dtype], 97)
+    with pytest.raises(Exception, match=r"leaves out \['post_norm'\]"):
+        bad = spec.model_copy(deep=True)
+        del bad.layers["t"].parts["post_norm"]
+        Decoder(bad, DT[dtype], gpu)
+
+
+# -- toy models under the scheduler ------------------------------------------------------------
+
+
+def greedy_with_plain_model(model, mixers, prompt, n_new):
+    ids, out = list(prompt), []
+    for _ in range(n_new):
+        t = int(torch.argmax(plain_model(model, ids, mixers)[-1]))
+        out.append(t)
+        ids.append(t)
+    return out
+
+
+@pytest.mark.parametrize("ahead", [0, 1])
+def test_the_scheduler_serves_a_model_without_paged_layers(gpu, ahead):
+    """Every layer keeps state of fixed size and none keeps keys: no group of pages exists,
+    slots are the only limit, prompts are cut into portions and requests wait for a slot."""
+    from halite_amd.engine import InferenceEngine
+
+    spec = toy_spec({"m": PartSpec(kind="running_mean", hidden_size=64), "n": PartSpec(kind="running_mean", hidden_size=64)},
+                    [LayerRun(layer="m"), LayerRun(layer="n"), LayerRun(layer="m")])
+    model = Decoder(spec, torch.float32, gpu)
+    fill_random(model, seed=5, std=0.08)
+    runner = ModelRunner(model, ServerConfig(page_size=16, max_seqs_per_forward=2, max_tokens_per_forward=16,
+                                             chunked_prefill_size=7, scheduling_steps_ahead=ahead), ModelConfig(dtype="float32"))
+    assert runner.cache.groups == []
+    engine = InferenceEngine(runner)
+
+    def mean(part, x, positions, i, run, memo):
+        return (torch.cumsum(x, 0) / torch.arange(1, x.shape[0] + 1)[:, None]) @ part.w_weight.float().cpu().T
+
+    prompts = [[int(t) % 97 for t in tiny.random_tokens(tiny.TINY_A, n, 30 + n)] for n in (23, 2, 9, 40)]
+    results = engine.infer_batch([(i, p, {"max_new_tokens": 6, "temperature": 0.0}) for i, p in enumerate(prompts)])
+    for r, p in zip(results, prompts):
+        assert r.output_ids[0] == greedy_with_plain_model(model, {"m": mean, "n": mean}, p, 6)
+    st = engine.stats
+    assert st.max_running == 2 and st.retractions == 0 and max(st.tokens_per_step) <= 16
+    assert runner.cache.idle()
+
+
+@pytest.mark.parametrize("ahead", [0, 1])
+def test_the_scheduler_serves_two_groups_of_pages_and_retracts(gpu, ahead):
+    """Layers with a window beside layers with all keys, each kind with pages of its own, and
+    so few pages that requests are retracted: the tokens are those of the plain model, and
+    the retractions come in bursts with headroom, not one per step."""
+    from halite_amd.engine import InferenceEngine
+
+    rope_p = dict(rotary_dim=16, theta=10000.0, interleaved=False)
+    spec = toy_spec({"w": attention_spec(window=12), "f": attention_spec(kv=1)},
+                    [LayerRun(layer="w"), LayerRun(layer="f"), LayerRun(layer="w")])
+    model = Decoder(spec, torch.float32, gpu)
+    fill_random(model, seed=6, std=0.08)
+    runner = ModelRunner(model, ServerConfig(kv_cache_num_tokens=152, page_size=8, max_seqs_per_forward=8,
+                                             max_tokens_per_forward=24, chunked_prefill_size=10,
+                                             default_init_new_token_ratio=0.05, retract_decode_steps=6,
+                                             scheduling_steps_ahead=ahead), ModelConfig(dtype="float32"))
+    assert len(runner.cache.groups) == 2
+    engine = InferenceEngine(runner)
+
+    def att(part, x, positions, i, run, memo):
+        return plain_attention_layer(part, x, positions, rope_p)[0]
+
+    prompts = [[int(t) % 97 for t in tiny.random_tokens(tiny.TINY_A, n, 50 + n)] for n in (21, 5, 13, 30)]
+    results = engine.infer_batch([(i, p, {"max_new_tokens": 24, "temperature": 0.0}) for i, p in enumerate(prompts)])
+    for r, p in zip(results, prompts):
+        assert r.output_ids[0] == greedy_with_plain_model(model, {"w": att, "f": att}, p, 24)
+    st = engine.stats
+    assert 0 < st.retractions <= 6, st.retractions
+    assert runner.cache.idle()
+    runner.cache.check()

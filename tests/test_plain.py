@@ -37,6 +37,47 @@ def test_llama3_scaling_bands():
     assert torch.allclose(P.llama3_scaled_frequencies(f, 1.0, 1.0, 4.0, 64), f, rtol=1e-6)
 
 
+def test_llama3_scaling_meets_both_bands_at_their_edges():
+    # What fixes the blend beside the reference's text: the scaled frequency is a
+    # continuous function of the frequency.  On a dense sweep over all three bands the
+    # ratio scaled/unscaled is 1 where wavelengths are short, 1/factor where they are
+    # long, rises from the one to the other in between and meets both at the edges.  A
+    # blend with its two weights swapped jumps by the factor at each edge; one that is
+    # linear in the wavelength instead of the frequency is off in the middle.
+    orig, factor, lo, hi = 8192, 8.0, 1.0, 4.0
+    f_low_edge, f_high_edge = 2 * math.pi * lo / orig, 2 * math.pi * hi / orig
+    f = torch.logspace(math.log10(f_low_edge / 30), math.log10(f_high_edge * 30), 4001, dtype=torch.float64).float()
+    ratio = (P.llama3_scaled_frequencies(f, factor, lo, hi, orig) / f).double()
+    fd = f.double()
+    short, long_ = fd > f_high_edge * 1.0001, fd < f_low_edge * 0.9999
+    mid = (fd > f_low_edge * 1.0001) & (fd < f_high_edge * 0.9999)
+    assert short.sum() > 500 and long_.sum() > 500 and mid.sum() > 500
+    assert torch.allclose(ratio[short], torch.ones_like(ratio[short]), atol=1e-6)
+    assert torch.allclose(ratio[long_], torch.full_like(ratio[long_], 1 / factor), atol=1e-6)
+    assert (ratio[1:] >= ratio[:-1] - 1e-6).all()  # never falls as the frequency rises
+    assert ((ratio[mid] > 1 / factor) & (ratio[mid] < 1)).all()
+    step = (ratio[1:] - ratio[:-1]).abs().max()
+    assert step < 5e-3, f"the ratio jumps by {step} between neighbours of a dense sweep"
+    # half-way between the edges in frequency, the ratio is half-way between 1/factor and 1
+    middle = torch.tensor([(f_low_edge + f_high_edge) / 2], dtype=torch.float32)
+    got = float(P.llama3_scaled_frequencies(middle, factor, lo, hi, orig) / middle)
+    assert abs(got - (1 / factor + 1) / 2) < 1e-5
+
+
+def test_llama3_scaling_of_the_8b_head():
+    # head size 128 at the 8B's constants: six frequencies fall between the bands, so a
+    # blend with swapped weights is no longer decreasing along the head
+    f = P.inverse_frequencies(128, 500000.0)
+    g = P.llama3_scaled_frequencies(f, 8.0, 1.0, 4.0, 8192)
+    wl = 2 * math.pi / f
+    mid = ~(wl < 8192 / 4.0) & ~(wl > 8192 / 1.0)
+    assert int(mid.sum()) == 6
+    assert (g[:-1] > g[1:]).all()
+    assert ((g[mid] < f[mid]) & (g[mid] > f[mid] / 8.0)).all()
+    s = (8192 * f[mid].double() / (2 * math.pi) - 1.0) / 3.0  # position between the edges, in frequency
+    assert torch.allclose(g[mid].double() / f[mid].double(), (1 - s) / 8.0 + s, rtol=1e-5)
+
+
 def test_llama3_scaling_matches_two_where_form():
     # the reference's vectorised form (src/halite/transformers/position.py:264-284)
     f = P.inverse_frequencies(64, 500000.0)

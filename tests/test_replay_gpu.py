@@ -91,6 +91,25 @@ def test_bfloat16_run_of_a_folder_stored_in_float32(folders):
     replay.compare(rows, ref, TOL["bfloat16"])
 
 
+def test_a_reader_that_does_not_scale_gets_whole_rows(folders, monkeypatch):
+    """Where the product before a norm has prepared its rows but the part after cannot
+    finish the norm in its own product (a gated feed-forward too large at 17 to 32 rows:
+    forced here by the threshold), the rows are made whole by a kernel of their own, and
+    the logits are those of the plain implementation."""
+    from halite_amd.kernels import ops
+
+    made = []
+    whole = ops.NormedRows.materialize
+    monkeypatch.setattr(ops.NormedRows, "materialize", lambda self: made.append(self.shape[0]) or whole(self))
+    monkeypatch.setattr(ops, "GATED_MID_ELEMENTS", 0)
+    folder, requests, ref = folders[("B", "bfloat16")]
+    trace = replay.portions({"r2": requests["r2"], "r4": requests["r4"]}, sizes=(20, 31, 17, 24, 32, 19))
+    runner = make_runner(folder, "bfloat16", replay.peak_tokens(trace))
+    rows = replay.collect(trace, replay.run_trace(runner, trace), 512)
+    replay.compare(rows, ref, TOL["bfloat16"])
+    assert made and all(17 <= m <= 32 for m in made)
+
+
 def test_steps_of_few_tokens_take_the_fused_kernels(folders, monkeypatch):
     """With the tiled weight copy a bf16 step of at most 32 tokens runs rotation and append
     inside the q, k, v product and every norm but the first and the last inside the

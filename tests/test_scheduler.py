@@ -266,3 +266,95 @@ def test_stop_strings():
     assert done[1].output_ids == full[:first]
     assert done[2].output_ids == full and done[2].finished_reason.reason == "length"
     assert cache.idle()
+
+
+def _tight_pool_run(retract_decode_steps):
+    """16 short requests that together outgrow a pool of 399 one-token pages.  Returns the
+    prompts, the scheduler, the finished requests and the number of steps that retracted."""
+    ps = prompts([4 + i % 5 for i in range(16)])
+    sched, model, cache = make(num_pages=400, page_size=1, n_slots=16, max_tokens_per_forward=256,
+                               default_init_new_token_ratio=0.05, retract_decode_steps=retract_decode_steps)
+    for i, p in enumerate(ps):
+        sched.add_request(Request(i, p, SamplingParams(max_new_tokens=60, ignore_eos=True)))
+    done, events, seen = {}, 0, 0
+    while True:
+        out = sched.step()
+        if out is None:
+            break
+        done.update({r.id: r for r in out})
+        if sched.stats.retractions != seen:
+            events, seen = events + 1, sched.stats.retractions
+    sched.check_idle()
+    cache.check()
+    return ps, sched, done, events
+
+
+def test_retraction_leaves_headroom_so_that_the_next_steps_do_not_retract_again():
+    # infer/engine/batch.py:478-481: requests give way until those that stay can decode
+    # retract_decode_steps more tokens.  Making room for the step at hand only (which a
+    # headroom of one step amounts to) has to retract again a step or two later, and the
+    # request that went is run anew each time it is let in again.
+    ps, sched, done, events = _tight_pool_run(20)
+    _, short_sched, short_done, short_events = _tight_pool_run(1)
+    for i, p in enumerate(ps):
+        assert done[i].output_ids == expected(p, 60) == short_done[i].output_ids
+    assert 0 < events <= 3, events
+    assert short_events >= 3 * events
+    assert sched.stats.retractions <= 12
+    rerun = sched.stats.prefill_tokens - sum(len(p) for p in ps)
+    short_rerun = short_sched.stats.prefill_tokens - sum(len(p) for p in ps)
+    assert 0 < rerun < short_rerun
+    assert rerun <= 320  # 302 as measured; one retraction per step re-runs 369
+
+
+def test_a_model_without_paged_layers_is_limited_by_slots_only():
+    from halite_amd.parts.base import StateNeed
+
+    cache = CacheManager({}, {}, {0: {"mean": StateNeed((4,))}}, page_size=4, num_pages=2, n_slots=3, allocate=False)
+    model = FakeModel(cache)
+    sched = Scheduler(cache, ServerConfig(page_size=4, max_seqs_per_forward=3, max_tokens_per_forward=16,
+                                          chunked_prefill_size=8), model, context_len=512)
+    ps = prompts([30, 5, 17, 9, 2])
+    for i, p in enumerate(ps):
+        sched.add_request(Request(i, p, SamplingParams(max_new_tokens=10, ignore_eos=True)))
+    done = {r.id: r for r in sched.run_to_completion()}
+    assert len(done) == 5 and sched.stats.retractions == 0 and sched.stats.max_running == 3
+    for i, p in enumerate(ps):
+        assert done[i].output_ids == expected(p, 10)
+    for plan in model.plans:
+        assert sum(k for _, k, _ in plan) <= 16 and all(k <= 8 for _, k, _ in plan)
+    sched.check_idle()
+    cache.check()
+
+
+def test_two_groups_one_with_a_window():
+    # layers with all keys and layers with a window of 6 have pages of their own; the
+    # group without a window is the one that runs out
+    needs = {0: PagedKVNeed(1, 8), 1: PagedKVNeed(1, 8, window=6), 2: PagedKVNeed(1, 8)}
+    ps = prompts([14, 9, 11, 6])
+    want = [expected(p, 40) for p in ps]
+
+    def run(num_pages):
+        cache = CacheManager(needs, page_size=4, num_pages=num_pages, n_slots=8, allocate=False)
+        assert len(cache.groups) == 2
+        model = FakeModel(cache)
+        sched = Scheduler(cache, ServerConfig(page_size=4, max_seqs_per_forward=8, max_tokens_per_forward=32,
+                                              default_init_new_token_ratio=0.05), model, context_len=512)
+        for i, p in enumerate(ps):
+            sched.add_request(Request(i, p, SamplingParams(max_new_tokens=40, ignore_eos=True)))
+        done = {r.id: r for r in sched.run_to_completion()}
+        for i in range(4):
+            assert done[i].output_ids == want[i]
+        sched.check_idle()
+        cache.check()
+        return sched
+
+    roomy = run(200)
+    assert roomy.stats.retractions == 0 and roomy.stats.max_running == 4
+    tight = run(31)
+    assert tight.stats.retractions > 0
+    # a request that the windowed group could hold but the other could not is refused
+    cache = CacheManager(needs, page_size=4, num_pages=5, n_slots=8, allocate=False)
+    sched = Scheduler(cache, ServerConfig(page_size=4), FakeModel(cache), context_len=512)
+    with pytest.raises(ValueError, match="can never fit"):
+        sched.add_request(Request(0, list(range(10)), SamplingParams(max_new_tokens=20)))

@@ -161,3 +161,63 @@ def test_random_mode_writes_a_loadable_folder(tmp_path, raw):
     assert torch.equal(model.embedding.weight, fa.tensor("model.embed_tokens.weight"))
     for f in (fa, fb, fc):
         f.close()
+
+
+def _two_shards(folder, raw, w, drop_from_shard=None):
+    """The folder's tensors in two files and an index, as large models are stored."""
+    from safetensors.torch import save_file as pkg_save
+
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(raw, f)
+    names = list(w)
+    first = {n: w[n].contiguous() for n in names[::2]}
+    second = {n: w[n].contiguous() for n in names[1::2]}
+    index = {"metadata": {}, "weight_map": {**{n: "model-00001-of-00002.safetensors" for n in first},
+                                            **{n: "model-00002-of-00002.safetensors" for n in second}}}
+    if drop_from_shard is not None:
+        first.pop(drop_from_shard, None), second.pop(drop_from_shard, None)
+    pkg_save(first, os.path.join(folder, "model-00001-of-00002.safetensors"))
+    pkg_save(second, os.path.join(folder, "model-00002-of-00002.safetensors"))
+    with open(os.path.join(folder, "model.safetensors.index.json"), "w") as f:
+        json.dump(index, f)
+
+
+def test_a_folder_of_shards_loads_like_the_single_file(tmp_path):
+    raw = tiny.TINY_A
+    w = tiny.random_weights(raw, 4)
+    one, two = str(tmp_path / "one"), str(tmp_path / "two")
+    tiny.write_model_folder(one, raw, w)
+    _two_shards(two, raw, w)
+    arch, cfg, a = _model(raw)
+    _, _, b = _model(raw)
+    load_weights(a, arch.weight_map(cfg), one)
+    load_weights(b, arch.weight_map(cfg), two)
+    assert [s.path for s in a.param_slots()] == [s.path for s in b.param_slots()]
+    for pa, pb in zip(a.named_parts().values(), b.named_parts().values()):
+        for name in pa.param_decls():
+            ta, tb = (getattr(p, name.replace(".", "_"), None) for p in (pa, pb))
+            if ta is not None:
+                assert torch.equal(ta, tb)
+    assert torch.equal(a.layers["1"].mixer.w_qkv, b.layers["1"].mixer.w_qkv)
+    assert torch.equal(a.layers["0"].parts()["ff"].w_gate_up, b.layers["0"].parts()["ff"].w_gate_up)
+    assert torch.equal(a.head.weight, w["lm_head.weight"])
+
+
+def test_a_missing_shard_and_a_tensor_missing_from_its_shard_are_named(tmp_path):
+    raw = tiny.TINY_A
+    w = tiny.random_weights(raw, 4)
+    arch, cfg, model = _model(raw)
+    gone = str(tmp_path / "gone")
+    _two_shards(gone, raw, w)
+    os.remove(os.path.join(gone, "model-00002-of-00002.safetensors"))
+    with pytest.raises(WeightError, match="missing shard file model-00002-of-00002.safetensors"):
+        load_weights(model, arch.weight_map(cfg), gone)
+    lacks = str(tmp_path / "lacks")
+    _two_shards(lacks, raw, w, drop_from_shard="model.layers.1.mlp.up_proj.weight")
+    with pytest.raises(WeightError) as e:
+        load_weights(model, arch.weight_map(cfg), lacks)
+    assert e.value.missing == ["model.layers.1.mlp.up_proj.weight"]
+    assert "the index lists model.layers.1.mlp.up_proj.weight in model-0000" in str(e.value)
+    with pytest.raises(WeightError, match="no model.safetensors and no model.safetensors.index.json"):
+        load_weights(model, arch.weight_map(cfg), str(tmp_path / "nothing"))
