@@ -7,7 +7,11 @@ The default run decodes a batch of 8 requests whose contexts end at the configur
 context length (8,192 tokens); a step is one decode step of the engine: building the
 batch, the forward pass from the paged cache, greedy sampling and reading the tokens
 back.  The same line carries the prefill of one 2,048-token prompt, the decode step's
-fraction of the HBM roofline, and decode rates at batch 1 and 64.
+fraction of the HBM roofline, decode rates at batch 1 and 64 (contexts that end at 8,192
+and 512-token prompts), the host's share of a step, what the kernel families of a step
+reach against their rooflines (HIP events around each call of an eager step), and what
+this GPU gives a plain copy and a large library product (the attainable figures beside
+the published peaks).  ``--more-points`` adds further batches, contexts and prompt lengths.
 """
 
 from __future__ import annotations
@@ -86,6 +90,99 @@ def prefill_flops(c, n_layers, t) -> float:
     attention = 2.0 * t * t * c.num_attention_heads * c.head_dim * n_layers
     head = 2.0 * c.vocab_size * c.hidden_size
     return linear + attention + head
+
+
+class Families:
+    """HIP events around every call of the kernel wrappers, by family, for one eager step.
+    A call inside another measured call (a product that picks its kernel) counts once."""
+
+    GEMM = ("linear", "gemm_bf16_skinny", "gemm_bf16_skinny_norm", "qkv_rope_append", "gemm_f32")
+    ELEMENTWISE = ("rmsnorm", "silu_mul", "rope_append", "embedding", "residual_add")
+
+    def __init__(self):
+        self.spans = []
+        self.depth = 0
+        self.saved = []
+
+    def _wrap(self, owner, name, family):
+        import torch
+
+        fn = getattr(owner, name)
+        self.saved.append((owner, name, fn))
+
+        def timed(*a, **kw):
+            if self.depth:
+                return fn(*a, **kw)
+            self.depth += 1
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            try:
+                return fn(*a, **kw)
+            finally:
+                end.record()
+                self.depth -= 1
+                self.spans.append((family, start, end))
+
+        setattr(owner, name, timed)
+
+    def __enter__(self):
+        from halite_amd.kernels import attention as attention_kernels
+        from halite_amd.kernels import ops
+
+        for name in self.GEMM:
+            self._wrap(ops, name, "gemm")
+        for name in self.ELEMENTWISE:
+            self._wrap(ops, name, "elementwise")
+        self._wrap(attention_kernels, "paged_attention", "attention")
+        return self
+
+    def __exit__(self, *exc):
+        for owner, name, fn in reversed(self.saved):
+            setattr(owner, name, fn)
+        self.saved = []
+
+    def totals_ms(self) -> dict:
+        import torch
+
+        torch.cuda.synchronize()
+        out = {}
+        for family, start, end in self.spans:
+            out[family] = out.get(family, 0.0) + start.elapsed_time(end)
+        return out
+
+
+def probe_gpu(torch) -> dict:
+    """What this GPU gives the simplest streaming kernel and a large library product: a
+    copy of 2 GiB (bytes read plus bytes written over time), a read of 2 GiB, and an
+    8192^3 bf16 product.  The rooflines above use the published peaks; these are the
+    attainable ones."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.int16, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+
+    def best(fn, reps=5):
+        times = []
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            times.append(a.elapsed_time(b) * 1e-3)
+        return min(times[1:])
+
+    t_copy = best(lambda: dst.copy_(src))
+    t_read = best(lambda: torch.max(src.view(torch.int32)))
+    del dst
+    m = 8192
+    a = torch.randn((m, m), dtype=torch.bfloat16, device="cuda")
+    b = torch.randn((m, m), dtype=torch.bfloat16, device="cuda")
+    t_mm = best(lambda: torch.mm(a, b.t()))
+    return {
+        "copy_gbps": round(2 * 2 * n / t_copy / 1e9, 1),
+        "read_gbps": round(2 * n / t_read / 1e9, 1),
+        "gemm_8192_tflops": round(2.0 * m**3 / t_mm / 1e12, 1),
+    }
 
 
 def engine_workload(args) -> int:
@@ -200,6 +297,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=None, help="context length at the end of decoding")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration (named in the record)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--more-points", action="store_true",
+                    help="further batches (16, 32, 128), contexts (32,768 and 131,072) and prompts (8,192 and 16,384)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the prefill (for profiles)")
@@ -235,13 +334,17 @@ def main() -> int:
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     if args.prefill_only:
         batches, context = [1], max(4096, args.prefill_tokens + 64)
-    pool_tokens = max(batches) * (context + 64) + 4096
+    # (batch, context at the end of decoding) of every point beyond the headline
+    more = [(16, context), (32, context), (128, context), (8, 32768), (1, 131072)] if args.more_points else []
+    pool_tokens = max([b * (context + 64) for b in batches] + [b * (c + 64) for b, c in more]) + 4096
+    longest = max([context] + [c for _, c in more] + ([16384 + 64] if args.more_points else []))
     runner = ModelRunner.from_random(
         cfg, seed=0,
-        server_config=ServerConfig(kv_cache_num_tokens=pool_tokens, max_seqs_per_forward=max(batches) + 1,
+        server_config=ServerConfig(kv_cache_num_tokens=pool_tokens,
+                                   max_seqs_per_forward=max(batches + [b for b, _ in more]) + 1,
                                    max_tokens_per_forward=16384, use_cudagraph=not args.no_graph,
-                                   cudagraph_max_batch_size=max(batches)),
-        model_config=ModelConfig(dtype=args.dtype, context_len=context),
+                                   cudagraph_max_batch_size=max(batches + [b for b, _ in more])),
+        model_config=ModelConfig(dtype=args.dtype, context_len=longest),
     )
     sampler = Sampler(runner.device)
     greedy = SamplingParams(temperature=0.0)
@@ -250,10 +353,12 @@ def main() -> int:
     def sync():
         torch.cuda.synchronize()
 
-    def decode_run(batch: int, steps: int, warmup: int):
-        """Prefills ``batch`` prompts so that the contexts end at ``context`` after
-        the last timed step, then times ``steps`` decode steps."""
-        prompt_len = context - steps - warmup
+    def decode_run(batch: int, steps: int, warmup: int, end_context: int = context, families: bool = False):
+        """Prefills ``batch`` prompts so that the contexts end at ``end_context`` after
+        the last timed step, then times ``steps`` decode steps.  Returns the seconds, the
+        mean number of cached tokens of a step, the GPU's share of the time (events around
+        every step) and, if asked for, the families' times of one more, eager step."""
+        prompt_len = end_context - steps - warmup - (2 if families else 0)
         slots = [runner.admit() for _ in range(batch)]
         last = []
         for s in slots:
@@ -269,11 +374,18 @@ def main() -> int:
                "top_p": SamplingParams(temperature=0.8, top_p=0.9), "top_k": SamplingParams(temperature=0.8, top_k=50),
                "all": SamplingParams(temperature=0.8, top_k=50, top_p=0.9, min_p=0.05)}[args.sampling]
         params, seeds, draws = [how] * batch, list(range(batch)), [0] * batch
+        marks = []
 
-        def one_step(tokens):
+        def one_step(tokens, mark=False):
+            if mark:
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
             segs = [Segment(s, runner.cache.length(s), [t], [0]) for s, t in zip(slots, tokens)]
             logits = runner.step(segs)
             toks, _ = sampler.forward(logits, params, seeds, draws)
+            if mark:
+                b.record()
+                marks.append((a, b))
             return toks.tolist()
 
         for _ in range(warmup):
@@ -281,20 +393,36 @@ def main() -> int:
         sync()
         t0 = time.perf_counter()
         for _ in range(steps):
-            last = one_step(last)
+            last = one_step(last, mark=True)
         sync()
         dt = time.perf_counter() - t0
+        gpu_s = sum(a.elapsed_time(b) for a, b in marks) * 1e-3
         kv_tokens = sum(runner.cache.length(s) for s in slots) - batch * steps / 2.0
+        fam = None
+        if families:
+            # one more step, eager (every kernel launched from the host), with events
+            # around every call of a kernel wrapper
+            graph, runner.server_config.use_cudagraph = runner.server_config.use_cudagraph, False
+            try:
+                last = one_step(last)  # the eager path's first call (allocations, library loads)
+                with Families() as f:
+                    one_step(last)
+                fam = f.totals_ms()
+            finally:
+                runner.server_config.use_cudagraph = graph
         for s in slots:
             runner.free(s)
-        return dt, kv_tokens
+        return dt, kv_tokens, gpu_s, fam
 
-    def prefill_run(T=args.prefill_tokens):
+    def prefill_run(T=args.prefill_tokens, families: bool = False):
         ids = torch.randint(0, cfg.vocab_size, (T,), generator=gen).numpy().astype(np.int32)
-        times = []
-        for i in range(4):
+        times, fam = [], None
+        for i in range(5 if families else 4):
             s = runner.admit()
             sync()
+            measure = Families() if (families and i == 4) else None
+            if measure:
+                measure.__enter__()
             t0 = time.perf_counter()
             portion = args.prefill_portion or T
             for start in range(0, T, portion):  # the whole prompt, or one portion a step
@@ -303,31 +431,49 @@ def main() -> int:
             tok, _ = sampler.forward(logits, [greedy], [0], [0])
             tok.tolist()
             sync()
-            times.append(time.perf_counter() - t0)
+            if measure:
+                measure.__exit__()
+                fam = measure.totals_ms()
+            else:
+                times.append(time.perf_counter() - t0)
             runner.free(s)
         t = min(times[1:])
         peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
-        return {
+        out = {
             "value": round(T / t, 1),
             "tokens": T,
             "ms": round(t * 1e3, 3),
             "frac": round(prefill_flops(cfg, n_layers, T) / t / peak, 4),
         }
+        if fam:
+            linear = 2.0 * T * n_layers * (layer_params(cfg) - 2 * cfg.hidden_size) + 2.0 * cfg.vocab_size * cfg.hidden_size
+            attention = 2.0 * T * T * cfg.num_attention_heads * cfg.head_dim * n_layers
+            out["gemm_ms"] = round(fam.get("gemm", 0.0), 3)
+            out["gemm_frac"] = round(linear / (fam["gemm"] * 1e-3) / peak, 4) if fam.get("gemm") else None
+            out["attention_ms"] = round(fam.get("attention", 0.0), 3)
+            out["attention_frac"] = round(attention / (fam["attention"] * 1e-3) / peak, 4) if fam.get("attention") else None
+            out["elementwise_ms"] = round(fam.get("elementwise", 0.0), 3)
+        return out
 
     if args.prefill_only:
-        print(json.dumps({"metric": "prefill tokens per second", "layers": n_layers, "prefill": prefill_run()}), flush=True)
+        print(json.dumps({"metric": "prefill tokens per second", "layers": n_layers,
+                          "prefill": prefill_run(families=True)}), flush=True)
         return 0
 
     # -- the headline: batch 8 -------------------------------------------------------
     results = {}
     for b in batches:
         steps = args.steps if b == args.batch else max(8, args.steps // 2)
-        dt, kv_tokens = decode_run(b, steps, args.warmup)
-        results[b] = (b * steps / dt, dt / steps, kv_tokens, steps)
-        print(f"[bench] decode batch {b}: {results[b][0]:.1f} tok/s, {results[b][1] * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
-    value, step_s, kv_tokens, _ = results[args.batch]
+        results[b] = (steps, *decode_run(b, steps, args.warmup, families=(b == args.batch)))
+        print(f"[bench] decode batch {b}: {b * steps / results[b][1]:.1f} tok/s, "
+              f"{results[b][1] / steps * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    steps, dt, kv_tokens, gpu_s, fam = results[args.batch]
+    value, step_s = args.batch * steps / dt, dt / steps
     need = decode_bytes(cfg, n_layers, args.batch, kv_tokens, elt)
     achieved = need / step_s
+
+    def frac_of(batch, end_context, n_steps, seconds, cached):
+        return round(decode_bytes(cfg, n_layers, batch, cached, elt) / (seconds / n_steps) / HBM_BYTES_PER_S, 4)
 
     record = {
         "metric": f"decode tokens per second (Llama-3.1-8B shape, batch {args.batch}, context {context})",
@@ -368,11 +514,54 @@ def main() -> int:
             "unit": "GB/s",
             "frac": round(achieved / HBM_BYTES_PER_S, 4),
         },
+        # the step's wall time against the time the GPU works on it (events around every step)
+        "host": {"wall_ms": round(step_s * 1e3, 4), "gpu_ms": round(gpu_s / steps * 1e3, 4),
+                 "share": round(max(0.0, 1.0 - gpu_s / dt), 4)},
     }
+    if fam:
+        # one eager step with events around every kernel wrapper: the weight stream of the
+        # products and the cache stream of attention, each against 8 TB/s
+        weights = decode_bytes(cfg, n_layers, args.batch, 0, elt)
+        cache = need - weights
+        record["families"] = {
+            "gemm": {"ms": round(fam.get("gemm", 0.0), 3), "frac": round(weights / (fam["gemm"] * 1e-3) / HBM_BYTES_PER_S, 4)},
+            "attention": {"ms": round(fam.get("attention", 0.0), 3),
+                          "frac": round(cache / (fam["attention"] * 1e-3) / HBM_BYTES_PER_S, 4)},
+            "elementwise": {"ms": round(fam.get("elementwise", 0.0), 3)},
+            "how": "one eager step, HIP events around each call",
+        }
 
     if not args.no_points:
-        record["points"] = {f"decode_b{b}": round(results[b][0], 2) for b in (1, 64) if b in results}
-        record["prefill"] = prefill_run()
+        points = {}
+        for b in (1, 64):
+            if b in results:
+                n_steps, seconds, cached, _, _ = results[b]
+                points[f"decode_b{b}"] = round(b * n_steps / seconds, 2)
+                points[f"decode_b{b}_frac"] = frac_of(b, context, n_steps, seconds, cached)
+        # BASELINE's other reading of the decode points: 512-token prompts
+        for b in (1, 8, 64):
+            n_steps = max(8, args.steps // 2)
+            seconds, cached, _, _ = decode_run(b, n_steps, args.warmup, end_context=512 + n_steps + args.warmup)
+            points[f"decode_p512_b{b}"] = round(b * n_steps / seconds, 2)
+            points[f"decode_p512_b{b}_frac"] = frac_of(b, 0, n_steps, seconds, cached)
+        for b, c in more:
+            n_steps = max(8, args.steps // 4)
+            seconds, cached, _, _ = decode_run(b, n_steps, 4, end_context=c)
+            points[f"decode_b{b}_ctx{c}"] = round(b * n_steps / seconds, 2)
+            points[f"decode_b{b}_ctx{c}_frac"] = frac_of(b, c, n_steps, seconds, cached)
+            print(f"[bench] decode batch {b} context {c}: {points[f'decode_b{b}_ctx{c}']} tok/s", file=sys.stderr, flush=True)
+        record["points"] = points
+        record["prefill"] = prefill_run(families=True)
+        if args.more_points:
+            for T in (8192, 16384):
+                extra = prefill_run(T)
+                points[f"prefill_{T}"] = extra["value"]
+                points[f"prefill_{T}_frac"] = extra["frac"]
+        record["probe"] = probe_gpu(torch)
+        record["roofline"]["frac_of_measured_read"] = round(achieved / (record["probe"]["read_gbps"] * 1e9), 4)
+        record["prefill"]["frac_of_measured_gemm"] = round(
+            prefill_flops(cfg, n_layers, record["prefill"]["tokens"]) / (record["prefill"]["ms"] * 1e-3)
+            / (record["probe"]["gemm_8192_tflops"] * 1e12), 4)
     print(json.dumps(record), flush=True)
     return 0
 

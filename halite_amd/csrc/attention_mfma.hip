@@ -23,7 +23,14 @@
 // item per wave, nothing goes through LDS, and the key range of a long request is cut
 // into many items.  Prompt portions run four items per workgroup (up to RT_BIG tiles
 // each): the waves walk the union of their key ranges together and load each block of
-// keys and values once, into LDS, one block ahead.
+// keys and values once, into LDS, one block ahead.  Such a workgroup has eight waves in two
+// halves: both halves hold the same four items, the first takes the even steps of the key
+// walk and the second the odd ones (so the causal work splits evenly), each with LDS
+// buffers of its own, and at the end the second half hands its sums to the first through
+// LDS, where they are joined by the log-sum-exp rule.  A workgroup then has a CU to itself
+// and is done in half the time, and since the host lists the longest walks first the
+// workgroups that start late are the short ones: a single prompt of 2,048 tokens, whose
+// 512 items of very different length used to start all at once, is balanced that way.
 //
 // The pages are read in one of three ways: pages in the kernel's fragment order (TILED:
 // one contiguous KB per MFMA operand, see kv_key_offset in hal_common.h), row-major pages
@@ -78,8 +85,8 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // Two waves per SIMD leave 256 registers each, which keeps the accumulators in VGPRs (no
 // copies to and from AGPRs around every MFMA); the largest head sizes need more.
 #define MIN_WAVES_PER_SIMD (D > 160 ? 1 : 2)
-template <int RT, bool POW2, bool PAGE32, bool SHARED, bool TILED, int KB>
-__global__ void __launch_bounds__(256, MIN_WAVES_PER_SIMD)
+template <int RT, bool POW2, bool PAGE32, bool SHARED, bool TILED, int KB, int HALVES>
+__global__ void __launch_bounds__(256 * HALVES, MIN_WAVES_PER_SIMD)
 attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
                       int out_row_stride, const int* __restrict__ items,
                       const int* __restrict__ n_items_ptr, const int* __restrict__ seg_q_start,
@@ -89,7 +96,10 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                       float* __restrict__ part_o, float* __restrict__ part_ml, int H, int K,
                       int page_size, int page_shift, float scale_log2e, int window,
                       int max_items) {
-  const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
+  static_assert(HALVES == 1 || (SHARED && HALVES == 2), "only the kernel with LDS has two halves");
+  // wave: within its half (it names the item and the fragments the wave loads)
+  const int lane = threadIdx.x % HAL_WAVE, wave = (threadIdx.x / HAL_WAVE) % WAVES;
+  const int half_id = __builtin_amdgcn_readfirstlane(threadIdx.x / (HAL_WAVE * WAVES));
   // Workgroups go to the eight XCDs in turn (linear id modulo 8) and each XCD has an L2 of
   // its own: the ids are renumbered so that an XCD gets a contiguous run of (kv head, item
   // block) pairs, i.e. the tiles that read one head's keys meet in one L2.
@@ -297,7 +307,14 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   // while this step is worked on; a fragment lies there in lane order, as the MFMA wants
   // it back.
   constexpr int NF = 2 * KT + DT, FPW = (NF + WAVES - 1) / WAVES;
-  __shared__ u32x4 frag_lds[SHARED ? 2 : 1][SHARED ? SUBS * NF : 1][HAL_WAVE];
+  // [half of the workgroup][buffer][fragment][lane]; at the end, with two halves, the same
+  // memory carries the second half's sums to the first: [wave][value][lane] floats
+  constexpr int FRAG_BYTES = HALVES * (SHARED ? 2 : 1) * (SHARED ? SUBS * NF : 1) * HAL_WAVE * 16;
+  constexpr int XCH_VALUES = RT * DT * 4 + 2 * RT;
+  constexpr int XCH_BYTES = HALVES == 2 ? WAVES * XCH_VALUES * HAL_WAVE * 4 : 0;
+  __shared__ __align__(16) unsigned char lds_raw[FRAG_BYTES > XCH_BYTES ? FRAG_BYTES : XCH_BYTES];
+  typedef u32x4 (*frag_buffers_t)[SHARED ? SUBS * NF : 1][HAL_WAVE];
+  frag_buffers_t frag_lds = (frag_buffers_t)lds_raw + half_id * (SHARED ? 2 : 1);
   bf16x8 staged[SHARED ? SUBS * FPW : 1];
   int pages_ahead[SUBS];  // of the step after the next
   auto fetch = [&](int j0, const int (&pages)[SUBS]) {
@@ -326,16 +343,20 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
 #pragma unroll
     for (int u = 0; u < SUBS; ++u) pages[u] = page_at(j0 + 32 * u);
   };
+  // the steps of the walk go to the halves in turn: STRIDE keys from one step of a half to
+  // its next; both halves make the same number of rounds (and meet at the same barriers)
+  constexpr int STRIDE = KB * HALVES;
   if constexpr (SHARED) {
+    const int j_mine = j_first + half_id * KB;
     int pages[SUBS];
-    pages_of(j_first, pages);
-    fetch(j_first, pages);
-    stash(j_first, 0);
-    if (j_first + KB < walk_end) {
-      pages_of(j_first + KB, pages);
-      fetch(j_first + KB, pages);
+    pages_of(j_mine, pages);
+    fetch(j_mine, pages);
+    stash(j_mine, 0);
+    if (j_mine + STRIDE < walk_end) {
+      pages_of(j_mine + STRIDE, pages);
+      fetch(j_mine + STRIDE, pages);
     }
-    pages_of(j_first + 2 * KB, pages_ahead);
+    pages_of(j_mine + 2 * STRIDE, pages_ahead);
     __syncthreads();
   } else {
     page_0 = page_at(j_first), page_1 = page_at(j_first + 32), page_2 = page_at(j_first + 64);
@@ -346,13 +367,14 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   }
 
   int half = 0;
-  for (int j0 = j_first; j0 < walk_end; j0 += KB) {
+  for (int jj = j_first; jj < walk_end; jj += STRIDE) {
+    const int j0 = jj + half_id * KB;  // (a second half may have a last round without keys)
     const bool tail = j0 + KB > kv_len;  // some of the keys are not written yet
-    const bool more = j0 + KB < walk_end;
+    const bool more = j0 + STRIDE < walk_end;
     int page_3 = 0;
     int pages_later[SUBS];
     if constexpr (SHARED) {
-      pages_of(j0 + 3 * KB, pages_later);
+      pages_of(j0 + 3 * STRIDE, pages_later);
     } else {
       page_3 = page_at(j0 + 96);
 #pragma unroll
@@ -372,7 +394,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     for (int rt = 0; rt < RT; ++rt)
       // a step wholly after the tile's last row or before its first row's window does
       // nothing for this tile
-      active[rt] = j0 <= p_last[rt] && j0 + KB - 1 >= lo_first[rt] && j0 < kv_end && j0 + KB > kv_begin;
+      active[rt] = j0 <= p_last[rt] && j0 + KB - 1 >= lo_first[rt] && j0 < kv_end && j0 + KB > kv_begin &&
+                   j0 < walk_end;
 #pragma unroll
     for (int u = 0; u < SUBS; ++u) {
       if constexpr (SHARED) {
@@ -490,8 +513,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     if constexpr (SHARED) {
       // the other half was read in the step before this one, and every wave has passed
       // the barrier since
-      if (more) stash(j0 + KB, half ^ 1);
-      if (j0 + 2 * KB < walk_end) fetch(j0 + 2 * KB, pages_ahead);
+      if (more) stash(j0 + STRIDE, half ^ 1);
+      if (j0 + 2 * STRIDE < walk_end) fetch(j0 + 2 * STRIDE, pages_ahead);
       __syncthreads();
       half ^= 1;
 #pragma unroll
@@ -504,6 +527,40 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       page_0 = page_1;
       page_1 = page_2;
       page_2 = page_3;
+    }
+  }
+
+  if constexpr (HALVES == 2) {
+    // The second half's sums go to the first through LDS (the loop's last barrier has
+    // passed, so the fragment buffers are free), lane to lane: wave w of both halves has
+    // the same item, so the same rows in the same lanes.  Joined by the log-sum-exp rule.
+    float* xch = (float*)lds_raw + (size_t)wave * XCH_VALUES * HAL_WAVE + lane;
+    if (half_id == 1) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        xch[(2 * rt) * HAL_WAVE] = m[rt];
+        xch[(2 * rt + 1) * HAL_WAVE] = l[rt];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) xch[(2 * RT + (rt * DT + dt) * 4 + r) * HAL_WAVE] = o[rt][dt][r];
+      }
+    }
+    __syncthreads();
+    if (half_id == 1) return;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const float m1 = xch[(2 * rt) * HAL_WAVE], l1 = xch[(2 * rt + 1) * HAL_WAVE];
+      const float m_new = fmaxf(m[rt], m1);
+      const float m_sub = m_new == -INFINITY ? 0.f : m_new;
+      const float a0 = fast_exp2(m[rt] - m_sub), a1 = fast_exp2(m1 - m_sub);
+      l[rt] = l[rt] * a0 + l1 * a1;
+      m[rt] = m_new;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          o[rt][dt][r] = o[rt][dt][r] * a0 + xch[(2 * RT + (rt * DT + dt) * 4 + r) * HAL_WAVE] * a1;
     }
   }
 
@@ -699,6 +756,12 @@ extern "C" int hal_attention_mfma_head_dim() { return D; }
 #endif
 #define KB_BIG HAL_KB_BIG
 
+// Halves of a workgroup of that kernel (see the top of the file).
+#ifndef HAL_HALVES_BIG
+#define HAL_HALVES_BIG 2
+#endif
+#define HALVES_BIG HAL_HALVES_BIG
+
 extern "C" int hal_attention_mfma_rows_per_big_item() { return 16 * RT_BIG; }
 
 // All arrays are device pointers.  `items` [max_items, 8] lists the work on segments of
@@ -735,22 +798,22 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
   if ((page_size & (page_size - 1)) == 0)
     for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
   const int waves = WAVES;
-#define LAUNCH_ATTENTION(RT_, SHARED_, KB_, LIST, MAX, COUNT)                                      \
+#define LAUNCH_ATTENTION(RT_, SHARED_, KB_, HV_, LIST, MAX, COUNT)                                 \
   {                                                                                               \
     dim3 grid(((MAX) + waves - 1) / waves, K);                                                    \
-    auto kernel = attention_mfma_kernel<RT_, false, false, SHARED_, false, KB_>;                  \
-    if (tiled) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, D % 32 == 0, KB_>;        \
-    else if (page_shift >= 5) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, false, KB_>; \
-    else if (page_shift >= 0) kernel = attention_mfma_kernel<RT_, true, false, SHARED_, false, KB_>; \
-    hipLaunchKernelGGL(kernel, grid, dim3(waves * HAL_WAVE), 0, stream, (const bf16_t*)q,         \
+    auto kernel = attention_mfma_kernel<RT_, false, false, SHARED_, false, KB_, HV_>;             \
+    if (tiled) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, D % 32 == 0, KB_, HV_>;   \
+    else if (page_shift >= 5) kernel = attention_mfma_kernel<RT_, true, true, SHARED_, false, KB_, HV_>; \
+    else if (page_shift >= 0) kernel = attention_mfma_kernel<RT_, true, false, SHARED_, false, KB_, HV_>; \
+    hipLaunchKernelGGL(kernel, grid, dim3(waves * HAL_WAVE * HV_), 0, stream, (const bf16_t*)q,   \
                        q_row_stride, (bf16_t*)out, out_row_stride, LIST, COUNT, seg_q_start,      \
                        seg_q_len, seg_kv_len, block_table, bt_stride, (const bf16_t*)k_pages,     \
                        (const bf16_t*)v_pages, part_o, part_ml, H, K, page_size, page_shift,      \
                        scale_log2e, window, MAX);                                                 \
     HAL_LAUNCH_CHECK();                                                                           \
   }
-  if (max_items > 0) LAUNCH_ATTENTION(1, false, 32, items, max_items, counts)
-  if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, true, KB_BIG, big_items, max_big, counts + 1)
+  if (max_items > 0) LAUNCH_ATTENTION(1, false, 32, 1, items, max_items, counts)
+  if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, true, KB_BIG, HALVES_BIG, big_items, max_big, counts + 1)
 #undef LAUNCH_ATTENTION
   if (max_merges > 0) {
     if (merge_parts > 0 && merge_parts <= MERGE_FEW_PARTS)
