@@ -396,6 +396,16 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       // nothing for this tile
       active[rt] = j0 <= p_last[rt] && j0 + KB - 1 >= lo_first[rt] && j0 < kv_end && j0 + KB > kv_begin &&
                    j0 < walk_end;
+    if constexpr (SHARED && RT > 1) {
+      // With LDS the tiles of a wave go together: a step that concerns one of them is worked
+      // on for all (the masks take care of the others), so that the products of a step are
+      // one run of instructions without branches.  Only the last steps of a walk differ.
+      bool any = false;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) any = any || active[rt];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) active[rt] = any;
+    }
 #pragma unroll
     for (int u = 0; u < SUBS; ++u) {
       if constexpr (SHARED) {
