@@ -371,7 +371,12 @@ def main() -> int:
         prompt_len = end_context - steps - warmup - (2 + EXTRA_MARKED if families else 0)
         slots = [runner.admit() for _ in range(batch)]
         last = []
-        for s in slots:
+        t_said = time.perf_counter()
+        for i_slot, s in enumerate(slots):
+            if time.perf_counter() - t_said > 30:  # a long set-up says that it is alive
+                sync()
+                print(f"[bench] batch {batch}: prompt {i_slot} of {batch} ...", file=sys.stderr, flush=True)
+                t_said = time.perf_counter()
             ids = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=gen).numpy().astype(np.int32)
             pos, tok = 0, None
             while pos < prompt_len:

@@ -1,9 +1,14 @@
 // C[M, N] = A[M, K] * W[N, K]^T in true float32: plain fused multiply-adds on the
 // vector units, no matrix-core mode of reduced precision.  W has the layout of a
 // bias-free linear layer's weight ([out, in], src/halite/transformers/feedforward.py:
-// 204-212; src/halite/transformers/infer/attention.py:21-24).  Each output element
-// is one chain of K multiply-adds in index order, whatever M is, so a token's
-// result does not depend on what else is in the batch.
+// 204-212; src/halite/transformers/infer/attention.py:21-24).
+//
+// Two kernels.  The tiled one (any M): each output element is one chain of K multiply-adds
+// in index order.  The one for at most 16 rows (decode steps), which the tiled one serves
+// at 1/64 to 1/4 of its tile: a wave takes a few columns of the output, its lanes take
+// every 64th group of four k each, and the lanes' partial sums are added in a fixed tree.
+// In both a token's result depends on its own row alone, not on what else is in the batch;
+// between the two the order of the additions differs, i.e. the last bits may.
 #include "hal_common.h"
 #include "hal_api.h"
 
@@ -64,12 +69,76 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
   }
 }
 
+// ---- at most 16 rows ------------------------------------------------------------------------
+// A wave computes MB x NC outputs (MB * NC = 64).  Lane l holds the partial sums of the k's
+// 4 (l + 64 i) .. + 3, added in rising k.  Then the 64 sums of a wave are added across the
+// lanes in six halving steps (a lane keeps the half of the values that its bit picks and
+// hands the other half to its partner), after which lane l holds output l whole.
+template <int MB, int NC>
+__global__ void __launch_bounds__(256)
+gemm_f32_skinny_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
+                       float* __restrict__ C, int ldc, int M, int N, int K) {
+  static_assert(MB * NC == HAL_WAVE, "one output per lane");
+  const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
+  const int n0 = (blockIdx.x * 4 + wave) * NC;
+  if (n0 >= N) return;
+  const float* wrow[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) wrow[c] = W + (size_t)(n0 + c < N ? n0 + c : N - 1) * ldw;
+  float v[MB * NC];
+#pragma unroll
+  for (int i = 0; i < MB * NC; ++i) v[i] = 0.f;
+  for (int k = lane * 4; k < K; k += HAL_WAVE * 4) {  // K is a multiple of 4
+    float4 w[NC], a[MB];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) w[c] = *(const float4*)(wrow[c] + k);
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+      a[m] = m < M ? *(const float4*)(A + (size_t)m * lda + k) : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        float s = v[m * NC + c];
+        s = fmaf(a[m].x, w[c].x, s);
+        s = fmaf(a[m].y, w[c].y, s);
+        s = fmaf(a[m].z, w[c].z, s);
+        s = fmaf(a[m].w, w[c].w, s);
+        v[m * NC + c] = s;
+      }
+  }
+#pragma unroll
+  for (int half = HAL_WAVE / 2; half >= 1; half /= 2) {
+    const bool upper = (lane & half) != 0;
+#pragma unroll
+    for (int i = 0; i < half; ++i) {
+      const float keep = upper ? v[i + half] : v[i];
+      const float give = upper ? v[i] : v[i + half];
+      v[i] = keep + __shfl_xor(give, half, HAL_WAVE);
+    }
+  }
+  const int m = lane / NC, c = lane % NC;
+  if (m < M && n0 + c < N) C[(size_t)m * ldc + n0 + c] = v[0];
+}
+
 extern "C" int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, float* C, int ldc,
                             int M, int N, int K, hipStream_t stream) {
   HAL_REQUIRE(M >= 0 && N > 0 && K > 0, "hal_gemm_f32: bad sizes M=%d N=%d K=%d", M, N, K);
   HAL_REQUIRE(lda >= K && ldw >= K && ldc >= N, "hal_gemm_f32: leading dimensions %d %d %d", lda,
               ldw, ldc);
   if (M == 0) return 0;
+  if (M <= 16 && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && ((uintptr_t)A % 16) == 0 &&
+      ((uintptr_t)W % 16) == 0) {
+    if (M <= 8) {
+      hipLaunchKernelGGL((gemm_f32_skinny_kernel<8, 8>), dim3((N + 31) / 32), dim3(256), 0, stream, A, lda,
+                         W, ldw, C, ldc, M, N, K);
+    } else {
+      hipLaunchKernelGGL((gemm_f32_skinny_kernel<16, 4>), dim3((N + 15) / 16), dim3(256), 0, stream, A, lda,
+                         W, ldw, C, ldc, M, N, K);
+    }
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid((N + GF_BN - 1) / GF_BN, (M + GF_BM - 1) / GF_BM);
   HAL_REQUIRE(grid.y <= 65535, "hal_gemm_f32: M=%d exceeds the grid limit", M);
   hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, A, lda, W, ldw, C, ldc, M, N, K);

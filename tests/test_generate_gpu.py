@@ -208,6 +208,9 @@ def test_cleanup_gives_the_memory_back_and_initialize_brings_the_engine_back(mod
     server = ServerConfig(kv_cache_num_tokens=65536, use_cudagraph=True)
     prompt = tiny.random_tokens(tiny.TINY_B, 20, 7)
     params = {"max_new_tokens": 12, "temperature": 0.0}
+    import gc
+
+    gc.collect()  # what earlier tests left behind must not go away in the middle of the count
     torch.cuda.synchronize()
     base = torch.cuda.memory_allocated()
     engine = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="bfloat16"))

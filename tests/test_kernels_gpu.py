@@ -479,14 +479,24 @@ def test_attention_mfma_hundred_thousand_keys(gpu, tiled):
     close(out, want.float().view(1, H * D), 1.2e-2, "attention over 100,003 keys")
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 256, 64), (5, 331, 120), (64, 200, 352), (130, 96, 1000), (3, 4096, 4096)])
+@pytest.mark.parametrize("M,N,K", [(1, 256, 64), (5, 331, 120), (8, 257, 1000), (9, 130, 36), (16, 1000, 352), (17, 96, 64),
+                                   (64, 200, 352), (130, 96, 1000), (3, 4096, 4096), (2, 50, 30)])
 def test_gemm_f32(gpu, M, N, K):
     a, w = rnd(M, K, seed=50), rnd(N, K, seed=51)
     want = (a.double() @ w.double().T).float()
     close(ops.gemm_f32(a.to(gpu), w.to(gpu)), want, 3e-6, "gemm_f32")
-    # a row's result does not depend on the other rows of the batch
+    # a row's result does not depend on the other rows of the batch, bit for bit: with
+    # other rows beside it (the same kernel, at most 16 rows or more) ...
+    whole = ops.gemm_f32(a.to(gpu), w.to(gpu))
+    others = a.clone()
+    others[1:] = rnd(M, K, seed=52)[1:] * 3.0
+    assert torch.equal(whole[:1].cpu(), ops.gemm_f32(others.to(gpu), w.to(gpu))[:1].cpu())
+    # ... and alone, where both take the kernel for few rows (the two kernels add in
+    # different orders: the last bits may differ between them)
     alone = ops.gemm_f32(a[:1].to(gpu).contiguous(), w.to(gpu))
-    assert torch.equal(alone.cpu(), ops.gemm_f32(a.to(gpu), w.to(gpu))[:1].cpu())
+    if M <= 16:
+        assert torch.equal(alone.cpu(), whole[:1].cpu())
+    close(alone, whole[:1], 2e-6, "a row alone and in a larger batch")
 
 
 @pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 48, 64])
