@@ -425,14 +425,14 @@ def main() -> int:
         if families:
             # one more step, eager (every kernel launched from the host), with events
             # around every call of a kernel wrapper
-            graph, runner.server_config.use_cudagraph = runner.server_config.use_cudagraph, False
+            graph, runner.graphs_allowed = runner.graphs_allowed, False
             try:
                 last = one_step(last)  # the eager path's first call (allocations, library loads)
                 with Families() as f:
                     one_step(last)
                 fam = f.totals_ms()
             finally:
-                runner.server_config.use_cudagraph = graph
+                runner.graphs_allowed = graph
         for s in slots:
             runner.free(s)
         return dt, kv_tokens, gpu_s, fam

@@ -8,6 +8,9 @@ fields of the configuration objects: ``sampling.<field>`` (SamplingParams),
     python -m halite_amd.cli.generate --model DIR --prompt-ids 1,2,3 \\
         sampling.temperature=0.8 sampling.max_new_tokens=24 server.page_size=16
 
+Instead of ``--model``, ``--random CONFIG.json`` (with ``--weights-seed``) runs a model of
+that configuration with seeded random weights, drawn on the device and never written.
+
 Prompts are token ids (``--prompt-ids``, repeatable; ``--prompt-file`` with one JSON
 list a line) or seeded uniform-random ids of given lengths (``--prompt-lens``).
 Results are printed as one JSON object a line.
@@ -26,7 +29,10 @@ from ..config import ModelConfig, ServerConfig, parse_overrides, read_config
 
 def parse_args(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--model", type=str, required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--model", type=str, help="folder with config.json and model.safetensors")
+    ap.add_argument("--random", type=str, metavar="CONFIG.json",
+                    help="instead of --model: a config.json whose model gets seeded random weights N(0, 0.02)")
+    ap.add_argument("--weights-seed", type=int, default=0, help="seed of the random weights of --random")
     ap.add_argument("--prompt-ids", action="append", default=[], help="comma-separated token ids; repeatable")
     ap.add_argument("--prompt-file", type=str, help="file with one JSON list of token ids a line")
     ap.add_argument("--prompt-lens", type=str, help="comma-separated lengths of random prompts")
@@ -66,7 +72,15 @@ def generate(args) -> int:
     from ..engine import InferenceEngine
     from ..sampling import SamplingParams
 
-    _, cfg = read_config(args.model)
+    if bool(args.model) == bool(args.random):
+        raise SystemExit("give one of --model DIR and --random CONFIG.json")
+    if args.random:
+        from ..config import parse_config
+
+        with open(args.random) as f:
+            _, cfg = parse_config(json.load(f))
+    else:
+        _, cfg = read_config(args.model)
     prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
     if args.prompt_file:
         with open(args.prompt_file) as f:
@@ -78,9 +92,13 @@ def generate(args) -> int:
     if not prompts:
         raise SystemExit("no prompts: give --prompt-ids, --prompt-file or --prompt-lens")
 
-    engine = InferenceEngine.from_pretrained(
-        args.model, ServerConfig(**over["server"]), ModelConfig(**over["model"]), seed=args.seed
-    )
+    server, model = ServerConfig(**over["server"]), ModelConfig(**over["model"])
+    if args.random:
+        from ..engine.runner import ModelRunner
+
+        engine = InferenceEngine(ModelRunner.from_random(cfg, args.weights_seed, server, model), None, seed=args.seed)
+    else:
+        engine = InferenceEngine.from_pretrained(args.model, server, model, seed=args.seed)
     params = SamplingParams(**over["sampling"])
     results = engine.infer_batch([(i, p, params) for i, p in enumerate(prompts)])
     for r in results:

@@ -93,6 +93,12 @@ class ModelRunner:
         self._token_feed = None
         kv_heads = [n.n_kv_heads for n in needs.values()] or [1]
         self._min_kv_heads = min(kv_heads)
+        # graphs replay a model only if every part of it reads what varies on the device
+        self.graphs_allowed = (
+            self.server_config.use_cudagraph and self.device.type == "cuda"
+            and all(p.graph_safe for p in self.model.named_parts().values())
+            and all(b.graph_safe for b in self.model.layers.values())
+        )
         self.graph_replays = 0
         self.released = False
         self.has_weights = True  # the model comes filled; restore() gives one that is not
@@ -216,7 +222,7 @@ class ModelRunner:
         src/halite/transformers/infer/engine/model_runner.py:159-239).  Needs an idle
         cache: every size is run once with one-token requests that are freed again.
         Returns the sizes that have a graph afterwards."""
-        if not self.server_config.use_cudagraph:
+        if not self.graphs_allowed:
             return []
         if not self.cache.idle():
             raise RuntimeError("graphs are recorded ahead of time only while no request is live")
@@ -279,7 +285,7 @@ class ModelRunner:
         self.check_segments(segments, self.vocab_size if token_feed is None else token_feed.numel())
         spans = [(s.slot, s.start + s.tokens.size) for s in segments]
         graph_step = (
-            self.server_config.use_cudagraph
+            self.graphs_allowed
             and len(segments) <= self.server_config.cudagraph_max_batch_size
             and all(s.tokens.size == 1 and s.want == [0] for s in segments)
         )

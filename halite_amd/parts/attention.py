@@ -36,6 +36,7 @@ class Attention(Mixer):
     """
 
     Params = AttentionParams
+    graph_safe = True
     takes_normed_rows = True
     folds_next_norm = True
 

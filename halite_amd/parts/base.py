@@ -79,6 +79,12 @@ class Part:
     """Base of all parts."""
 
     Params: ClassVar[type[BaseModel]]
+    # True: what ``forward`` launches depends only on how many tokens each segment of the
+    # step has and how many rows are wanted; everything else (token ids, positions, pages,
+    # slots, lengths of the contexts) it reads on the device, from the step's arrays.  A
+    # step recorded into a graph can then be replayed for another step of that shape.  A
+    # model is run from graphs only if all of its parts say so.
+    graph_safe: ClassVar[bool] = False
 
     def __init__(self, params: BaseModel, build: BuildContext):
         self.p = params
@@ -236,6 +242,7 @@ class Arrangement:
 
     roles: ClassVar[dict[str, "Registry"]] = {}
     optional: ClassVar[tuple[str, ...]] = ()
+    graph_safe: ClassVar[bool] = False  # as for Part
 
     def __init__(self, parts: dict[str, Part | None]):
         self._parts = dict(parts)

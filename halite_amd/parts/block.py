@@ -22,6 +22,7 @@ class PreNormBlock(Arrangement):
     norm (or to the model's final norm) instead of adding it itself.
     """
 
+    graph_safe = True
     roles = {"mixer_norm": NORMS, "mixer": MIXERS, "ff_norm": NORMS, "ff": FEED_FORWARDS}
     takes_next_norm = True  # forward() accepts next_norm=
 

@@ -21,6 +21,7 @@ class TokenEmbedding(Embedding):
     residual stream."""
 
     Params = EmbeddingParams
+    graph_safe = True
 
     def param_decls(self):
         return {"weight": ParamDecl((self.p.vocab_size, self.p.size))}
@@ -43,6 +44,7 @@ class LinearHead(Head):
     (src/halite/transformers/transformer.py:59-61), bound by the model builder."""
 
     Params = LinearHeadParams
+    graph_safe = True
 
     def param_decls(self):
         if self.p.tied:

@@ -30,6 +30,7 @@ class GatedFeedForward(FeedForward):
     the multiply are float32 on the accumulators or on the product's output."""
 
     Params = GatedParams
+    graph_safe = True
     takes_normed_rows = True
     folds_next_norm = True
 

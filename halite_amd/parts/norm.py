@@ -22,6 +22,7 @@ class RMSNorm(Norm):
     norm in a block (src/halite/transformers/block.py:56-74) is fused in."""
 
     Params = RMSNormParams
+    graph_safe = True
 
     def param_decls(self):
         return {"weight": ParamDecl((self.p.size,), init="ones")}

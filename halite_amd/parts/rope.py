@@ -80,6 +80,7 @@ class Rope(RotaryPositionEncoding):
     keys and values to the cache."""
 
     Params = RopeParams
+    graph_safe = True
 
     def __init__(self, params, build):
         super().__init__(params, build)

@@ -254,6 +254,19 @@ def test_command_line(models, tmp_path):
     proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "halite_make_random_model"), "--config", str(cfgfile),
                            "--out", str(out), "--seed", "3", "--dtype", "float32"], capture_output=True, text=True)
     assert proc.returncode == 0 and (out / "model.safetensors").exists() and (out / "config.json").exists()
+    # --random CONFIG.json: the same configuration with weights drawn on the device; the seed decides
+    def random_run(seed):
+        cmd = [sys.executable, "-m", "halite_amd.cli.generate", "--random", str(cfgfile), "--weights-seed", str(seed),
+               "--prompt-ids", "5,17,3", "sampling.temperature=0", "sampling.max_new_tokens=5", "model.dtype=float32"]
+        proc = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        return json.loads(proc.stdout.strip())["output_ids"][0]
+
+    first = random_run(3)
+    assert len(first) == 5 and first == random_run(3)
+    proc = subprocess.run([sys.executable, "-m", "halite_amd.cli.generate", "--prompt-ids", "1"], cwd=ROOT,
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode != 0 and "--model DIR and --random" in proc.stderr
 
 
 def test_a_dropped_engine_does_not_disturb_a_capture(models):
