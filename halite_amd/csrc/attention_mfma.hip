@@ -70,6 +70,26 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16
 // 2^x for x <= 0 (results below the normal range may flush to zero)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// The larger of x in this lane and in the lane 32 (16) places away: the swap instructions
+// exchange register halves (quarters) between two registers on the vector unit itself,
+// where a shuffle is a trip through the LDS hardware that the wave waits for.
+__device__ __forceinline__ float max_across_32(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float max_across_16(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return fmaxf(a, b);
+}
+// 16 bytes of every lane from global memory straight into LDS: the wave's 64 pieces land
+// one after the other from `lds` on (the same address for the whole wave).
+__device__ __forceinline__ void load_to_lds(const bf16_t* src, void* lds) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+}
+
 // item: {segment, first row of tile 0, first key, end key, first partial slot or -1,
 //        first row of tile 1, of tile 2, of tile 3 (or -1)}
 // An item of the one-tile kernel carries its segment's first token, number of tokens and
@@ -98,7 +118,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                       int max_items) {
   static_assert(HALVES == 1 || (SHARED && HALVES == 2), "only the kernel with LDS has two halves");
   // wave: within its half (it names the item and the fragments the wave loads)
-  const int lane = threadIdx.x % HAL_WAVE, wave = (threadIdx.x / HAL_WAVE) % WAVES;
+  const int lane = threadIdx.x % HAL_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane((threadIdx.x / HAL_WAVE) % WAVES);
   const int half_id = __builtin_amdgcn_readfirstlane(threadIdx.x / (HAL_WAVE * WAVES));
   // Workgroups go to the eight XCDs in turn (linear id modulo 8) and each XCD has an L2 of
   // its own: the ids are renumbered so that an XCD gets a contiguous run of (kv head, item
@@ -241,39 +262,48 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   };
   // One fragment is what one MFMA takes from the block of 32 keys, 16 bytes a lane:
   // (t, ks) of the keys, dt of the values.
-  auto load_key_frag = [&](int j0, int page, int t, int ks) -> bf16x8 {
-    const int d0 = ks * 32 + quad * 8;
-    if (D % 32 != 0 && d0 >= D) return zero8();
+  // (a lane whose 8 dimensions lie past a head size that is no multiple of 32 is pointed
+  // at the 16 before them: what it reads meets zeros of Q)
+  auto key_frag_ptr = [&](int j0, int page, int t, int ks) -> const bf16_t* {
+    int d0 = ks * 32 + quad * 8;
+    if (D % 32 != 0 && d0 >= D) d0 -= 16;
     if constexpr (TILED) {  // the fragment is one contiguous KB
       const bf16_t* base =
           k_pages + (((size_t)page * K + g) * page_size + (j0 & (page_size - 1))) * D;
-      return ld16(base + (t * KT + ks) * 512 + lane * 8);
+      return base + (t * KT + ks) * 512 + lane * 8;
     } else if constexpr (PAGE32) {
       const bf16_t* base =
           k_pages + (((size_t)page * K + g) * page_size + (j0 & (page_size - 1))) * D;
-      return ld16(base + koff0 + t * 4 * D + ks * 32);
+      return base + (koff0 - quad * 8) + t * 4 * D + d0;
     } else {
       const int j = key_index(j0, t);
       const long long pg = bt[page_of(j)];
-      return ld16(k_pages + (((size_t)pg * K + g) * page_size + slot_of(j)) * D + d0);
+      return k_pages + (((size_t)pg * K + g) * page_size + slot_of(j)) * D + d0;
     }
   };
-  auto load_value_frag = [&](int j0, int page, int dt) -> bf16x8 {
+  auto load_key_frag = [&](int j0, int page, int t, int ks) -> bf16x8 {
+    if (D % 32 != 0 && ks * 32 + quad * 8 >= D) return zero8();
+    return ld16(key_frag_ptr(j0, page, t, ks));
+  };
+  auto value_frag_ptr = [&](int j0, int page, int dt) -> const bf16_t* {
     // lane loads V^T[dim dt*16 + col][keys jv .. jv+8]
     if constexpr (TILED) {
       const bf16_t* base =
           v_pages + (((size_t)page * K + g) * page_size + (j0 & (page_size - 1))) * D;
-      return ld16(base + dt * 512 + lane * 8);
+      return base + dt * 512 + lane * 8;
     } else if constexpr (PAGE32) {
       const bf16_t* base =
           v_pages + ((size_t)page * K + g) * D * page_size + (j0 & (page_size - 1));
-      return ld16(base + voff + (size_t)dt * 16 * page_size);
+      return base + voff + (size_t)dt * 16 * page_size;
     } else {
       const int jv = value_index(j0);
       const long long pg = bt[page_of(jv)];
-      return ld16(v_pages + ((size_t)pg * K + g) * D * page_size + slot_of(jv) +
-                  (size_t)(dt * 16 + col) * page_size);
+      return v_pages + ((size_t)pg * K + g) * D * page_size + slot_of(jv) +
+             (size_t)(dt * 16 + col) * page_size;
     }
+  };
+  auto load_value_frag = [&](int j0, int page, int dt) -> bf16x8 {
+    return ld16(value_frag_ptr(j0, page, dt));
   };
   // unwritten slots may hold anything, NaN included, and 0 * NaN must not get in: in the
   // last block of the request the values of keys past the end are cleared
@@ -298,149 +328,18 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     else return 0;
   };
 
-  // Without LDS: this block's values and the next block's keys (a second buffer) are asked
-  // for at the block's start; deeper or shallower schedules measured the same or worse.
-  int page_0 = 0, page_1 = 0, page_2 = 0;
-  bf16x8 kcur[2][KT], knext[SHARED ? 1 : 2][SHARED ? 1 : KT], vf[DT];
-  // With LDS: fragment f of a block of 32 keys (keys first, then values) is loaded by wave
-  // f % 4 into registers one step ahead, and written to the other half of the LDS buffer
-  // while this step is worked on; a fragment lies there in lane order, as the MFMA wants
-  // it back.
-  constexpr int NF = 2 * KT + DT, FPW = (NF + WAVES - 1) / WAVES;
-  // [half of the workgroup][buffer][fragment][lane]; at the end, with two halves, the same
-  // memory carries the second half's sums to the first: [wave][value][lane] floats
-  constexpr int FRAG_BYTES = HALVES * (SHARED ? 2 : 1) * (SHARED ? SUBS * NF : 1) * HAL_WAVE * 16;
-  constexpr int XCH_VALUES = RT * DT * 4 + 2 * RT;
-  constexpr int XCH_BYTES = HALVES == 2 ? WAVES * XCH_VALUES * HAL_WAVE * 4 : 0;
-  __shared__ __align__(16) unsigned char lds_raw[FRAG_BYTES > XCH_BYTES ? FRAG_BYTES : XCH_BYTES];
-  typedef u32x4 (*frag_buffers_t)[SHARED ? SUBS * NF : 1][HAL_WAVE];
-  frag_buffers_t frag_lds = (frag_buffers_t)lds_raw + half_id * (SHARED ? 2 : 1);
-  bf16x8 staged[SHARED ? SUBS * FPW : 1];
-  int pages_ahead[SUBS];  // of the step after the next
-  auto fetch = [&](int j0, const int (&pages)[SUBS]) {
-#pragma unroll
-    for (int u = 0; u < SUBS; ++u)
-#pragma unroll
-      for (int i = 0; i < FPW; ++i) {
-        const int f = wave + WAVES * i;
-        if (f < 2 * KT) staged[u * FPW + i] = load_key_frag(j0 + 32 * u, pages[u], f / KT, f % KT);
-        else if (f < NF) staged[u * FPW + i] = load_value_frag(j0 + 32 * u, pages[u], f - 2 * KT);
-      }
-  };
-  auto stash = [&](int j0, int half) {
-#pragma unroll
-    for (int u = 0; u < SUBS; ++u)
-#pragma unroll
-      for (int i = 0; i < FPW; ++i) {
-        const int f = wave + WAVES * i;
-        if (f >= NF) continue;
-        bf16x8 v = staged[u * FPW + i];
-        if (f >= 2 * KT && j0 + 32 * u + 32 > kv_len) v = clear_unwritten(j0 + 32 * u, v);
-        frag_lds[half][u * NF + f][lane] = __builtin_bit_cast(u32x4, v);
-      }
-  };
-  auto pages_of = [&](int j0, int (&pages)[SUBS]) {
-#pragma unroll
-    for (int u = 0; u < SUBS; ++u) pages[u] = page_at(j0 + 32 * u);
-  };
-  // the steps of the walk go to the halves in turn: STRIDE keys from one step of a half to
-  // its next; both halves make the same number of rounds (and meet at the same barriers)
-  constexpr int STRIDE = KB * HALVES;
-  if constexpr (SHARED) {
-    const int j_mine = j_first + half_id * KB;
-    int pages[SUBS];
-    pages_of(j_mine, pages);
-    fetch(j_mine, pages);
-    stash(j_mine, 0);
-    if (j_mine + STRIDE < walk_end) {
-      pages_of(j_mine + STRIDE, pages);
-      fetch(j_mine + STRIDE, pages);
-    }
-    pages_of(j_mine + 2 * STRIDE, pages_ahead);
-    __syncthreads();
-  } else {
-    page_0 = page_at(j_first), page_1 = page_at(j_first + 32), page_2 = page_at(j_first + 64);
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int ks = 0; ks < KT; ++ks) kcur[t][ks] = load_key_frag(j_first, page_0, t, ks);
-  }
-
-  int half = 0;
-  for (int jj = j_first; jj < walk_end; jj += STRIDE) {
-    const int j0 = jj + half_id * KB;  // (a second half may have a last round without keys)
-    const bool tail = j0 + KB > kv_len;  // some of the keys are not written yet
-    const bool more = j0 + STRIDE < walk_end;
-    int page_3 = 0;
-    int pages_later[SUBS];
-    if constexpr (SHARED) {
-      pages_of(j0 + 3 * STRIDE, pages_later);
-    } else {
-      page_3 = page_at(j0 + 96);
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) vf[dt] = load_value_frag(j0, page_0, dt);
-      if (more) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int ks = 0; ks < KT; ++ks) knext[t][ks] = load_key_frag(j0 + 32, page_1, t, ks);
-      }
-    }
-
-    // ---- S^T = K Q^T for KB keys (tiles of 16), all row tiles ----------------------
-    f32x4 s[RT][SUBS][2];
-    bool active[RT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-      // a step wholly after the tile's last row or before its first row's window does
-      // nothing for this tile
-      active[rt] = j0 <= p_last[rt] && j0 + KB - 1 >= lo_first[rt] && j0 < kv_end && j0 + KB > kv_begin &&
-                   j0 < walk_end;
-    if constexpr (SHARED && RT > 1) {
-      // With LDS the tiles of a wave go together: a step that concerns one of them is worked
-      // on for all (the masks take care of the others), so that the products of a step are
-      // one run of instructions without branches.  Only the last steps of a walk differ.
-      bool any = false;
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) any = any || active[rt];
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) active[rt] = any;
-    }
-#pragma unroll
-    for (int u = 0; u < SUBS; ++u) {
-      if constexpr (SHARED) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int ks = 0; ks < KT; ++ks)
-            kcur[t][ks] = __builtin_bit_cast(bf16x8, frag_lds[half][u * NF + t * KT + ks][lane]);
-      }
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          s[rt][u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-          if (active[rt]) {
-#pragma unroll
-            for (int ks = 0; ks < KT; ++ks)
-              s[rt][u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][ks], bq[rt][ks],
-                                                                    s[rt][u][t], 0, 0, 0);
-          }
-        }
-      }
-    }
-
-    bf16x8 pb[RT][SUBS];
-    float alpha[RT];
+  // ---- one step's mask and online softmax, for every row tile: scores in, probabilities
+  // (as the B operand of the second product) and the factor for the old sums out.  Of every
+  // block of 32 keys this lane has the keys quad*8 + e, e = 0..7.  Raw scores; the scale
+  // (positive) goes into the exponent's multiply-add.
+  auto softmax_step = [&](int j0, const f32x4 (&s)[RT][SUBS][2], const bool (&active)[RT],
+                          bf16x8 (&pb)[RT][SUBS], float (&alpha)[RT]) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       alpha[rt] = 1.f;
 #pragma unroll
       for (int u = 0; u < SUBS; ++u) pb[rt][u] = zero8();
       if (!active[rt]) continue;
-      // ---- mask and online softmax: of every block of 32 keys this lane has the keys
-      // quad*8 + e, e = 0..7.  Raw scores; the scale (positive) goes into the exponent's
-      // multiply-add.
       float sv[SUBS * 8];
       float m_raw = -INFINITY;
       const bool full = j0 >= kv_begin && j0 + KB <= kv_end && j0 + KB - 1 <= p_first[rt] &&
@@ -461,8 +360,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
           m_raw = fmaxf(m_raw, sv[e]);
         }
       }
-      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 16, HAL_WAVE));
-      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32, HAL_WAVE));
+      m_raw = max_across_16(max_across_32(m_raw));
       const float m_tile = m_raw * scale_log2e;
       // The running maximum only has to keep exp2(s - m) in range, so it is raised
       // only when the step's maximum exceeds it by more than 2^RESCALE_SLACK: then
@@ -489,11 +387,9 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
         pb[rt][u] = __builtin_bit_cast(bf16x8, praw);
       }
     }
-
-    // ---- O^T += V^T P^T ------------------------------------------------------------
+    // rescale the sums only if some row of the tile raised its maximum
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      // rescale the sums only if some row of the tile raised its maximum
       if (__builtin_amdgcn_ballot_w64(alpha[rt] != 1.f) != 0) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -501,13 +397,248 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
           for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha[rt];
       }
     }
+  };
+  // a step wholly after the tile's last row or before its first row's window does nothing
+  // for this tile
+  auto tile_active = [&](int j0, int rt) {
+    return j0 <= p_last[rt] && j0 + KB - 1 >= lo_first[rt] && j0 < kv_end && j0 + KB > kv_begin &&
+           j0 < walk_end;
+  };
+
+  constexpr int FK = 2 * KT;                       // key fragments of a block of 32 keys
+  constexpr int NFK = SUBS * FK, NFV = SUBS * DT;  // key and value fragments of a step
+  constexpr int XCH_VALUES = RT * DT * 4 + 2 * RT;
+  constexpr int XCH_BYTES = HALVES == 2 ? WAVES * XCH_VALUES * HAL_WAVE * 4 : 0;
+  // With LDS: [half of the workgroup][keys: two buffers of NFK fragments, values: two of
+  // NFV][lane]: a fragment lies there in lane order, as the MFMA wants it back.  At the end,
+  // with two halves, the same memory carries the second half's sums to the first:
+  // [wave][value][lane] floats.
+  constexpr int FRAG_BYTES = SHARED ? HALVES * 2 * (NFK + NFV) * HAL_WAVE * 16 : 16;
+  __shared__ __align__(16) unsigned char lds_raw[FRAG_BYTES > XCH_BYTES ? FRAG_BYTES : XCH_BYTES];
+
+  if constexpr (SHARED) {
+    // Fragment f of a step is brought in by wave f % 4, straight from global memory into
+    // LDS (every lane names its own 16 bytes; they land in lane order).  The steps of the
+    // walk go to the halves in turn: STRIDE keys from one step of a half to its next; both
+    // halves make the same number of steps (the second may have a last one without keys).
+    //
+    // A step of a half is two blocks of instructions with a barrier before each:
+    //   barrier 1: the loads that the half asked for a step ago have landed, the buffers of
+    //     the step before are free;
+    //   the block for the vector units: ask for the keys of the step after the next and the
+    //     values of the next step, read this step's first values from LDS, softmax;
+    //   barrier 2 (no data waits for it: it keeps the halves apart);
+    //   the block for the matrix cores: probabilities times values of this step, then keys
+    //     times queries of the next step, with every LDS read asked for one run of
+    //     products before its use.
+    // The second half passes one barrier more before its first step and is thereby half a
+    // step behind: one half's softmax runs while the other half's products do.  Left to
+    // themselves the two waves of a SIMD fall into step with each other, and the vector
+    // units and the matrix cores take turns.
+    typedef u32x4 frag_t[HAL_WAVE];
+    frag_t* const kbuf = (frag_t*)lds_raw + (size_t)half_id * 2 * (NFK + NFV);
+    frag_t* const vbuf = kbuf + 2 * NFK;
+    constexpr int STRIDE = KB * HALVES;
+    const int n_steps = (walk_end - j_first + STRIDE - 1) / STRIDE;
+    auto j_of = [&](int i) { return j_first + i * STRIDE + half_id * KB; };
+    auto pages_of = [&](int j0, int (&pages)[SUBS]) {
 #pragma unroll
-    for (int u = 0; u < SUBS; ++u) {
-      if constexpr (SHARED) {
+      for (int u = 0; u < SUBS; ++u) pages[u] = page_at(j0 + 32 * u);
+    };
+    auto ask_keys = [&](int j0, const int (&pages)[SUBS], int b) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-          vf[dt] = __builtin_bit_cast(bf16x8, frag_lds[half][u * NF + 2 * KT + dt][lane]);
-      } else if (tail) {
+      for (int i = 0; i < (NFK + WAVES - 1) / WAVES; ++i) {
+        const int f = wave + WAVES * i;
+        if (f < NFK)
+          load_to_lds(key_frag_ptr(j0 + 32 * (f / FK), pages[f / FK], (f % FK) / KT, f % KT),
+                      kbuf + b * NFK + f);
+      }
+    };
+    auto ask_values = [&](int j0, const int (&pages)[SUBS], int b) {
+#pragma unroll
+      for (int i = 0; i < (NFV + WAVES - 1) / WAVES; ++i) {
+        const int f = wave + WAVES * i;
+        if (f < NFV)
+          load_to_lds(value_frag_ptr(j0 + 32 * (f / DT), pages[f / DT], f % DT), vbuf + b * NFV + f);
+      }
+    };
+    // the values of keys past the request's end are cleared where they landed, by the wave
+    // that asked for them (after its loads have come, before the barrier that shows them)
+    auto clear_tail_values = [&](int j0, int b) {
+#pragma unroll
+      for (int i = 0; i < (NFV + WAVES - 1) / WAVES; ++i) {
+        const int f = wave + WAVES * i;
+        if (f < NFV && j0 + 32 * (f / DT) + 32 > kv_len) {
+          u32x4* at = &vbuf[b * NFV + f][lane];
+          *at = __builtin_bit_cast(
+              u32x4, clear_unwritten(j0 + 32 * (f / DT), __builtin_bit_cast(bf16x8, *at)));
+        }
+      }
+    };
+    auto loads_landed = [] { __builtin_amdgcn_s_waitcnt(0x0F70); };  // vmcnt(0)
+    auto phase_barrier = [] {
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    constexpr int FR = FK > DT ? FK : DT;
+    bf16x8 fa[FR], fb[FR];  // two sets of fragment registers, filled in turn
+    auto read_keys = [&](bf16x8 (&f)[FR], int b, int u) {
+#pragma unroll
+      for (int x = 0; x < FK; ++x) f[x] = __builtin_bit_cast(bf16x8, kbuf[b * NFK + u * FK + x][lane]);
+    };
+    auto read_values = [&](bf16x8 (&f)[FR], int b, int u) {
+#pragma unroll
+      for (int x = 0; x < DT; ++x) f[x] = __builtin_bit_cast(bf16x8, vbuf[b * NFV + u * DT + x][lane]);
+    };
+    f32x4 s[RT][SUBS][2];
+    // consecutive products go to different sums, so none waits for the one before it
+    auto keys_times_queries = [&](const bf16x8 (&f)[FR], int u) {
+#pragma unroll
+      for (int ks = 0; ks < KT; ++ks)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            s[rt][u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                f[t * KT + ks], bq[rt][ks], ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[rt][u][t], 0, 0, 0);
+    };
+    bf16x8 pb[RT][SUBS];
+    auto probabilities_times_values = [&](const bf16x8 (&f)[FR], int u) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[dt], pb[rt][u], o[rt][dt], 0, 0, 0);
+    };
+
+    int pages_1[SUBS], pages_2[SUBS];  // of the next step and of the one after it
+    {
+      int pages_0[SUBS];
+      pages_of(j_of(0), pages_0);
+      pages_of(j_of(1), pages_1);
+      pages_of(j_of(2), pages_2);
+      ask_keys(j_of(0), pages_0, 0);
+      ask_values(j_of(0), pages_0, 0);
+      if (1 < n_steps) ask_keys(j_of(1), pages_1, 1);
+      loads_landed();
+      if (j_of(0) + KB > kv_len) clear_tail_values(j_of(0), 0);
+      __syncthreads();
+    }
+    if constexpr (HALVES == 2) {
+      if (half_id == 1) phase_barrier();
+    }
+    read_keys(fa, 0, 0);
+    if constexpr (SUBS == 2) read_keys(fb, 0, 1);
+    keys_times_queries(fa, 0);
+    if constexpr (SUBS == 2) keys_times_queries(fb, 1);
+
+    for (int i = 0; i < n_steps; ++i) {
+      const int j0 = j_of(i), b = i & 1;
+      int pages_3[SUBS];
+      pages_of(j_of(i + 3), pages_3);
+      phase_barrier();  // 1
+      if (i + 2 < n_steps) ask_keys(j_of(i + 2), pages_2, b);
+      if (i + 1 < n_steps) ask_values(j_of(i + 1), pages_1, b ^ 1);
+      read_values(fa, b, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // The tiles of a wave go together: a step that concerns one of them is worked on for
+      // all (the masks take care of the others); only the last steps of a walk differ.
+      bool active[RT];
+      bool any = false;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) any = any || tile_active(j0, rt);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) active[rt] = any;
+      float alpha[RT];
+      softmax_step(j0, s, active, pb, alpha);
+      // 2: the barrier instruction alone (no data waits for it, and a fence would wait for
+      // the loads that were asked for a moment ago)
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      // (a step that concerns no tile has probabilities of zero, and after the last step
+      // the scores of a step that does not exist are computed from what the buffer holds
+      // and never looked at: the run of products has no branch)
+      if constexpr (SUBS == 2) {
+        read_values(fb, b, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        probabilities_times_values(fa, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_keys(fa, b ^ 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        probabilities_times_values(fb, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        read_keys(fb, b ^ 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        keys_times_queries(fa, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        keys_times_queries(fb, 1);
+      } else {
+        read_keys(fb, b ^ 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        probabilities_times_values(fa, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        keys_times_queries(fb, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      loads_landed();
+      if (i + 1 < n_steps && j_of(i + 1) + KB > kv_len) clear_tail_values(j_of(i + 1), b ^ 1);
+#pragma unroll
+      for (int u = 0; u < SUBS; ++u) {
+        pages_1[u] = pages_2[u];
+        pages_2[u] = pages_3[u];
+      }
+    }
+    if constexpr (HALVES == 2) {
+      if (half_id == 0) phase_barrier();  // as many barriers as the second half
+    }
+  } else {
+    // Without LDS: this block's values and the next block's keys (a second buffer) are asked
+    // for at the block's start; deeper or shallower schedules measured the same or worse.
+    int page_0 = page_at(j_first), page_1 = page_at(j_first + 32), page_2 = page_at(j_first + 64);
+    bf16x8 kcur[2][KT], knext[2][KT], vf[DT];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int ks = 0; ks < KT; ++ks) kcur[t][ks] = load_key_frag(j_first, page_0, t, ks);
+
+    for (int j0 = j_first; j0 < walk_end; j0 += KB) {
+      const bool tail = j0 + KB > kv_len;  // some of the keys are not written yet
+      const bool more = j0 + KB < walk_end;
+      const int page_3 = page_at(j0 + 96);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vf[dt] = load_value_frag(j0, page_0, dt);
+      if (more) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int ks = 0; ks < KT; ++ks) knext[t][ks] = load_key_frag(j0 + 32, page_1, t, ks);
+      }
+
+      // ---- S^T = K Q^T for 32 keys (two tiles of 16), all row tiles -------------------
+      f32x4 s[RT][SUBS][2];
+      bool active[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        active[rt] = tile_active(j0, rt);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          s[rt][0][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+          if (active[rt]) {
+#pragma unroll
+            for (int ks = 0; ks < KT; ++ks)
+              s[rt][0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kcur[t][ks], bq[rt][ks],
+                                                                    s[rt][0][t], 0, 0, 0);
+          }
+        }
+      }
+      bf16x8 pb[RT][SUBS];
+      float alpha[RT];
+      softmax_step(j0, s, active, pb, alpha);
+
+      // ---- O^T += V^T P^T ----------------------------------------------------------
+      if (tail) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) vf[dt] = clear_unwritten(j0, vf[dt]);
       }
@@ -516,20 +647,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
         if (!active[rt]) continue;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
-          o[rt][dt] =
-              __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb[rt][u], o[rt][dt], 0, 0, 0);
+          o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb[rt][0], o[rt][dt], 0, 0, 0);
       }
-    }
-    if constexpr (SHARED) {
-      // the other half was read in the step before this one, and every wave has passed
-      // the barrier since
-      if (more) stash(j0 + STRIDE, half ^ 1);
-      if (j0 + 2 * STRIDE < walk_end) fetch(j0 + 2 * STRIDE, pages_ahead);
-      __syncthreads();
-      half ^= 1;
-#pragma unroll
-      for (int u = 0; u < SUBS; ++u) pages_ahead[u] = pages_later[u];
-    } else {
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -539,11 +658,12 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       page_2 = page_3;
     }
   }
-
   if constexpr (HALVES == 2) {
-    // The second half's sums go to the first through LDS (the loop's last barrier has
-    // passed, so the fragment buffers are free), lane to lane: wave w of both halves has
-    // the same item, so the same rows in the same lanes.  Joined by the log-sum-exp rule.
+    // The second half's sums go to the first through LDS (after a barrier that every wave
+    // reaches with its last products done, so the fragment buffers are free), lane to lane:
+    // wave w of both halves has the same item, so the same rows in the same lanes.  Joined
+    // by the log-sum-exp rule.
+    __syncthreads();
     float* xch = (float*)lds_raw + (size_t)wave * XCH_VALUES * HAL_WAVE + lane;
     if (half_id == 1) {
 #pragma unroll
