@@ -423,14 +423,14 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     // halves make the same number of steps (the second may have a last one without keys).
     //
     // A step of a half is two blocks of instructions with a barrier before each:
-    //   barrier 1: the loads that the half asked for a step ago have landed, the buffers of
-    //     the step before are free;
-    //   the block for the vector units: ask for the keys of the step after the next and the
-    //     values of the next step, read this step's first values from LDS, softmax;
-    //   barrier 2 (no data waits for it: it keeps the halves apart);
-    //   the block for the matrix cores: probabilities times values of this step, then keys
-    //     times queries of the next step, with every LDS read asked for one run of
-    //     products before its use.
+    //   barrier 1 (no data waits for it: it keeps the halves apart);
+    //   the block for the vector units: softmax of this step's scores; then the loads that
+    //     the wave asked for a step ago have to have landed;
+    //   barrier 2: this step's values and the next step's keys are in LDS for all;
+    //   the block for the matrix cores: ask for the keys of the step after the next and the
+    //     values of the next step (their buffers were read for the last time before
+    //     barrier 1), then probabilities times values of this step and keys times queries
+    //     of the next, every LDS read asked for one run of products before its use.
     // The second half passes one barrier more before its first step and is thereby half a
     // step behind: one half's softmax runs while the other half's products do.  Left to
     // themselves the two waves of a SIMD fall into step with each other, and the vector
@@ -476,7 +476,14 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       }
     };
     auto loads_landed = [] { __builtin_amdgcn_s_waitcnt(0x0F70); };  // vmcnt(0)
-    auto phase_barrier = [] {
+    // barrier 1 is the instruction alone: no data waits for it (and a fence would wait for
+    // the loads that are on their way)
+    auto turn_barrier = [] {
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto data_barrier = [] {
       __builtin_amdgcn_sched_barrier(0);
       __syncthreads();
       __builtin_amdgcn_sched_barrier(0);
@@ -522,11 +529,10 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       ask_values(j_of(0), pages_0, 0);
       if (1 < n_steps) ask_keys(j_of(1), pages_1, 1);
       loads_landed();
-      if (j_of(0) + KB > kv_len) clear_tail_values(j_of(0), 0);
       __syncthreads();
     }
     if constexpr (HALVES == 2) {
-      if (half_id == 1) phase_barrier();
+      if (half_id == 1) turn_barrier();
     }
     read_keys(fa, 0, 0);
     if constexpr (SUBS == 2) read_keys(fb, 0, 1);
@@ -537,11 +543,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       const int j0 = j_of(i), b = i & 1;
       int pages_3[SUBS];
       pages_of(j_of(i + 3), pages_3);
-      phase_barrier();  // 1
-      if (i + 2 < n_steps) ask_keys(j_of(i + 2), pages_2, b);
-      if (i + 1 < n_steps) ask_values(j_of(i + 1), pages_1, b ^ 1);
-      read_values(fa, b, 0);
-      __builtin_amdgcn_sched_barrier(0);
+      turn_barrier();  // 1
       // The tiles of a wave go together: a step that concerns one of them is worked on for
       // all (the masks take care of the others); only the last steps of a walk differ.
       bool active[RT];
@@ -552,17 +554,21 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       for (int rt = 0; rt < RT; ++rt) active[rt] = any;
       float alpha[RT];
       softmax_step(j0, s, active, pb, alpha);
-      // 2: the barrier instruction alone (no data waits for it, and a fence would wait for
-      // the loads that were asked for a moment ago)
       __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
+      loads_landed();
+      if (j0 + KB > kv_len) clear_tail_values(j0, b);
+      data_barrier();  // 2
       // (a step that concerns no tile has probabilities of zero, and after the last step
       // the scores of a step that does not exist are computed from what the buffer holds
       // and never looked at: the run of products has no branch)
+      __builtin_amdgcn_s_setprio(2);  // the products go first where both halves could issue
+      read_values(fa, b, 0);
+      if constexpr (SUBS == 2) read_values(fb, b, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (i + 2 < n_steps) ask_keys(j_of(i + 2), pages_2, b);
+      if (i + 1 < n_steps) ask_values(j_of(i + 1), pages_1, b ^ 1);
+      __builtin_amdgcn_sched_barrier(0);
       if constexpr (SUBS == 2) {
-        read_values(fb, b, 1);
-        __builtin_amdgcn_sched_barrier(0);
         probabilities_times_values(fa, 0);
         __builtin_amdgcn_sched_barrier(0);
         read_keys(fa, b ^ 1, 0);
@@ -582,8 +588,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
         keys_times_queries(fb, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
-      loads_landed();
-      if (i + 1 < n_steps && j_of(i + 1) + KB > kv_len) clear_tail_values(j_of(i + 1), b ^ 1);
+      __builtin_amdgcn_s_setprio(0);
 #pragma unroll
       for (int u = 0; u < SUBS; ++u) {
         pages_1[u] = pages_2[u];
@@ -591,7 +596,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       }
     }
     if constexpr (HALVES == 2) {
-      if (half_id == 0) phase_barrier();  // as many barriers as the second half
+      if (half_id == 0) turn_barrier();  // as many barriers as the second half
     }
   } else {
     // Without LDS: this block's values and the next block's keys (a second buffer) are asked
