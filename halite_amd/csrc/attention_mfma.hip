@@ -19,18 +19,19 @@
 // a lane's eight probabilities are eight consecutive keys, which is one 16-byte load of
 // the transposed values.
 //
-// Two kernels come from one body.  Decode tokens (segments of at most 16 rows) run one
+// Two kernels come from one file.  Decode tokens (segments of at most 16 rows) run one
 // item per wave, nothing goes through LDS, and the key range of a long request is cut
 // into many items.  Prompt portions run four items per workgroup (up to RT_BIG tiles
-// each): the waves walk the union of their key ranges together and load each block of
-// keys and values once, into LDS, one block ahead.  Such a workgroup has eight waves in two
-// halves: both halves hold the same four items, the first takes the even steps of the key
-// walk and the second the odd ones (so the causal work splits evenly), each with LDS
-// buffers of its own, and at the end the second half hands its sums to the first through
-// LDS, where they are joined by the log-sum-exp rule.  A workgroup then has a CU to itself
-// and is done in half the time, and since the host lists the longest walks first the
-// workgroups that start late are the short ones: a single prompt of 2,048 tokens, whose
-// 512 items of very different length used to start all at once, is balanced that way.
+// each): the waves walk the union of their key ranges together, and each block of keys and
+// values goes once from global memory straight into LDS, a step ahead.  Such a workgroup has
+// eight waves in two halves: both halves hold the same four items, the first takes the even
+// steps of the key walk and the second the odd ones (so the causal work splits evenly), each
+// with LDS buffers of its own, and at the end the second half hands its sums to the first
+// through LDS, where they are joined by the log-sum-exp rule.  A workgroup then has a CU to
+// itself and is done in half the time, and since the host lists the longest walks first the
+// workgroups that start late are the short ones.  The halves run half a step apart: the
+// softmax of one (vector units) against the products of the other (matrix cores); see the
+// loop.
 //
 // The pages are read in one of three ways: pages in the kernel's fragment order (TILED:
 // one contiguous KB per MFMA operand, see kv_key_offset in hal_common.h), row-major pages
@@ -52,6 +53,7 @@ static_assert(HAL_HEAD_DIM % 16 == 0 && HAL_HEAD_DIM >= 16 && HAL_HEAD_DIM <= 25
 #define KT ((D + 31) / 32)  // 32-wide steps over the head dimension for Q K^T
 #define DT (D / 16)         // 16-wide tiles of the head dimension for P V
 #define ITEM_INTS 8
+#define BIG_ITEM_INTS 16  // items of the kernel for long segments
 #define RESCALE_SLACK 8.0f  // in powers of two
 #define MERGE_FEW_PARTS 8   // up to here a merge item is one wave's work
 
@@ -140,21 +142,26 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   const int item = uniform(bx * WAVES + wave);
   // the item is asked for together with the live count (an index past the list's end is
   // clamped for the address only): one trip to memory instead of two
-  constexpr bool INLINE_SEG = !SHARED && RT == 1;
-  int pre[ITEM_INTS];
+  // (the kernel for long segments finds in its items of 16 what the other looks up: the
+  // segment's scalars and the key range that the workgroup's four items walk together)
+  constexpr bool INLINE_SEG = SHARED || RT == 1;
+  constexpr int STRIDE_INTS = SHARED ? BIG_ITEM_INTS : ITEM_INTS;
+  constexpr int PRE_INTS = SHARED ? 13 : ITEM_INTS;
+  int pre[PRE_INTS];
   if constexpr (INLINE_SEG) {
-    const int* ip = items + (size_t)(item < max_items ? item : max_items - 1) * ITEM_INTS;
+    const int* ip = items + (size_t)(item < max_items ? item : max_items - 1) * STRIDE_INTS;
 #pragma unroll
-    for (int i = 0; i < ITEM_INTS; ++i) pre[i] = ip[i];
+    for (int i = 0; i < PRE_INTS; ++i) pre[i] = ip[i];
   }
   const int n_items = *n_items_ptr;
   // SHARED: the four waves of a workgroup have items of one segment (the host lists them
-  // so) and walk the union of their key ranges together; the keys and values of a block
-  // are loaded once, by all four, into LDS.  A wave without an item of its own (the list
-  // ends, or the host padded the group) still loads and waits at the barriers.
+  // so, in whole runs of four, padded with items that have no rows and no keys) and walk
+  // the union of their key ranges together; the keys and values of a block are loaded once,
+  // by all four, into LDS.  A wave whose item is padding still loads and waits at the
+  // barriers.
   if (SHARED ? bx * WAVES >= n_items : item >= n_items) return;
   const bool have_item = item < n_items;
-  const int* it = items + (size_t)(have_item ? item : bx * WAVES) * ITEM_INTS;
+  const int* it = items + (size_t)(have_item ? item : bx * WAVES) * STRIDE_INTS;
   auto iv = [&](int i) {
     if constexpr (INLINE_SEG) return pre[i];
     else return it[i];
@@ -165,21 +172,14 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   const int partial = have_item ? uniform(iv(4)) : -1;
   int walk_begin = kv_begin, walk_end = kv_end;  // the keys this wave walks through
   if constexpr (SHARED) {
-    walk_begin = 0x7fffffff, walk_end = 0;
-    for (int w = 0; w < WAVES; ++w) {
-      if (bx * WAVES + w >= n_items) break;
-      const int* other = items + (size_t)(bx * WAVES + w) * ITEM_INTS;
-      const int b = uniform(other[2]), e = uniform(other[3]);
-      if (b < e) {
-        walk_begin = b < walk_begin ? b : walk_begin;
-        walk_end = e > walk_end ? e : walk_end;
-      }
-    }
+    walk_begin = uniform(pre[11]), walk_end = uniform(pre[12]);
     if (walk_begin >= walk_end) return;  // the same for all four waves
   }
   const int G = H / K;
   int q_start, q_len, kv_len;
-  if constexpr (INLINE_SEG) {
+  if constexpr (SHARED) {
+    q_start = uniform(pre[8]), q_len = uniform(pre[9]), kv_len = uniform(pre[10]);
+  } else if constexpr (INLINE_SEG) {
     q_start = uniform(pre[5]), q_len = uniform(pre[6]), kv_len = uniform(pre[7]);
   } else {
     q_start = uniform(seg_q_start[seg]), q_len = uniform(seg_q_len[seg]);
@@ -900,7 +900,7 @@ extern "C" int hal_attention_mfma_head_dim() { return D; }
 extern "C" int hal_attention_mfma_rows_per_big_item() { return 16 * RT_BIG; }
 
 // All arrays are device pointers.  `items` [max_items, 8] lists the work on segments of
-// at most 16 query rows (one tile per wave), `big_items` [max_big, 8] the work on longer
+// at most 16 query rows (one tile per wave), `big_items` [max_big, 16] the work on longer
 // segments (hal_attention_mfma_rows_per_big_item() rows per wave), `merges`
 // [max_merges, 8] the row tiles whose key range was cut.  counts = {items, big items,
 // merges} holds the live numbers, so a captured launch can serve varying counts.

@@ -265,12 +265,13 @@ class StepContext:
         if key not in self._plans:
             self.upload()
 
-            def piece(name, rows):
+            def piece(name, rows, ints=8):
                 off, _ = self._packer.offsets[plan.name + name]
-                return self._dev[off : off + rows * 8].view(rows, 8)
+                return self._dev[off : off + rows * ints].view(rows, ints)
 
             counts = self._view(plan.name + "_counts")
-            self._plans[key] = (plan, piece("_items", plan.cap_items), piece("_big", plan.cap_big),
+            self._plans[key] = (plan, piece("_items", plan.cap_items),
+                                piece("_big", plan.cap_big, attention_kernels.BIG_ITEM_INTS),
                                 piece("_merges", plan.cap_merges), counts)
         return self._plans[key]
 

@@ -23,6 +23,7 @@ KEYS_PER_BLOCK = 32
 MIN_SPLIT_KEYS = 128
 TARGET_WAVES = 2048
 WAVES_PER_GROUP = 4  # waves of a workgroup of the kernel for long segments: they share keys through LDS
+BIG_ITEM_INTS = 16  # an item of that kernel: 8 as the others, then what its workgroup would have to look up
 
 
 @dataclass
@@ -32,8 +33,11 @@ class AttentionPlan:
     ``items`` [n, 8]: segment, first row, first key, end key, first partial slot or -1,
     then the segment's first token, number of tokens and number of keys — tiles of 16 rows
     of segments with at most 16 rows (decode tokens);
-    ``big_items`` [n, 8] for longer segments: the first five the same, then the first rows
-    of the item's further tiles (-1: none), ``rows_big`` rows per item;
+    ``big_items`` [n, 16] for longer segments: the first five the same, then the first rows
+    of the item's further tiles (-1: none), ``rows_big`` rows per item; then the segment's
+    first token, number of tokens and number of keys, and the first and end key of the walk
+    of the item's run of four (a workgroup's waves), so that a workgroup knows all it needs
+    after one trip to memory;
     ``merges`` [n, 8]: segment, first row of a 16-row tile, first partial slot, number of
     partials, slots between partials, the segment's first token and number of tokens.
     A segment's first token is the sum of the lengths of the segments before it."""
@@ -117,7 +121,7 @@ def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, seg_scal
     keys) in those places."""
     n_tiles = len(seg_ids)
     if n_tiles == 0:
-        return np.zeros((0, 8), np.int32), np.zeros((0, 8), np.int32), first_slot
+        return np.zeros((0, BIG_ITEM_INTS if group > 1 else 8), np.int32), np.zeros((0, 8), np.int32), first_slot
     base = kv_b - kv_b % KEYS_PER_BLOCK
     n_pieces = np.maximum(1, -(-(kv_e - base) // chunk))
     n_items = int(n_pieces.sum())
@@ -154,21 +158,21 @@ def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, seg_scal
     merges[:, 4] = slots_per_tile
     merges[:, 5:7] = seg_scalars[merges[:, 0], :2]
     if group > 1:
-        items = _group_items(items, piece, group)
+        items = _group_items(items, piece, group, seg_scalars)
     else:
         # the longest key ranges first: the waves that run longest start earliest
         items = items[np.argsort(-(items[:, 3] - items[:, 2]), kind="stable")]
     return items, merges, first_slot + n_split * slots_per_tile
 
 
-def _group_items(items: np.ndarray, piece: np.ndarray, group: int) -> np.ndarray:
+def _group_items(items: np.ndarray, piece: np.ndarray, group: int, seg_scalars: np.ndarray) -> np.ndarray:
     """Orders items so that every run of ``group`` items (a workgroup's waves) belongs to
     one segment and to the same piece of neighbouring tiles, i.e. walks nearly the same
     keys; a run that cannot be filled is padded with items that have no rows and no keys.
     The runs with the longest walk come first."""
     n = len(items)
     if n == 0:
-        return np.zeros((0, 8), np.int32)
+        return np.zeros((0, BIG_ITEM_INTS), np.int32)
     order = np.lexsort((np.arange(n), piece, items[:, 0]))  # segment, then piece, then tile
     seg, pc = items[order, 0], piece[order]
     new_class = np.concatenate(([True], (seg[1:] != seg[:-1]) | (pc[1:] != pc[:-1])))
@@ -188,7 +192,12 @@ def _group_items(items: np.ndarray, piece: np.ndarray, group: int) -> np.ndarray
     first_key = np.where(live, runs[:, :, 2], np.iinfo(np.int32).max).min(axis=1)
     end_key = np.where(live, runs[:, :, 3], 0).max(axis=1)
     walk = np.where(live.any(axis=1), end_key - first_key, 0)
-    return runs[np.argsort(-walk, kind="stable")].reshape(total, 8)
+    wide = np.zeros((total // group, group, BIG_ITEM_INTS), dtype=np.int32)
+    wide[:, :, :8] = runs
+    wide[:, :, 8:11] = seg_scalars[runs[:, 0, 0]][:, None, :]
+    wide[:, :, 11] = np.where(live.any(axis=1), first_key, 0)[:, None]
+    wide[:, :, 12] = end_key[:, None]
+    return wide[np.argsort(-walk, kind="stable")].reshape(total, BIG_ITEM_INTS)
 
 
 def _group_tiles(seg_ids, rho0s, kv_b, kv_e, per_item: int):

@@ -16,7 +16,16 @@ def check_plan(plan, q_len, kv_len, group, window):
     for r in range(0, plan.n_big, 4):
         run = plan.big_items[r : r + 4]
         assert len(set(run[:, 0].tolist())) == 1 and run[0, 1] >= 0
-    for arr, is_big in ((plan.items, False), (plan.big_items, True)):
+    # the long segments' items are 16 wide: after the eight, the segment's first token, tokens
+    # and keys, and the first and end key that the run of four walks together
+    for r in range(0, plan.n_big, 4):
+        run = plan.big_items[r : r + 4]
+        seg = int(run[0, 0])
+        live = run[run[:, 3] > run[:, 2]]
+        assert (run[:, 8:11] == [int(sum(q_len[:seg])), int(q_len[seg]), int(kv_len[seg])]).all()
+        assert (run[:, 11] == live[:, 2].min()).all() and (run[:, 12] == live[:, 3].max()).all()
+        assert (run[:, 13:] == 0).all()
+    for arr, is_big in ((plan.items, False), (plan.big_items[:, :8], True)):
         for seg, rho0, b, e, partial, *more in arr.tolist():
             if is_big and rho0 < 0:
                 assert (b, e, partial, more) == (0, 0, -1, [-1, -1, -1])
