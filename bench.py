@@ -437,7 +437,7 @@ def main() -> int:
             runner.free(s)
         return dt, kv_tokens, gpu_s, fam
 
-    def prefill_run(T=args.prefill_tokens, families: bool = False):
+    def prefill_run(T=args.prefill_tokens, families: bool = False, portion: int = 0):
         ids = torch.randint(0, cfg.vocab_size, (T,), generator=gen).numpy().astype(np.int32)
         times, fam = [], None
         for i in range(5 if families else 4):
@@ -447,7 +447,7 @@ def main() -> int:
             if measure:
                 measure.__enter__()
             t0 = time.perf_counter()
-            portion = args.prefill_portion or T
+            portion = portion or args.prefill_portion or T
             for start in range(0, T, portion):  # the whole prompt, or one portion a step
                 end = min(start + portion, T)
                 logits = runner.step([Segment(s, start, ids[start:end], [end - start - 1] if end == T else [])])
@@ -578,10 +578,15 @@ def main() -> int:
         record["points"] = points
         record["prefill"] = prefill_run(families=True)
         if args.more_points:
-            for T in (8192, 16384):
+            for T in (512, 8192, 16384):
                 extra = prefill_run(T)
                 points[f"prefill_{T}"] = extra["value"]
                 points[f"prefill_{T}_frac"] = extra["frac"]
+            # the default prompt in portions of 512 tokens, one a step (what a scheduler with
+            # chunked_prefill_size=512 runs)
+            extra = prefill_run(portion=512)
+            points["prefill_in_portions_of_512"] = extra["value"]
+            points["prefill_in_portions_of_512_frac"] = extra["frac"]
         record["probe"] = probe_gpu(torch)
         record["roofline"]["frac_of_measured_read"] = round(achieved / (record["probe"]["read_gbps"] * 1e9), 4)
         record["prefill"]["frac_of_measured_gemm"] = round(
