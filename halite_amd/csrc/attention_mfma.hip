@@ -188,6 +188,28 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   const int pos0 = kv_len - q_len;  // position of the segment's first token
   const int* bt = block_table + (size_t)seg * bt_stride;
 
+  // A step of the walk takes KB keys: 32 without LDS, 32 or 64 with it (SUBS blocks of 32).
+  static_assert(KB == 32 || (SHARED && KB == 64), "keys per step");
+  constexpr int SUBS = KB / 32;
+  const int j_first = walk_begin & ~31;
+  // PAGE32: page numbers are looked up (scalar loads) well before the loads that need them
+  auto page_at = [&](int j0) {
+    if constexpr (PAGE32) return uniform(bt[(j0 < walk_end ? j0 : j_first) >> page_shift]);
+    else return 0;
+  };
+  // with LDS: the pages of this half's first three steps are asked for here, so that they
+  // are on their way while the query rows' addresses are worked out
+  int pages_0[SHARED ? SUBS : 1], pages_1[SHARED ? SUBS : 1], pages_2[SHARED ? SUBS : 1];
+  if constexpr (SHARED) {
+#pragma unroll
+    for (int u = 0; u < SUBS; ++u) {
+      const int j_mine = j_first + half_id * KB + 32 * u;
+      pages_0[u] = page_at(j_mine);
+      pages_1[u] = page_at(j_mine + KB * HALVES);
+      pages_2[u] = page_at(j_mine + 2 * KB * HALVES);
+    }
+  }
+
   const int col = lane % 16, quad = lane / 16;
   // this lane's query row in every row tile
   bool row_ok[RT];
@@ -316,16 +338,6 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       raw[w] &= (ja <= last_key ? 0x0000ffffu : 0u) | (ja + 1 <= last_key ? 0xffff0000u : 0u);
     }
     return __builtin_bit_cast(bf16x8, raw);
-  };
-
-  // A step of the walk takes KB keys: 32 without LDS, 32 or 64 with it (SUBS blocks of 32).
-  static_assert(KB == 32 || (SHARED && KB == 64), "keys per step");
-  constexpr int SUBS = KB / 32;
-  const int j_first = walk_begin & ~31;
-  // PAGE32: page numbers are looked up (scalar loads) well before the loads that need them
-  auto page_at = [&](int j0) {
-    if constexpr (PAGE32) return uniform(bt[(j0 < walk_end ? j0 : j_first) >> page_shift]);
-    else return 0;
   };
 
   // ---- one step's mask and online softmax, for every row tile: scores in, probabilities
@@ -519,12 +531,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
           o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[dt], pb[rt][u], o[rt][dt], 0, 0, 0);
     };
 
-    int pages_1[SUBS], pages_2[SUBS];  // of the next step and of the one after it
-    {
-      int pages_0[SUBS];
-      pages_of(j_of(0), pages_0);
-      pages_of(j_of(1), pages_1);
-      pages_of(j_of(2), pages_2);
+    {  // (pages_1, pages_2: of the next step and of the one after it)
       ask_keys(j_of(0), pages_0, 0);
       ask_values(j_of(0), pages_0, 0);
       if (1 < n_steps) ask_keys(j_of(1), pages_1, 1);
