@@ -580,3 +580,132 @@ def test_the_scheduler_serves_two_groups_of_pages_and_retracts(gpu, ahead):
     assert 0 < st.retractions <= 6, st.retractions
     assert runner.cache.idle()
     runner.cache.check()
+
+
+# -- a whole toy architecture, from config.json keys of its own to generated tokens --------
+
+
+class ToyMixConfig(BaseModel):
+    """The keys of the toy's config.json; nothing of it is known to the framework."""
+
+    architectures: list[str]
+    width: int
+    vocab: int
+    kinds: list[str]  # per layer: "mean" (the running mean above) or "attention"
+    heads: int
+    kv_heads: int
+    head_size: int
+    inner: int
+    eps: float
+    theta: float
+    context: int
+    window: int | None = None  # of the attention layers after the first
+    torch_dtype: str | None = None
+
+
+def toy_mix_spec(cfg: ToyMixConfig) -> ModelSpec:
+    norm = PartSpec(kind="rmsnorm", size=cfg.width, eps=cfg.eps)
+    ff = PartSpec(kind="gated", hidden_size=cfg.width, intermediate_size=cfg.inner, activation="silu")
+    layers, seen_attention = {}, False
+    for i, kind in enumerate(cfg.kinds):
+        if kind == "mean":
+            mixer = PartSpec(kind="running_mean", hidden_size=cfg.width)
+        else:
+            mixer = PartSpec(kind="attention", hidden_size=cfg.width, n_heads=cfg.heads, n_kv_heads=cfg.kv_heads,
+                             head_dim=cfg.head_size, scale=cfg.head_size**-0.5, position="rope",
+                             window=cfg.window if seen_attention else None)
+            seen_attention = True
+        layers[f"L{i}"] = LayerSpec(arrangement="pre_norm", parts=dict(mixer_norm=norm, mixer=mixer, ff_norm=norm, ff=ff))
+    return ModelSpec(
+        architecture="ToyMixForCausalLM", vocab_size=cfg.vocab, hidden_size=cfg.width, max_positions=cfg.context,
+        embedding=PartSpec(kind="embedding", vocab_size=cfg.vocab, size=cfg.width),
+        positions={"rope": PartSpec(kind="rope", head_dim=cfg.head_size, rotary_dim=cfg.head_size, theta=cfg.theta,
+                                    interleaved=False, max_positions=cfg.context)},
+        layers=layers, order=[LayerRun(layer=name) for name in layers], final_norm=norm,
+        head=PartSpec(kind="linear_head", vocab_size=cfg.vocab, size=cfg.width, tied=True),
+    )
+
+
+def toy_mix_weight_map(cfg: ToyMixConfig) -> dict:
+    # one table for both kinds of layer: a layer takes the names of the parameters it has
+    return {
+        "toy.table": "embedding.weight",
+        "toy.#.before_mixer": "layers.#.mixer_norm.weight",
+        "toy.#.mean": "layers.#.mixer.w.weight",
+        "toy.#.q": "layers.#.mixer.q.weight",
+        "toy.#.k": "layers.#.mixer.k.weight",
+        "toy.#.v": "layers.#.mixer.v.weight",
+        "toy.#.o": "layers.#.mixer.out.weight",
+        "toy.#.before_ff": "layers.#.ff_norm.weight",
+        "toy.#.gate": "layers.#.ff.linear_gate.weight",
+        "toy.#.up": "layers.#.ff.linear_proj.weight",
+        "toy.#.down": "layers.#.ff.linear_out.weight",
+        "toy.last_norm": "final_norm.weight",
+    }
+
+
+TOY_MIX = dict(architectures=["ToyMixForCausalLM"], width=64, vocab=211, kinds=["mean", "attention", "attention", "mean"],
+               heads=4, kv_heads=2, head_size=16, inner=88, eps=1e-5, theta=10000.0, context=256, window=24)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_architecture_from_its_config_file_to_generated_tokens(gpu, dtype, tmp_path):
+    """An architecture of its own (config keys, layer kinds that differ from layer to layer,
+    tensor names) is registered here; the framework's folder writer, loader, engine,
+    scheduler and sampler then serve it as they serve the built-in one."""
+    import json
+
+    from halite_amd.config.registry import Architecture, register_architecture
+    from halite_amd.engine.engine import InferenceEngine
+    from halite_amd.weights import WeightError
+    from halite_amd.weights.random_init import write_random_model
+
+    arch = register_architecture(Architecture("ToyMixForCausalLM", ToyMixConfig, toy_mix_spec, toy_mix_weight_map))
+    try:
+        found, cfg = parse_config(dict(TOY_MIX))
+        assert found is arch and cfg.kinds == TOY_MIX["kinds"]
+        folder = write_random_model(str(tmp_path / "toy"), cfg, seed=3, dtype=dtype, std=0.08)
+        with open(f"{folder}/config.json") as f:
+            assert json.load(f)["kinds"] == TOY_MIX["kinds"]
+        server = ServerConfig(kv_cache_num_tokens=512, page_size=16, max_seqs_per_forward=4, chunked_prefill_size=16,
+                              max_tokens_per_forward=32, max_prefill_tokens=32)
+        engine = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype=dtype))
+        model = engine.model_runner.model
+        assert [type(model.layers[n].mixer).__name__ for n in model.spec.layers] == ["RunningMean", "Attention", "Attention", "RunningMean"]
+        assert len(engine.model_runner.cache.groups) == 2  # all keys; a window of them
+        rope_p = dict(rotary_dim=16, theta=10000.0, interleaved=False)
+
+        def mean(part, x, positions, i, run, memo):
+            return (torch.cumsum(x, 0) / torch.arange(1, x.shape[0] + 1)[:, None]) @ part.w_weight.float().cpu().T
+
+        def att(part, x, positions, i, run, memo):
+            return plain_attention_layer(part, x, positions, rope_p)[0]
+
+        mixers = {"L0": mean, "L1": att, "L2": att, "L3": mean}
+        prompts = [[int(t) % 211 for t in tiny.random_tokens(tiny.TINY_A, n, 60 + n)] for n in (41, 3, 70)]
+        results = engine.infer_batch([(p, {"max_new_tokens": 12, "temperature": 0.0}) for p in prompts])
+        margin = 1e-4 if dtype == "float32" else 0.06
+        for p, r in zip(prompts, results):
+            out = r.output_ids[0]
+            assert len(out) == 12
+            logits = plain_model(model, p + out, mixers)
+            for j, tok in enumerate(out):  # the chosen token is the plain model's best, or within rounding of it
+                row = logits[len(p) - 1 + j]
+                assert float(row.max() - row[tok]) <= margin * max(1.0, float(row.abs().max())), (len(p), j)
+        assert engine.stats.prefill_tokens >= sum(len(p) for p in prompts) and engine.model_runner.cache.idle()
+        # the loader's one error speaks the toy's tensor names
+        from safetensors import safe_open
+        from safetensors.torch import save_file
+
+        with safe_open(f"{folder}/model.safetensors", "pt") as f:
+            tensors = {k: f.get_tensor(k) for k in f.keys()}
+        tensors.pop("toy.L0.mean")
+        tensors["toy.L3.q"] = torch.zeros(2, 2)
+        save_file(tensors, f"{folder}/model.safetensors")
+        with pytest.raises(WeightError) as e:
+            InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype=dtype))
+        assert "toy.L0.mean" in str(e.value) and "toy.L3.q" in str(e.value)
+    finally:
+        from halite_amd.config.registry import ARCHITECTURES
+
+        ARCHITECTURES.pop("ToyMixForCausalLM", None)
