@@ -4,6 +4,7 @@
 // type of activations and cache (float or bf16).
 #include "hal_common.h"
 #include "hal_api.h"
+#include <stdlib.h>
 
 // ---------------------------------------------------------------------------------
 // h[t, :] = table[ids[t], :]  (float32 residual stream)
@@ -587,6 +588,184 @@ __global__ void rope_append_vec_kernel(T* __restrict__ qkv, int row_stride,
   }
 }
 
+// The same for steps of many tokens (prompt portions): a workgroup takes eight consecutive
+// tokens.  Their positions and pages are looked up once, by eight threads (one chain of
+// trips to memory per eight tokens instead of one per token); the rotations of all eight
+// are one pool of work items; and where the eight are one request's positions 8j .. 8j+7
+// their values go through LDS, in with 16-byte loads and out eight slots of a dimension
+// at a time (a page keeps eight consecutive slots of a dimension side by side in both
+// layouts).  A token whose position lies outside the table is left alone and one whose
+// page is not valid is rotated and not appended, as in the kernels above.
+#define RG_TOKENS 8
+#define RG_THREADS 1024
+template <typename T>
+__global__ void __launch_bounds__(RG_THREADS)
+rope_append_group_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
+                         const int* __restrict__ token_seg, const int* __restrict__ block_table,
+                         int bt_stride, const float* __restrict__ cos_t,
+                         const float* __restrict__ sin_t, int table_len, T* __restrict__ k_pages,
+                         T* __restrict__ v_pages, int n_tokens, int H, int K, int D, int rot,
+                         int interleaved, int page_size, int n_pages, bool tiled) {
+  __shared__ int s_pos[RG_TOKENS], s_off[RG_TOKENS];
+  __shared__ int s_lead[RG_TOKENS];  // 0: the token writes its own values; 1: its run's first does; 2: it is that first
+  __shared__ long long s_page[RG_TOKENS];
+  extern __shared__ __align__(16) unsigned char rg_values[];  // [8 tokens][K * D] of T
+  const int t0 = blockIdx.x * RG_TOKENS;
+  const int n = n_tokens - t0 < RG_TOKENS ? n_tokens - t0 : RG_TOKENS;
+  const int half = rot / 2;
+  if (threadIdx.x < RG_TOKENS) {
+    const int i = threadIdx.x;
+    int pos = -1, off = 0, lead = 0;
+    long long page = -1;
+    if (i < n) {
+      const int t = t0 + i;
+      pos = positions[t];
+      const int seg = token_seg[t];
+      const bool ok = pos >= 0 && (rot == 0 || pos < table_len);
+      if (ok) {
+        page = block_table[(size_t)seg * bt_stride + pos / page_size];
+        off = pos % page_size;
+        if (page < 0 || page >= n_pages) page = -1;
+        const int first = t - off % 8;  // where the first token of this token's run of eight would be
+        if (page >= 0 && first >= 0 && first + 7 < n_tokens &&
+            token_seg[first] == seg && token_seg[first + 7] == seg &&
+            positions[first] == pos - off % 8 && positions[first + 7] == pos - off % 8 + 7)
+          lead = off % 8 == 0 ? 2 : 1;
+      } else {
+        pos = -1;
+      }
+    }
+    s_pos[i] = pos, s_off[i] = off, s_lead[i] = lead, s_page[i] = page;
+  }
+  __syncthreads();
+
+  // ---- q and k: rotate in place, k also into its page --------------------------------
+  const int cph = interleaved ? rot / 8 : half / 8;  // work items of a head
+  const int per_token = (H + K) * cph;
+  for (int item = threadIdx.x; item < n * per_token; item += blockDim.x) {
+    const int i = item / per_token, idx = item % per_token;
+    const int pos = s_pos[i];
+    if (pos < 0) continue;
+    const long long page = s_page[i];
+    const int off = s_off[i];
+    T* row = qkv + (size_t)(t0 + i) * row_stride;
+    const float* cp = cos_t + (size_t)pos * half;
+    const float* sp = sin_t + (size_t)pos * half;
+    const int head = idx / cph;
+    T* hp = row + (size_t)head * D;
+    T* kp = (head >= H && page >= 0) ? k_pages + ((size_t)page * K + (head - H)) * page_size * D
+                                     : nullptr;
+    if (!interleaved) {
+      const int j = (idx % cph) * 8;
+      float a[2][4], b[2][4], c[2][4], sn[2][4], y0[2][4], y1[2][4];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        load4(hp + j + 4 * u, a[u]);
+        load4(hp + j + half + 4 * u, b[u]);
+        load4(cp + j + 4 * u, c[u]);
+        load4(sp + j + 4 * u, sn[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          y0[u][e] = a[u][e] * c[u][e] - b[u][e] * sn[u][e];
+          y1[u][e] = a[u][e] * sn[u][e] + b[u][e] * c[u][e];
+        }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        store4(hp + j + 4 * u, y0[u]);
+        store4(hp + j + half + 4 * u, y1[u]);
+        if (kp) {
+          store4(kp + kv_key_offset(tiled, page_size, D, off, j + 4 * u), y0[u]);
+          store4(kp + kv_key_offset(tiled, page_size, D, off, j + half + 4 * u), y1[u]);
+        }
+      }
+    } else {
+      const int e0 = (idx % cph) * 8, j = e0 / 2;
+      float a[2][4], c[4], sn[4], y[2][4];
+      load4(hp + e0, a[0]);
+      load4(hp + e0 + 4, a[1]);
+      load4(cp + j, c);
+      load4(sp + j, sn);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float x0 = a[e / 2][(2 * e) % 4], x1 = a[e / 2][(2 * e) % 4 + 1];
+        y[e / 2][(2 * e) % 4] = x0 * c[e] - x1 * sn[e];
+        y[e / 2][(2 * e) % 4 + 1] = x0 * sn[e] + x1 * c[e];
+      }
+      store4(hp + e0, y[0]);
+      store4(hp + e0 + 4, y[1]);
+      if (kp) {
+        store4(kp + kv_key_offset(tiled, page_size, D, off, e0), y[0]);
+        store4(kp + kv_key_offset(tiled, page_size, D, off, e0 + 4), y[1]);
+      }
+    }
+  }
+  // dimensions of k beyond the rotated ones pass through
+  const int rest8 = (D - rot) / 8;
+  for (int item = threadIdx.x; item < n * K * rest8; item += blockDim.x) {
+    const int i = item / (K * rest8), idx = item % (K * rest8);
+    if (s_pos[i] < 0 || s_page[i] < 0) continue;
+    const int g = idx / rest8, d = rot + (idx % rest8) * 8;
+    const T* row = qkv + (size_t)(t0 + i) * row_stride;
+    float a[2][4];
+    load4(row + (size_t)(H + g) * D + d, a[0]);
+    load4(row + (size_t)(H + g) * D + d + 4, a[1]);
+    T* kp = k_pages + ((size_t)s_page[i] * K + g) * page_size * D;
+    store4(kp + kv_key_offset(tiled, page_size, D, s_off[i], d), a[0]);
+    store4(kp + kv_key_offset(tiled, page_size, D, s_off[i], d + 4), a[1]);
+  }
+
+  // ---- values ---------------------------------------------------------------------
+  // A token whose run of eight positions (from a multiple of eight on) is all in this step
+  // leaves its values to the run's first token; that token's workgroup brings the eight rows
+  // into LDS and writes eight slots of every dimension at a time.  (The run's other tokens
+  // may be the next workgroup's: their values are only read.)
+  const int KD = K * D;
+  for (int i = 0; i < n; ++i) {
+    if (s_lead[i] != 2) continue;  // the same for the whole workgroup
+    T* staged = (T*)rg_values;
+    constexpr int PER = 16 / sizeof(T);  // elements of a 16-byte piece
+    __syncthreads();  // (the run before this one has been written)
+    for (int c = threadIdx.x; c < RG_TOKENS * KD / PER; c += blockDim.x) {
+      const int r = c / (KD / PER), e = (c % (KD / PER)) * PER;
+      *(uint4*)(staged + (size_t)r * KD + e) =
+          *(const uint4*)(qkv + (size_t)(t0 + i + r) * row_stride + (size_t)(H + K) * D + e);
+    }
+    __syncthreads();
+    const long long page = s_page[i];
+    const int off = s_off[i];
+    for (int idx = threadIdx.x; idx < KD; idx += blockDim.x) {
+      const int g = idx / D, d = idx % D;
+      __attribute__((aligned(16))) T vals[RG_TOKENS];
+#pragma unroll
+      for (int r = 0; r < RG_TOKENS; ++r) vals[r] = staged[(size_t)r * KD + idx];
+      T* vp = v_pages + ((size_t)page * K + g) * D * page_size +
+              kv_value_offset(tiled, page_size, D, off, d);
+      if constexpr (sizeof(T) == 2) {
+        *(uint4*)vp = *(const uint4*)vals;
+      } else {
+        *(uint4*)vp = *(const uint4*)vals;
+        *(uint4*)(vp + 4) = *(const uint4*)(vals + 4);
+      }
+    }
+  }
+  const int d8 = D / 8;
+  for (int item = threadIdx.x; item < n * K * d8; item += blockDim.x) {
+    const int i = item / (K * d8), idx = item % (K * d8);
+    if (s_pos[i] < 0 || s_page[i] < 0 || s_lead[i] != 0) continue;
+    const int g = idx / d8, d = (idx % d8) * 8;
+    __attribute__((aligned(16))) T vals[8];
+    const uint4* vr = (const uint4*)(qkv + (size_t)(t0 + i) * row_stride + (size_t)(H + K + g) * D + d);
+#pragma unroll
+    for (int u = 0; u < (int)(sizeof(T) / 2); ++u) ((uint4*)vals)[u] = vr[u];
+    T* vp = v_pages + ((size_t)s_page[i] * K + g) * D * page_size;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) vp[kv_value_offset(tiled, page_size, D, s_off[i], d + e)] = vals[e];
+  }
+}
+
 extern "C" int hal_rope_append(void* qkv, int dtype, int row_stride, const int* positions,
                                const int* token_seg, const int* block_table, int bt_stride,
                                const float* cos_t, const float* sin_t, int table_len,
@@ -606,6 +785,26 @@ extern "C" int hal_rope_append(void* qkv, int dtype, int row_stride, const int* 
               "(page %d, head %d)", page_size, D);
   const bool vec = D % 8 == 0 && row_stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
                    (interleaved ? rot % 8 == 0 : rot % 16 == 0);
+  // many tokens: eight to a workgroup (the values of eight tokens must fit LDS)
+  const size_t group_lds = (size_t)RG_TOKENS * K * D * (dtype == HAL_F32 ? 4 : 2);
+  // (measured with 32 + 8 + 8 heads of 128: the same at 1,024 tokens, 14 against 18 us at
+  // 2,048, 42 against 62 us at 8,192; below that the kernels above, which have more
+  // workgroups in flight, are faster)
+  if (vec && K > 0 && n_tokens >= 1536 && page_size % 8 == 0 && rot > 0 && group_lds <= 48 * 1024) {
+    const dim3 grid((n_tokens + RG_TOKENS - 1) / RG_TOKENS);
+    if (dtype == HAL_F32)
+      hipLaunchKernelGGL(rope_append_group_kernel<float>, grid, dim3(RG_THREADS), group_lds, stream,
+                         (float*)qkv, row_stride, positions, token_seg, block_table, bt_stride,
+                         cos_t, sin_t, table_len, (float*)k_pages, (float*)v_pages, n_tokens, H, K,
+                         D, rot, interleaved, page_size, n_pages, tiled != 0);
+    else
+      hipLaunchKernelGGL(rope_append_group_kernel<bf16_t>, grid, dim3(RG_THREADS), group_lds, stream,
+                         (bf16_t*)qkv, row_stride, positions, token_seg, block_table, bt_stride,
+                         cos_t, sin_t, table_len, (bf16_t*)k_pages, (bf16_t*)v_pages, n_tokens, H,
+                         K, D, rot, interleaved, page_size, n_pages, tiled != 0);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   if (vec) {
     int items = (H + K) * (rot / 8) / (interleaved ? 1 : 2);
     if (K * (D / 8) > items) items = K * (D / 8);

@@ -156,15 +156,11 @@ def from_tiled(kt, vt):
     return kp, vp
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("interleaved", [False, True])
-@pytest.mark.parametrize("H,K,D,rot,page,tiled", [
-    (4, 2, 16, 16, 4, False), (6, 2, 48, 48, 16, False), (3, 1, 32, 16, 8, False), (8, 8, 128, 128, 64, False),
-    (8, 8, 128, 128, 64, True), (3, 1, 32, 16, 32, True), (4, 2, 64, 64, 32, True), (2, 1, 96, 40, 64, True)])
-def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page, tiled):
+def rope_case(gpu, dtype, interleaved, H, K, D, rot, page, tiled, lens, starts):
     dt = DT[dtype]
-    n_seg, table_w = 4, -(-64 // page)
-    lens, starts = [5, 1, 9, 20], [3, 40, 0, 6]  # runs of eight aligned positions and ragged ends
+    n_seg = len(lens)
+    reach = max(s + n for s, n in zip(starts, lens))  # positions in use
+    table_w = -(-reach // page)
     T = sum(lens)
     qkv = rnd(T, (H + 2 * K) * D, seed=9).to(dt)
     positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).to(torch.int32)
@@ -172,7 +168,7 @@ def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page, tiled):
     n_pages = n_seg * table_w + 8
     bt = torch.randperm(n_pages - 1, generator=torch.Generator().manual_seed(1))[: n_seg * table_w].view(n_seg, table_w) + 1
     inv = P.inverse_frequencies(rot, 10000.0)
-    cos, sin = P.rotation_table(torch.arange(64), inv)
+    cos, sin = P.rotation_table(torch.arange(reach), inv)
     kp = torch.zeros(n_pages, K, page, D, dtype=dt, device=gpu)
     vp = torch.zeros(n_pages, K, D, page, dtype=dt, device=gpu)
     got = qkv.to(gpu).clone()
@@ -188,19 +184,42 @@ def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page, tiled):
     rk = torch.cat((rotate(k[..., :rot], c, s), k[..., rot:]), -1)
     tol = 1e-6 if dtype == "float32" else 8e-3
     close(got[:, : H * D].view(T, H, D), rq, tol, "rotated q")
+    close(got[:, H * D : (H + K) * D].view(T, K, D), rk, tol, "rotated k")
     assert torch.equal(got[:, (H + K) * D :].cpu(), qkv[:, (H + K) * D :])  # v untouched
     kpc, vpc = kp.float().cpu(), vp.float().cpu()
     if tiled:
         kpc, vpc = from_tiled(kpc, vpc)
+    pg = bt[token_seg.long(), positions.long() // page]
+    off = positions.long() % page
+    close(kpc[pg, :, off, :], rk, tol, "k pages")
+    assert torch.equal(vpc[pg, :, :, off], v.to(dt).float())
     written = torch.zeros(n_pages, page, dtype=torch.bool)
-    for t in range(T):
-        pos, seg = int(positions[t]), int(token_seg[t])
-        pg, off = int(bt[seg, pos // page]), pos % page
-        close(kpc[pg, :, off, :], rk[t], tol, "k page")
-        assert torch.equal(vpc[pg, :, :, off], v[t].to(dt).float())
-        written[pg, off] = True
+    written[pg, off] = True
     assert float(kpc.abs().sum(dim=(1, 3))[~written].sum()) == 0  # nothing else was written
     assert float(vpc.abs().sum(dim=(1, 2))[~written].sum()) == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("H,K,D,rot,page,tiled", [
+    (4, 2, 16, 16, 4, False), (6, 2, 48, 48, 16, False), (3, 1, 32, 16, 8, False), (8, 8, 128, 128, 64, False),
+    (8, 8, 128, 128, 64, True), (3, 1, 32, 16, 32, True), (4, 2, 64, 64, 32, True), (2, 1, 96, 40, 64, True)])
+def test_rope_append(gpu, dtype, interleaved, H, K, D, rot, page, tiled):
+    # runs of eight aligned positions and ragged ends
+    rope_case(gpu, dtype, interleaved, H, K, D, rot, page, tiled, [5, 1, 9, 20], [3, 40, 0, 6])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("H,K,D,rot,page,tiled", [
+    (6, 2, 48, 48, 16, False), (8, 8, 128, 128, 64, True), (4, 2, 64, 64, 32, True), (2, 1, 96, 40, 64, True),
+    (3, 1, 32, 16, 8, False)])
+def test_rope_append_of_many_tokens(gpu, dtype, interleaved, H, K, D, rot, page, tiled):
+    """Steps of many tokens take a kernel of their own (eight tokens to a workgroup): runs of
+    eight positions that start inside one workgroup's tokens and end in the next one's,
+    segments that end in the middle of a workgroup's tokens, a last workgroup with fewer."""
+    rope_case(gpu, dtype, interleaved, H, K, D, rot, page, tiled, [705, 1, 303, 611, 5], [3, 40, 0, 26, 8])
+    rope_case(gpu, dtype, interleaved, H, K, D, rot, page, tiled, [2048], [512])
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 32])
