@@ -20,8 +20,12 @@
 // the transposed values.
 //
 // Two kernels come from one file.  Decode tokens (segments of at most 16 rows) run one
-// item per wave, nothing goes through LDS, and the key range of a long request is cut
-// into many items.  Prompt portions run four items per workgroup (up to RT_BIG tiles
+// item per wave and keys and values do not go through LDS: a workgroup takes a piece of a
+// tile's key range, its four waves a quarter of the piece each (four items), and their
+// sums are joined through LDS at the end, so that a range of one piece needs neither partial
+// results in memory nor the merge kernel, and a long range, cut into about as many pieces
+// as there are compute units to take them, a quarter as many partial results as waves.
+// Prompt portions run four items per workgroup (up to RT_BIG tiles
 // each): the waves walk the union of their key ranges together, and each block of keys and
 // values goes once from global memory straight into LDS, a step ahead.  Such a workgroup has
 // eight waves in two halves: both halves hold the same four items, the first takes the even
@@ -119,6 +123,12 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                       int page_size, int page_shift, float scale_log2e, int window,
                       int max_items) {
   static_assert(HALVES == 1 || (SHARED && HALVES == 2), "only the kernel with LDS has two halves");
+  // JOIN (the kernel without LDS for keys): the four items of a workgroup are four pieces of
+  // one tile's key range (the host lists them so, in whole runs of four, the last may be
+  // empty); their sums are joined through LDS at the end and the first wave writes the
+  // result, to the output or to the partial slot that its item names.
+  constexpr bool JOIN = !SHARED;
+  static_assert(!JOIN || RT == 1, "pieces are joined in the kernel for one tile per wave");
   // wave: within its half (it names the item and the fragments the wave loads)
   const int lane = threadIdx.x % HAL_WAVE;
   const int wave = __builtin_amdgcn_readfirstlane((threadIdx.x / HAL_WAVE) % WAVES);
@@ -159,7 +169,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   // the union of their key ranges together; the keys and values of a block are loaded once,
   // by all four, into LDS.  A wave whose item is padding still loads and waits at the
   // barriers.
-  if (SHARED ? bx * WAVES >= n_items : item >= n_items) return;
+  if (bx * WAVES >= n_items) return;  // items come in whole runs of four
   const bool have_item = item < n_items;
   const int* it = items + (size_t)(have_item ? item : bx * WAVES) * STRIDE_INTS;
   auto iv = [&](int i) {
@@ -706,12 +716,48 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     }
   }
 
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    // the denominator is spread over the four lanes that share a row
-    float lt = l[rt];
+  if constexpr (JOIN) {
+    // lane to lane: the four waves have the same rows in the same lanes.  Joined by the
+    // log-sum-exp rule, in wave order.
+    constexpr int JV = DT * 4 + 2;
+    __shared__ float joined[WAVES - 1][JV][HAL_WAVE];
+    float lt = l[0];
     lt += __shfl_xor(lt, 16, HAL_WAVE);
     lt += __shfl_xor(lt, 32, HAL_WAVE);
+    if (wave > 0) {
+      joined[wave - 1][0][lane] = m[0];
+      joined[wave - 1][1][lane] = lt;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) joined[wave - 1][2 + dt * 4 + r][lane] = o[0][dt][r];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < WAVES - 1; ++w) {
+      const float m1 = joined[w][0][lane], l1 = joined[w][1][lane];
+      const float m_new = fmaxf(m[0], m1);
+      const float m_sub = m_new == -INFINITY ? 0.f : m_new;
+      const float a0 = fast_exp2(m[0] - m_sub), a1 = fast_exp2(m1 - m_sub);
+      lt = lt * a0 + l1 * a1;
+      m[0] = m_new;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[0][dt][r] = o[0][dt][r] * a0 + joined[w][2 + dt * 4 + r][lane] * a1;
+    }
+    l[0] = lt;
+  }
+
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    // the denominator is spread over the four lanes that share a row (joined pieces: it is whole)
+    float lt = l[rt];
+    if constexpr (!JOIN) {
+      lt += __shfl_xor(lt, 16, HAL_WAVE);
+      lt += __shfl_xor(lt, 32, HAL_WAVE);
+    }
     if (!row_ok[rt]) continue;
     if (partial < 0) {
       const float inv = lt > 0.f ? 1.0f / lt : 0.f;
@@ -954,6 +1000,8 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
                        scale_log2e, window, MAX);                                                 \
     HAL_LAUNCH_CHECK();                                                                           \
   }
+  HAL_REQUIRE(max_items % WAVES == 0 && max_big % WAVES == 0,
+              "hal_attention_mfma: items come in runs of %d, a workgroup's waves", WAVES);
   if (max_items > 0) LAUNCH_ATTENTION(1, false, 32, 1, items, max_items, counts)
   if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, true, KB_BIG, HALVES_BIG, big_items, max_big, counts + 1)
 #undef LAUNCH_ATTENTION

@@ -111,7 +111,10 @@ int hal_sample_spread(const float* logits, int ld, int n_rows, int V, const floa
 int hal_attention_mfma_head_dim();
 int hal_attention_mfma_rows_per_big_item();
 // merge_parts: the most partial results that any merge item joins, or 0 if not known (the
-// kernel for many partials is taken then).
+// kernel for many partials is taken then).  Items of both lists come in runs of four, a
+// workgroup's waves (max_items and max_big are multiples of four): the one-tile items of a
+// run are four pieces of one piece of a tile's key range (the last may be empty), whose sums
+// the kernel joins itself, into the output or the run's partial slot.
 int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_stride,
                        const int* items, int max_items, const int* big_items, int max_big,
                        const int* merges, int max_merges, const int* counts,

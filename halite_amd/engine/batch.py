@@ -69,10 +69,9 @@ class StaticLayout:
     step lies at the same address step after step: what a captured graph needs.
     Made for decode-only steps of ``n_segs`` requests."""
 
-    def __init__(self, n_segs: int, bt_width: dict[int, int], max_items: int, device):
+    def __init__(self, n_segs: int, bt_width: dict[int, int], device):
         self.n_segs = n_segs
         self.bt_width = dict(bt_width)
-        self.max_items = max_items
         self.device = device
         self.buffer: torch.Tensor | None = None
         self.size = 0
@@ -198,10 +197,16 @@ class StepContext:
         self._plan_host[key] = plan
         plan.name = f"plan{len(self._plan_host)}"
         if self._dev is None:
-            cap = self.static.max_items if self.static is not None else None
-            if cap is not None:  # decode only: no long segments
-                plan.cap_items, plan.cap_merges, plan.cap_partials = cap, min(cap, self.n_segs), cap
-                plan.max_parts = 0  # the launches are recorded once for all later plans
+            cap = None
+            if self.static is not None:  # decode only: room for whatever the planner makes of these requests
+                tiles = self.n_segs * -(-(n_heads // n_kv_heads) // attention_kernels.ROWS_PER_ITEM)
+                most = attention_kernels.pieces_per_tile(tiles, n_kv_heads)
+                cap = plan.cap_items = attention_kernels.WAVES_PER_GROUP * tiles * most
+                # the launches are recorded once for all later plans: none of them cuts a key
+                # range into more pieces than this (into none at all where the tiles are many,
+                # and then nothing is merged)
+                plan.cap_merges, plan.cap_partials = (tiles, tiles * most) if most > 1 else (0, 0)
+                plan.max_parts = most
             self._packer.add(plan.name + "_items", plan.items, None if cap is None else cap * 8)
             self._packer.add(plan.name + "_big", plan.big_items)
             self._packer.add(plan.name + "_merges", plan.merges, None if cap is None else plan.cap_merges * 8)

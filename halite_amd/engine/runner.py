@@ -87,12 +87,10 @@ class ModelRunner:
         for pos in model.positions.values():
             if hasattr(pos, "tables"):
                 pos.tables(self.context_len)
-        self._graphs: dict[int, dict] = {}
+        self._graphs: dict[int, dict] = {}  # batch size -> layout and recorded decode step
         self._ahead = None  # (requests and positions, cache version, context) of a step put together ahead
         self.steps_taken_ahead = 0
         self._token_feed = None
-        kv_heads = [n.n_kv_heads for n in needs.values()] or [1]
-        self._min_kv_heads = min(kv_heads)
         # graphs replay a model only if every part of it reads what varies on the device
         self.graphs_allowed = (
             self.server_config.use_cudagraph and self.device.type == "cuda"
@@ -358,8 +356,7 @@ class ModelRunner:
         entry = self._graphs.get(B)
         if entry is None:
             width = {g.group_id: -(-self.context_len // g.page_size) for g in self.cache.groups}
-            cap = attention_kernels.TARGET_WAVES // self._min_kv_heads + 2 * B + 8
-            entry = self._graphs[B] = {"layout": StaticLayout(B, width, cap, self.device), "graph": None}
+            entry = self._graphs[B] = {"layout": StaticLayout(B, width, self.device), "graph": None}
         ctx = ahead
         if ctx is None:
             ctx = StepContext(segments, self.cache, self.device, self._staging, static=entry["layout"])

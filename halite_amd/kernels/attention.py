@@ -21,18 +21,34 @@ from . import library, ops
 ROWS_PER_ITEM = 16
 KEYS_PER_BLOCK = 32
 MIN_SPLIT_KEYS = 128
-TARGET_WAVES = 2048
-WAVES_PER_GROUP = 4  # waves of a workgroup of the kernel for long segments: they share keys through LDS
-BIG_ITEM_INTS = 16  # an item of that kernel: 8 as the others, then what its workgroup would have to look up
+TARGET_WAVES_LONG = 1024
+WAVES_PER_GROUP = 4  # waves of a workgroup
+BIG_ITEM_INTS = 16  # an item of the kernel for long segments: 8 as the others, then what its workgroup would have to look up
+# One-tile items: a tile's key range is cut into pieces, one per workgroup, of which there
+# should be about one per compute unit (what a compute unit has in flight bounds what it
+# reads a second, so an even share each counts for more than many waves: measured), and no
+# piece shorter than this many keys (below, a second piece and the merge cost more than the
+# shorter walk saves).
+COMPUTE_UNITS = 256
+MIN_PIECE_KEYS = 384
+
+
+def pieces_per_tile(n_tiles: int, n_kv_heads: int) -> int:
+    """Into how many pieces, at most, the key range of each of ``n_tiles`` one-tile items
+    is cut (every piece is one workgroup per key/value head)."""
+    return max(1, COMPUTE_UNITS // max(1, n_tiles * n_kv_heads))
 
 
 @dataclass
 class AttentionPlan:
     """Work lists of the matrix-core kernel for one step (rows are (token, head of the
     group) pairs, token-major):
-    ``items`` [n, 8]: segment, first row, first key, end key, first partial slot or -1,
-    then the segment's first token, number of tokens and number of keys — tiles of 16 rows
-    of segments with at most 16 rows (decode tokens);
+    ``items`` [n, 8]: segment, first row, first key, end key, partial slot or -1, then the
+    segment's first token, number of tokens and number of keys — tiles of 16 rows of segments
+    with at most 16 rows (decode tokens).  They come in runs of four, a workgroup's waves:
+    one piece of a tile's key range cut in four (the last of them may be empty), which the
+    workgroup joins itself, into the output or, where the range has several pieces, into the
+    run's partial slot;
     ``big_items`` [n, 16] for longer segments: the first five the same, then the first rows
     of the item's further tiles (-1: none), ``rows_big`` rows per item; then the segment's
     first token, number of tokens and number of keys, and the first and end key of the walk
@@ -53,8 +69,8 @@ class AttentionPlan:
     cap_big: int = 0
     cap_merges: int = 0
     cap_partials: int = 0
-    # the most partial results that a merge item joins; 0: not known (a static layout,
-    # whose kernel launches are fixed while the plans change)
+    # the most partial results that a merge item joins (under a static layout, whose kernel
+    # launches are fixed while the plans change: the most that any of its plans could have)
     max_parts: int = 0
 
     def __post_init__(self):
@@ -113,15 +129,14 @@ def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick):
     return seg_ids, r0, b, e
 
 
-def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, seg_scalars, more_tiles=None, group=1):
-    """Items and merge entries of tiles whose key ranges are cut into pieces of
-    ``chunk`` keys (pieces end on multiples of 32 keys).  ``more_tiles`` [n, k] holds
-    the first rows of an item's further 16-row tiles (-1: none); without it the items
-    carry their segment's row of ``seg_scalars`` [segments, 3] (first token, tokens,
-    keys) in those places."""
+def _cut_long(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, seg_scalars, more_tiles):
+    """Items and merge entries of the long segments' items, whose key ranges are cut into
+    pieces of ``chunk`` keys (pieces end on multiples of 32 keys).  ``more_tiles`` [n, k]
+    holds the first rows of an item's further 16-row tiles (-1: none); ``seg_scalars``
+    [segments, 3] the segments' first token, tokens and keys."""
     n_tiles = len(seg_ids)
     if n_tiles == 0:
-        return np.zeros((0, BIG_ITEM_INTS if group > 1 else 8), np.int32), np.zeros((0, 8), np.int32), first_slot
+        return np.zeros((0, BIG_ITEM_INTS), np.int32), np.zeros((0, 8), np.int32), first_slot
     base = kv_b - kv_b % KEYS_PER_BLOCK
     n_pieces = np.maximum(1, -(-(kv_e - base) // chunk))
     n_items = int(n_pieces.sum())
@@ -134,19 +149,14 @@ def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, seg_scal
     items[:, 2] = np.maximum(kv_b[tile_of], base[tile_of] + piece * chunk)
     items[:, 3] = np.minimum(kv_e[tile_of], base[tile_of] + (piece + 1) * chunk)
     items[:, 5:] = -1
-    if more_tiles is not None:
-        items[:, 5 : 5 + more_tiles.shape[1]] = more_tiles[tile_of]
-    else:
-        items[:, 5:8] = seg_scalars[items[:, 0]]
+    items[:, 5 : 5 + more_tiles.shape[1]] = more_tiles[tile_of]
     split = n_pieces[tile_of] > 1
     items[:, 4] = -1
     n_split = int(split.sum())
     items[split, 4] = first_slot + np.arange(n_split) * slots_per_tile
     # one merge entry per 16-row tile of every item that was cut
     cut = np.nonzero(n_pieces > 1)[0]
-    firsts = rho0s[cut][:, None]
-    if more_tiles is not None:
-        firsts = np.concatenate((firsts, more_tiles[cut]), axis=1)
+    firsts = np.concatenate((rho0s[cut][:, None], more_tiles[cut]), axis=1)
     sub = np.broadcast_to(np.arange(firsts.shape[1]), firsts.shape)
     keep = firsts >= 0
     rows_of = np.broadcast_to(cut[:, None], firsts.shape)[keep]
@@ -157,12 +167,54 @@ def _cut(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, seg_scal
     merges[:, 3] = n_pieces[rows_of]
     merges[:, 4] = slots_per_tile
     merges[:, 5:7] = seg_scalars[merges[:, 0], :2]
-    if group > 1:
-        items = _group_items(items, piece, group, seg_scalars)
-    else:
-        # the longest key ranges first: the waves that run longest start earliest
-        items = items[np.argsort(-(items[:, 3] - items[:, 2]), kind="stable")]
-    return items, merges, first_slot + n_split * slots_per_tile
+    return _group_items(items, piece, WAVES_PER_GROUP, seg_scalars), merges, first_slot + n_split * slots_per_tile
+
+
+def _cut_joined(seg_ids, rho0s, kv_b, kv_e, most_pieces, first_slot, seg_scalars):
+    """Items and merge entries of one-tile items whose key ranges are cut into at most
+    ``most_pieces`` pieces, one per workgroup, and every piece into four, one per wave (in
+    blocks of 32 keys, as evenly as they go; where a piece is short the last of the four are
+    empty).  A piece's four items stand in a row and carry the piece's partial slot, or -1
+    where the range is one piece; the longest pieces come first."""
+    n = len(seg_ids)
+    if n == 0:
+        return np.zeros((0, 8), np.int32), np.zeros((0, 8), np.int32), first_slot
+    base = kv_b - kv_b % KEYS_PER_BLOCK
+    blocks = -(-(kv_e - base) // KEYS_PER_BLOCK)
+    n_pieces = np.clip((kv_e - base) // MIN_PIECE_KEYS, 1, most_pieces)
+    total = int(n_pieces.sum())
+    tile_of = np.repeat(np.arange(n), n_pieces)
+    first_item = np.concatenate(([0], np.cumsum(n_pieces)[:-1]))
+    piece = np.arange(total) - first_item[tile_of]
+    # wave w of all the range's waves takes the blocks from ceil(w * blocks / waves) on
+    waves = (n_pieces * WAVES_PER_GROUP)[tile_of][:, None]
+    w = piece[:, None] * WAVES_PER_GROUP + np.arange(WAVES_PER_GROUP + 1)[None, :]
+    edge = base[tile_of][:, None] + -(-(w * blocks[tile_of][:, None]) // waves) * KEYS_PER_BLOCK
+    b = np.maximum(kv_b[tile_of][:, None], edge[:, :-1])
+    e = np.minimum(kv_e[tile_of][:, None], edge[:, 1:])
+    empty = b >= e
+    items = np.zeros((total, WAVES_PER_GROUP, 8), dtype=np.int32)
+    items[:, :, 0] = seg_ids[tile_of][:, None]
+    items[:, :, 1] = rho0s[tile_of][:, None]
+    items[:, :, 2] = np.where(empty, 0, b)
+    items[:, :, 3] = np.where(empty, 0, e)
+    items[:, :, 5:8] = seg_scalars[seg_ids[tile_of]][:, None, :]
+    split = n_pieces[tile_of] > 1
+    n_split = int(split.sum())
+    slots = np.full(total, -1, dtype=np.int64)
+    slots[split] = first_slot + np.arange(n_split)
+    items[:, :, 4] = slots[:, None]
+    cut = np.nonzero(n_pieces > 1)[0]
+    merges = np.zeros((len(cut), 8), dtype=np.int32)
+    merges[:, 0] = seg_ids[cut]
+    merges[:, 1] = rho0s[cut]
+    merges[:, 2] = slots[first_item[cut]]
+    merges[:, 3] = n_pieces[cut]
+    merges[:, 4] = 1
+    merges[:, 5:7] = seg_scalars[seg_ids[cut], :2]
+    keys = np.where(empty, 0, e).max(axis=1) - b[:, 0]  # a piece's first wave always has keys
+    order = np.argsort(-keys, kind="stable")
+    return items[order].reshape(total * WAVES_PER_GROUP, 8), merges, first_slot + n_split
 
 
 def _group_items(items: np.ndarray, piece: np.ndarray, group: int, seg_scalars: np.ndarray) -> np.ndarray:
@@ -226,30 +278,30 @@ def _group_tiles(seg_ids, rho0s, kv_b, kv_e, per_item: int):
 def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: int,
                rows_big: int = 64) -> AttentionPlan:
     """Cuts the step's query rows into tiles of 16 rows.  A segment of at most 16 rows
-    (decode tokens) gives one-tile items; a longer one gives items of ``rows_big / 16``
-    tiles that share the keys a wave loads.  Where there are too few items to fill the
-    GPU, an item's key range is cut into pieces whose partial results are merged."""
+    (decode tokens) gives one-tile items, four to a workgroup, which takes a piece of the
+    tile's key range; a longer segment gives items of ``rows_big / 16`` tiles that share the
+    keys a wave loads.  Where there are too few items to fill the GPU, a key range is cut
+    into pieces whose partial results are merged."""
     ql = np.asarray(seg_q_len, dtype=np.int64).reshape(-1)
     seg_scalars = np.stack((np.cumsum(ql) - ql, ql, np.asarray(seg_kv_len, dtype=np.int64).reshape(-1)), axis=1)
     per_item = max(1, rows_big // ROWS_PER_ITEM)
     small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: (r <= ROWS_PER_ITEM) | (per_item == 1))
     big = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: (r > ROWS_PER_ITEM) & (per_item > 1))
+    items, merges_s, slot = _cut_joined(*small, pieces_per_tile(len(small[0]), n_kv_heads), 0, seg_scalars)
     more = None
     if len(big[0]):
         *big, more = _group_tiles(*big, per_item)
-    n_items = len(small[0]) + len(big[0])
-    # a step with a long segment is cut for half as many waves: its workgroups have eight
-    # waves each, and pieces cost a pass over float32 partial results (prompt portions of 256
-    # to 1,024 tokens measured 2 to 4% faster as whole steps)
-    target = TARGET_WAVES if len(big[0]) == 0 else TARGET_WAVES // 2
-    if n_items * n_kv_heads * 2 >= target or n_items == 0:
+    # the long segments' workgroups have eight waves each, and pieces cost a pass over
+    # float32 partial results (prompt portions of 256 to 1,024 tokens measured 2 to 4% faster
+    # as whole steps cut for this many waves than for twice as many)
+    target = TARGET_WAVES_LONG
+    if len(big[0]) * n_kv_heads * 2 >= target or len(big[0]) == 0:
         chunk = 1 << 30  # enough items to fill the GPU: nothing is cut
     else:
-        total = int((small[3] - small[2]).sum() + (big[3] - big[2]).sum()) * n_kv_heads
+        total = int((big[3] - big[2]).sum()) * n_kv_heads
         chunk = -(-total // target)
         chunk = max(MIN_SPLIT_KEYS, -(-chunk // KEYS_PER_BLOCK) * KEYS_PER_BLOCK)
-    items, merges_s, slot = _cut(*small, chunk, 1, 0, seg_scalars)
-    big_items, merges_b, slot = _cut(*big, chunk, per_item, slot, seg_scalars, more, group=WAVES_PER_GROUP)
+    big_items, merges_b, slot = _cut_long(*big, chunk, per_item, slot, seg_scalars, more)
     merges = np.concatenate((merges_s, merges_b)) if len(merges_s) or len(merges_b) else np.zeros((0, 8), np.int32)
     return AttentionPlan(items, big_items, merges, slot, rows_big)
 

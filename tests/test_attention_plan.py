@@ -25,10 +25,24 @@ def check_plan(plan, q_len, kv_len, group, window):
         assert (run[:, 8:11] == [int(sum(q_len[:seg])), int(q_len[seg]), int(kv_len[seg])]).all()
         assert (run[:, 11] == live[:, 2].min()).all() and (run[:, 12] == live[:, 3].max()).all()
         assert (run[:, 13:] == 0).all()
+    # the one-tile items come in runs of four too: a piece of one tile's key range cut in four
+    # (some may be empty, the first never is), which the kernel joins into one result
+    assert plan.n_items % 4 == 0
+    for r in range(0, plan.n_items, 4):
+        run = plan.items[r : r + 4]
+        assert len(set(map(tuple, run[:, [0, 1, 4, 5, 6, 7]].tolist()))) == 1
+        live = run[run[:, 3] > run[:, 2]]
+        assert run[0, 3] > run[0, 2] and (live[1:, 2] == live[:-1, 3]).all() and (live[:-1, 3] % 32 == 0).all()
+        assert (run[run[:, 3] <= run[:, 2], 2:4] == 0).all()
+        blocks = -(-(live[:, 3] - live[:, 2] // 32 * 32) // 32)
+        assert blocks.max() - blocks.min() <= 1 or len(live) < 4
     for arr, is_big in ((plan.items, False), (plan.big_items[:, :8], True)):
         for seg, rho0, b, e, partial, *more in arr.tolist():
             if is_big and rho0 < 0:
                 assert (b, e, partial, more) == (0, 0, -1, [-1, -1, -1])
+                continue
+            if not is_big and b == e:  # an empty quarter of a short piece
+                assert (b, e) == (0, 0)
                 continue
             rows = q_len[seg] * group
             assert (rows > 16 and per_item > 1) == is_big
@@ -55,6 +69,15 @@ def check_plan(plan, q_len, kv_len, group, window):
             lo = t_lo if lo is None else min(lo, t_lo)
             hi = t_hi if hi is None else max(hi, t_hi)
         pieces.sort()
+        if len(tiles) == 1 and (rows <= 16 or per_item == 1):  # the quarters of a piece share its slot
+            whole = []
+            for b, e, p in pieces:
+                if whole and whole[-1][2] == p and (p >= 0 or whole[-1][1] == b):
+                    whole[-1] = (whole[-1][0], e, p)
+                else:
+                    whole.append((b, e, p))
+            pieces = whole
+            assert all(e - b >= 352 for b, e, _ in pieces) or len(pieces) == 1
         assert pieces[0][0] == lo and pieces[-1][1] == hi
         for (b0, e0, _), (b1, e1, _) in zip(pieces, pieces[1:]):
             assert e0 == b1 and e0 % 32 == 0
@@ -88,8 +111,11 @@ def test_every_row_and_key_is_covered_once(group, window, rows_big):
 
 
 def test_long_decode_is_split_and_prefill_is_not():
+    # eight requests, eight key/value heads: four pieces each fill the 256 compute units
     plan = plan_items(np.array([1] * 8), np.array([8192] * 8), 4, 8, 0)
-    assert plan.n_merges == 8 and plan.n_items > 8 * 4 and plan.n_big == 0
+    assert plan.n_merges == 8 and plan.n_items == 8 * 4 * 4 and plan.n_partials == 32 and plan.n_big == 0
+    assert (plan.merges[:, 3] == 4).all() and (plan.merges[:, 4] == 1).all()
+    assert plan.items[:4, 2:5].tolist() == [[0, 512, 0], [512, 1024, 0], [1024, 1536, 0], [1536, 2048, 0]]
     plan = plan_items(np.array([2048]), np.array([2048]), 4, 8, 0)
     assert plan.n_merges == 0 and plan.n_big == 2048 * 4 // 64 and plan.n_items == 0
     # neighbouring tiles ride together
@@ -103,3 +129,30 @@ def test_long_decode_is_split_and_prefill_is_not():
     check_plan(plan, q_len, kv_len, 4, 0)
     empty = plan_items(np.array([], dtype=np.int32), np.array([], dtype=np.int32), 4, 8, 0)
     assert empty.n_items == 0 and empty.n_big == 0
+
+
+def test_the_pieces_of_decode_tokens_key_ranges():
+    from halite_amd.kernels.attention import pieces_per_tile
+
+    # short ranges stay whole: one workgroup, its four waves a quarter each, nothing to merge
+    plan = plan_items(np.array([1] * 8), np.array([570] * 8), 4, 8, 0)
+    assert plan.n_items == 32 and plan.n_merges == 0 and plan.n_partials == 0
+    assert plan.items[:4, 2:5].tolist() == [[0, 160, -1], [160, 288, -1], [288, 448, -1], [448, 570, -1]]
+    # few keys: some quarters are empty
+    plan = plan_items(np.array([1]), np.array([40]), 4, 8, 0)
+    assert plan.items[:, 2:4].tolist() == [[0, 32], [0, 0], [32, 40], [0, 0]]
+    # no piece under 384 keys, whatever room there is
+    assert plan_items(np.array([1]), np.array([767]), 4, 8, 0).n_items == 4
+    plan = plan_items(np.array([1]), np.array([1200]), 4, 8, 0)
+    assert plan.n_items == 12 and plan.merges.tolist() == [[0, 0, 0, 3, 1, 0, 1, 0]]
+    # as many pieces as fill the compute units once, and none where the tiles alone do
+    assert [pieces_per_tile(n, 8) for n in (1, 2, 3, 8, 12, 16, 24, 32, 64)] == [32, 16, 10, 4, 2, 2, 1, 1, 1]
+    assert pieces_per_tile(1, 1) == 256 and pieces_per_tile(0, 8) == 256
+    plan = plan_items(np.array([1] * 64), np.array([30000] * 64), 4, 8, 0)
+    assert plan.n_items == 256 and plan.n_merges == 0
+    plan = plan_items(np.array([1]), np.array([131072]), 4, 8, 0)
+    assert plan.n_items == 128 and plan.merges[0, 3] == 32
+    # a mixed step: the decode tokens' pieces do not depend on the prompt portion beside them
+    mixed = plan_items(np.array([1, 700, 1]), np.array([5000, 700, 5000]), 4, 8, 0)
+    alone = plan_items(np.array([1, 1]), np.array([5000, 5000]), 4, 8, 0)
+    assert (mixed.items[:, 2:5] == alone.items[:, 2:5]).all() and mixed.n_big > 0

@@ -419,6 +419,20 @@ def test_attention_mfma(gpu, H, K, D, segs):
             attention_case(gpu, "bfloat16", H, K, D, page, segs, window, seed=31, use="mfma", tiled=True)
 
 
+@pytest.mark.parametrize("H,K,D", SHAPES)
+def test_attention_mfma_pieces_of_decode_tokens(gpu, H, K, D):
+    """Decode tokens against key ranges of one piece (joined in the workgroup, some of its four
+    quarters empty) and of several (joined there into partial results, then merged), at every
+    head size, with windows that start a range in the middle of a block."""
+    segs = [(2000, 1), (900, 1), (40, 1), (1199, 2), (383, 1)]
+    if 2 * (H // K) <= 16:  # every segment is one tile: three of the ranges are cut
+        q_len, kv_len = np.array([n for _, n in segs]), np.array([b + n for b, n in segs])
+        plan = attn_kernels.plan_items(q_len, kv_len, H // K, K, 0, attn_kernels.rows_per_big_item(D))
+        assert plan.n_big == 0 and sorted(plan.merges[:, 3].tolist()) == [2, 3, 5] and plan.n_items == 4 * 12
+    for page, window, tiled in ((16, 0, False), (64, 0, D % 32 == 0), (8, 37, False), (64, 1000, D % 32 == 0), (24, 601, False)):
+        attention_case(gpu, "bfloat16", H, K, D, page, segs, window, seed=33, use="mfma", tiled=tiled)
+
+
 def test_attention_mfma_split_keys(gpu):
     # few rows and many keys: the key range is cut and merged
     segs = [(3000, 1), (1500, 2), (4000, 1)]

@@ -400,3 +400,34 @@ def test_long_prompts_with_the_heads_of_the_8b_shape(dtype, tmp_path):
         rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
         replay.compare(rows, ref, TOL[dtype])
         del runner
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_decode_graph_serves_key_ranges_of_one_piece_and_of_several(dtype, tmp_path):
+    """A decode step's attention leaves a short key range whole (one workgroup, no partial
+    results) and cuts a longer one into pieces that the merge kernel joins.  One recorded step
+    serves both: a request decodes across the length where the second piece begins, beside one
+    that stays below it."""
+    from halite_amd.kernels import attention as attention_kernels
+
+    cfg = dict(LLAMA_8B_LAYERS, vocab_size=4096)
+    weights = tiny.random_weights(cfg, seed=12, std=0.02)
+    a, b = tiny.random_tokens(cfg, 1060, 80), tiny.random_tokens(cfg, 90, 81)
+    folder = str(tmp_path / "model")
+    tiny.write_model_folder(folder, cfg, weights, torch.float32 if dtype == "float32" else torch.bfloat16)
+    del weights
+    pc, pw = plain_llama.read_model_folder(folder)
+    ref = {"a": plain_llama.forward(pc, pw, a), "b": plain_llama.forward(pc, pw, b)}
+    del pw
+    edge = 2 * attention_kernels.MIN_PIECE_KEYS
+    assert edge + 30 <= len(a)
+    trace = [{"step": 0, "entries": [{"id": "a", "tokens": a[: edge - 30], "want": []}, {"id": "b", "tokens": b[:30], "want": []}], "end": []}]
+    for i in range(60):  # a's context passes the edge at i = 30
+        trace.append({"step": len(trace), "entries": [{"id": "a", "tokens": [a[edge - 30 + i]], "want": [0]},
+                                                       {"id": "b", "tokens": [b[30 + i]], "want": [0]}], "end": []})
+    trace[-1]["end"] = ["a", "b"]
+    server = ServerConfig(kv_cache_num_tokens=1280, page_size=64, max_seqs_per_forward=4, use_cudagraph=True)
+    runner = ModelRunner.from_pretrained(folder, server, ModelConfig(dtype=dtype))
+    rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
+    assert sorted(runner._graphs) == [2] and runner.graph_replays >= 56
+    replay.compare(rows, ref, TOL[dtype])
