@@ -24,7 +24,8 @@
 // tile's key range, its four waves a quarter of the piece each (four items), and their
 // sums are joined through LDS at the end, so that a range of one piece needs neither partial
 // results in memory nor the merge kernel, and a long range, cut into about as many pieces
-// as there are compute units to take them, a quarter as many partial results as waves.
+// as there are compute units to take them, a quarter as many partial results as waves; the
+// workgroup that finishes a tile's last piece merges the partial results in the same launch.
 // Prompt portions run four items per workgroup (up to RT_BIG tiles
 // each): the waves walk the union of their key ranges together, and each block of keys and
 // values goes once from global memory straight into LDS, a step ahead.  Such a workgroup has
@@ -56,7 +57,8 @@ static_assert(HAL_HEAD_DIM % 16 == 0 && HAL_HEAD_DIM >= 16 && HAL_HEAD_DIM <= 25
 #define D HAL_HEAD_DIM
 #define KT ((D + 31) / 32)  // 32-wide steps over the head dimension for Q K^T
 #define DT (D / 16)         // 16-wide tiles of the head dimension for P V
-#define ITEM_INTS 8
+#define ITEM_INTS 8        // merge items
+#define SMALL_ITEM_INTS 12  // items of the kernel for segments of one tile
 #define BIG_ITEM_INTS 16  // items of the kernel for long segments
 #define RESCALE_SLACK 8.0f  // in powers of two
 #define MERGE_FEW_PARTS 8   // up to here a merge item is one wave's work
@@ -98,9 +100,11 @@ __device__ __forceinline__ void load_to_lds(const bf16_t* src, void* lds) {
 
 // item: {segment, first row of tile 0, first key, end key, first partial slot or -1,
 //        first row of tile 1, of tile 2, of tile 3 (or -1)}
-// An item of the one-tile kernel carries its segment's first token, number of tokens and
-// number of keys in the last three places instead, so that the wave need not wait for the
-// item before it can ask for them.
+// An item of the one-tile kernel (12 ints) carries its segment's first token, number of
+// tokens and number of keys in the last three of the eight instead, so that the wave need
+// not wait for the item before it can ask for them; then the first partial slot of its tile
+// and the number of pieces of the tile's key range, if the kernel is to merge them itself
+// (else 0, 0), and two unused.
 // A wave works on up to RT tiles of 16 rows of one segment; the keys and values it
 // loads serve all of them.  The tiles need not be neighbours (the host lists neighbours:
 // they share nearly all of their keys).  A tile skips the steps whose keys lie wholly
@@ -119,9 +123,9 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                       const int* __restrict__ seg_q_len, const int* __restrict__ seg_kv_len,
                       const int* __restrict__ block_table, int bt_stride,
                       const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-                      float* __restrict__ part_o, float* __restrict__ part_ml, int H, int K,
-                      int page_size, int page_shift, float scale_log2e, int window,
-                      int max_items) {
+                      float* __restrict__ part_o, float* __restrict__ part_ml,
+                      int* __restrict__ counters, int H, int K, int page_size, int page_shift,
+                      float scale_log2e, int window, int max_items) {
   static_assert(HALVES == 1 || (SHARED && HALVES == 2), "only the kernel with LDS has two halves");
   // JOIN (the kernel without LDS for keys): the four items of a workgroup are four pieces of
   // one tile's key range (the host lists them so, in whole runs of four, the last may be
@@ -155,8 +159,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   // (the kernel for long segments finds in its items of 16 what the other looks up: the
   // segment's scalars and the key range that the workgroup's four items walk together)
   constexpr bool INLINE_SEG = SHARED || RT == 1;
-  constexpr int STRIDE_INTS = SHARED ? BIG_ITEM_INTS : ITEM_INTS;
-  constexpr int PRE_INTS = SHARED ? 13 : ITEM_INTS;
+  constexpr int STRIDE_INTS = SHARED ? BIG_ITEM_INTS : SMALL_ITEM_INTS;
+  constexpr int PRE_INTS = SHARED ? 13 : 10;
   int pre[PRE_INTS];
   if constexpr (INLINE_SEG) {
     const int* ip = items + (size_t)(item < max_items ? item : max_items - 1) * STRIDE_INTS;
@@ -716,37 +720,117 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     }
   }
 
+  bool merged_here = false;  // the result is the tile's whole one although the item has a partial slot
   if constexpr (JOIN) {
     // lane to lane: the four waves have the same rows in the same lanes.  Joined by the
-    // log-sum-exp rule, in wave order.
+    // log-sum-exp rule, in wave order; the result is the first wave's.
     constexpr int JV = DT * 4 + 2;
     __shared__ float joined[WAVES - 1][JV][HAL_WAVE];
+    __shared__ int arrived_before;
     float lt = l[0];
     lt += __shfl_xor(lt, 16, HAL_WAVE);
     lt += __shfl_xor(lt, 32, HAL_WAVE);
-    if (wave > 0) {
-      joined[wave - 1][0][lane] = m[0];
-      joined[wave - 1][1][lane] = lt;
+    auto join_waves = [&]() {
+      if (wave > 0) {
+        joined[wave - 1][0][lane] = m[0];
+        joined[wave - 1][1][lane] = lt;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) joined[wave - 1][2 + dt * 4 + r][lane] = o[0][dt][r];
+          for (int r = 0; r < 4; ++r) joined[wave - 1][2 + dt * 4 + r][lane] = o[0][dt][r];
+      }
+      __syncthreads();
+      if (wave > 0) return;
+#pragma unroll
+      for (int w = 0; w < WAVES - 1; ++w) {
+        const float m1 = joined[w][0][lane], l1 = joined[w][1][lane];
+        const float m_new = fmaxf(m[0], m1);
+        const float m_sub = m_new == -INFINITY ? 0.f : m_new;
+        const float a0 = fast_exp2(m[0] - m_sub), a1 = fast_exp2(m1 - m_sub);
+        lt = lt * a0 + l1 * a1;
+        m[0] = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            o[0][dt][r] = o[0][dt][r] * a0 + joined[w][2 + dt * 4 + r][lane] * a1;
+      }
+    };
+    join_waves();
+    // A tile whose key range has several pieces (items 8, 9: its first partial slot and their
+    // number): the piece's result goes to its partial slot, and the workgroup that finds all
+    // the others of the tile done merges them, so that no kernel has to follow for it.  Every
+    // tile has a counter, which the last one to come sets back to zero for the next launch.
+    // The partial results are read back in the order of the pieces whichever workgroup reads
+    // them, so the result does not depend on which came last.
+    const int n_pieces = uniform(pre[9]);
+    if (n_pieces > 1) {
+      // What one workgroup writes and another reads in the same launch goes through loads and
+      // stores of device scope (each a dword, a lane's values 64 apart so that an instruction
+      // covers 256 consecutive bytes), which pass the caches that are not coherent between
+      // workgroups; the count is taken after the stores have completed.
+      auto put = [](float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+      auto get = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+      const int first_slot = uniform(pre[8]);
+      int* counter = counters + (size_t)first_slot * K + g;
+      if (wave == 0) {
+        const size_t slot = (size_t)partial * K + g;
+        float* po = part_o + slot * 16 * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) put(po + (dt * 4 + r) * HAL_WAVE + lane, o[0][dt][r]);
+        if (quad == 0) {
+          float* pm = part_ml + (slot * 16 + col) * 2;
+          put(pm, m[0]);
+          put(pm + 1, lt);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the stores are done
+        if (lane == 0)
+          arrived_before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __syncthreads();
+      if (arrived_before != n_pieces - 1) return;
+      if (wave == 0 && lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      m[0] = -INFINITY;
+      lt = 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      // a wave takes every fourth piece, the loads of several in flight at a time
+      constexpr int U = DT <= 8 ? 4 : 2;
+      for (int i0 = wave; i0 < n_pieces; i0 += WAVES * U) {
+        f32x4 po[U][DT];
+        float pm[U], pl[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i = i0 + u * WAVES;
+          const size_t slot = (size_t)(first_slot + (i < n_pieces ? i : i0)) * K + g;
+          pm[u] = get(part_ml + (slot * 16 + col) * 2);
+          pl[u] = get(part_ml + (slot * 16 + col) * 2 + 1);
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) po[u][dt][r] = get(part_o + slot * 16 * D + (dt * 4 + r) * HAL_WAVE + lane);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (i0 + u * WAVES >= n_pieces) break;
+          const float m_new = fmaxf(m[0], pm[u]);
+          const float m_sub = m_new == -INFINITY ? 0.f : m_new;
+          const float a0 = fast_exp2(m[0] - m_sub), a1 = fast_exp2(pm[u] - m_sub);
+          lt = lt * a0 + pl[u] * a1;
+          m[0] = m_new;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[0][dt][r] = o[0][dt][r] * a0 + po[u][dt][r] * a1;
+        }
+      }
+      join_waves();
+      merged_here = true;
     }
-    __syncthreads();
     if (wave > 0) return;
-#pragma unroll
-    for (int w = 0; w < WAVES - 1; ++w) {
-      const float m1 = joined[w][0][lane], l1 = joined[w][1][lane];
-      const float m_new = fmaxf(m[0], m1);
-      const float m_sub = m_new == -INFINITY ? 0.f : m_new;
-      const float a0 = fast_exp2(m[0] - m_sub), a1 = fast_exp2(m1 - m_sub);
-      lt = lt * a0 + l1 * a1;
-      m[0] = m_new;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[0][dt][r] = o[0][dt][r] * a0 + joined[w][2 + dt * 4 + r][lane] * a1;
-    }
     l[0] = lt;
   }
 
@@ -759,7 +843,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
       lt += __shfl_xor(lt, 32, HAL_WAVE);
     }
     if (!row_ok[rt]) continue;
-    if (partial < 0) {
+    if (partial < 0 || merged_here) {
       const float inv = lt > 0.f ? 1.0f / lt : 0.f;
       bf16_t* op = out + (size_t)(q_start + qi[rt]) * out_row_stride + (size_t)head[rt] * D;
 #pragma unroll
@@ -952,20 +1036,24 @@ extern "C" int hal_attention_mfma_head_dim() { return D; }
 
 extern "C" int hal_attention_mfma_rows_per_big_item() { return 16 * RT_BIG; }
 
-// All arrays are device pointers.  `items` [max_items, 8] lists the work on segments of
+// All arrays are device pointers.  `items` [max_items, 12] lists the work on segments of
 // at most 16 query rows (one tile per wave), `big_items` [max_big, 16] the work on longer
 // segments (hal_attention_mfma_rows_per_big_item() rows per wave), `merges`
-// [max_merges, 8] the row tiles whose key range was cut.  counts = {items, big items,
-// merges} holds the live numbers, so a captured launch can serve varying counts.
+// [max_merges, 8] the row tiles whose key range was cut and whose partial results the merge
+// kernel joins.  counts = {items, big items, merges} holds the live numbers, so a captured
+// launch can serve varying counts.  `counters` [n_counters] (or null, if no item asks the
+// kernel to merge its tile's pieces itself) are zero before the call and zero after it;
+// calls that overlap on one GPU must not share them.
 extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_stride,
                                   const int* items, int max_items, const int* big_items,
                                   int max_big, const int* merges, int max_merges,
                                   const int* counts, const int* seg_q_start,
                                   const int* seg_q_len, const int* seg_kv_len,
                                   const int* block_table, int bt_stride, const void* k_pages,
-                                  const void* v_pages, float* part_o, float* part_ml, int H, int K,
-                                  int head_dim, int page_size, int tiled, float scale,
-                                  int window, int merge_parts, hipStream_t stream) {
+                                  const void* v_pages, float* part_o, float* part_ml,
+                                  int* counters, int n_counters, int H, int K, int head_dim,
+                                  int page_size, int tiled, float scale, int window,
+                                  int merge_parts, hipStream_t stream) {
   HAL_REQUIRE(head_dim == D, "hal_attention_mfma: built for head size %d, called with %d", D,
               head_dim);
   HAL_REQUIRE(H > 0 && K > 0 && H % K == 0, "hal_attention_mfma: %d heads, %d kv heads", H, K);
@@ -996,12 +1084,15 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
     hipLaunchKernelGGL(kernel, grid, dim3(waves * HAL_WAVE * HV_), 0, stream, (const bf16_t*)q,   \
                        q_row_stride, (bf16_t*)out, out_row_stride, LIST, COUNT, seg_q_start,      \
                        seg_q_len, seg_kv_len, block_table, bt_stride, (const bf16_t*)k_pages,     \
-                       (const bf16_t*)v_pages, part_o, part_ml, H, K, page_size, page_shift,      \
-                       scale_log2e, window, MAX);                                                 \
+                       (const bf16_t*)v_pages, part_o, part_ml, counters, H, K, page_size,        \
+                       page_shift, scale_log2e, window, MAX);                                     \
     HAL_LAUNCH_CHECK();                                                                           \
   }
   HAL_REQUIRE(max_items % WAVES == 0 && max_big % WAVES == 0,
               "hal_attention_mfma: items come in runs of %d, a workgroup's waves", WAVES);
+  HAL_REQUIRE(!counters || (part_o && part_ml && (long long)(max_items / WAVES) * K <= n_counters),
+              "hal_attention_mfma: %d counters and the partial buffers do not serve %d items of %d "
+              "kv heads", n_counters, max_items, K);
   if (max_items > 0) LAUNCH_ATTENTION(1, false, 32, 1, items, max_items, counts)
   if (max_big > 0) LAUNCH_ATTENTION(RT_BIG, true, KB_BIG, HALVES_BIG, big_items, max_big, counts + 1)
 #undef LAUNCH_ATTENTION

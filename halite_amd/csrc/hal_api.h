@@ -114,14 +114,16 @@ int hal_attention_mfma_rows_per_big_item();
 // kernel for many partials is taken then).  Items of both lists come in runs of four, a
 // workgroup's waves (max_items and max_big are multiples of four): the one-tile items of a
 // run are four pieces of one piece of a tile's key range (the last may be empty), whose sums
-// the kernel joins itself, into the output or the run's partial slot.
+// the kernel joins itself, into the output or the run's partial slot.  counters: zeroed
+// ints (left zeroed), one per (partial slot, kv head), for the one-tile items that ask the
+// kernel to merge their tile's partial results itself; null if none does.
 int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_stride,
                        const int* items, int max_items, const int* big_items, int max_big,
                        const int* merges, int max_merges, const int* counts,
                        const int* seg_q_start, const int* seg_q_len, const int* seg_kv_len,
                        const int* block_table, int bt_stride, const void* k_pages,
-                       const void* v_pages, float* part_o, float* part_ml, int H, int K,
-                       int head_dim, int page_size, int tiled, float scale, int window,
-                       int merge_parts, hipStream_t stream);
+                       const void* v_pages, float* part_o, float* part_ml, int* counters,
+                       int n_counters, int H, int K, int head_dim, int page_size, int tiled,
+                       float scale, int window, int merge_parts, hipStream_t stream);
 
 }  // extern "C"

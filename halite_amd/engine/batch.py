@@ -203,11 +203,14 @@ class StepContext:
                 most = attention_kernels.pieces_per_tile(tiles, n_kv_heads)
                 cap = plan.cap_items = attention_kernels.WAVES_PER_GROUP * tiles * most
                 # the launches are recorded once for all later plans: none of them cuts a key
-                # range into more pieces than this (into none at all where the tiles are many,
-                # and then nothing is merged)
-                plan.cap_merges, plan.cap_partials = (tiles, tiles * most) if most > 1 else (0, 0)
+                # range into more pieces than this (into none at all where the tiles are many),
+                # and by this number the kernel merges the pieces itself or leaves them to the
+                # merge kernel
+                plan.cap_partials = tiles * most if most > 1 else 0
+                plan.cap_merges = tiles if most > attention_kernels.MERGED_IN_KERNEL else 0
+                plan.merged_in_kernel = 1 < most <= attention_kernels.MERGED_IN_KERNEL
                 plan.max_parts = most
-            self._packer.add(plan.name + "_items", plan.items, None if cap is None else cap * 8)
+            self._packer.add(plan.name + "_items", plan.items, None if cap is None else cap * attention_kernels.SMALL_ITEM_INTS)
             self._packer.add(plan.name + "_big", plan.big_items)
             self._packer.add(plan.name + "_merges", plan.merges, None if cap is None else plan.cap_merges * 8)
             self._packer.add(plan.name + "_counts", plan.counts())
@@ -275,7 +278,7 @@ class StepContext:
                 return self._dev[off : off + rows * ints].view(rows, ints)
 
             counts = self._view(plan.name + "_counts")
-            self._plans[key] = (plan, piece("_items", plan.cap_items),
+            self._plans[key] = (plan, piece("_items", plan.cap_items, attention_kernels.SMALL_ITEM_INTS),
                                 piece("_big", plan.cap_big, attention_kernels.BIG_ITEM_INTS),
                                 piece("_merges", plan.cap_merges), counts)
         return self._plans[key]

@@ -23,7 +23,8 @@ KEYS_PER_BLOCK = 32
 MIN_SPLIT_KEYS = 128
 TARGET_WAVES_LONG = 1024
 WAVES_PER_GROUP = 4  # waves of a workgroup
-BIG_ITEM_INTS = 16  # an item of the kernel for long segments: 8 as the others, then what its workgroup would have to look up
+SMALL_ITEM_INTS = 12  # an item of the kernel for one-tile segments: 8, then its tile's first partial slot and pieces
+BIG_ITEM_INTS = 16  # an item of the kernel for long segments: 8, then what its workgroup would have to look up
 # One-tile items: a tile's key range is cut into pieces, one per workgroup, of which there
 # should be about one per compute unit (what a compute unit has in flight bounds what it
 # reads a second, so an even share each counts for more than many waves: measured), and no
@@ -31,6 +32,12 @@ BIG_ITEM_INTS = 16  # an item of the kernel for long segments: 8 as the others, 
 # shorter walk saves).
 COMPUTE_UNITS = 256
 MIN_PIECE_KEYS = 384
+# Up to this many pieces a tile the attention kernel merges the partial results itself (the
+# workgroup that finishes a tile last does, in the same launch: 1 to 3 us less than a merge
+# kernel behind it); more go to the merge kernel, which spreads a tile's partial results over
+# many workgroups (16 and 32 pieces measured 1 to 2 us faster so).
+MERGED_IN_KERNEL = 8
+N_COUNTERS = 1 << 14  # one per (tile that the kernel merges, key/value head); a tile has pieces only while these are few
 
 
 def pieces_per_tile(n_tiles: int, n_kv_heads: int) -> int:
@@ -43,12 +50,13 @@ def pieces_per_tile(n_tiles: int, n_kv_heads: int) -> int:
 class AttentionPlan:
     """Work lists of the matrix-core kernel for one step (rows are (token, head of the
     group) pairs, token-major):
-    ``items`` [n, 8]: segment, first row, first key, end key, partial slot or -1, then the
+    ``items`` [n, 12]: segment, first row, first key, end key, partial slot or -1, then the
     segment's first token, number of tokens and number of keys — tiles of 16 rows of segments
     with at most 16 rows (decode tokens).  They come in runs of four, a workgroup's waves:
-    one piece of a tile's key range cut in four (the last of them may be empty), which the
-    workgroup joins itself, into the output or, where the range has several pieces, into the
-    run's partial slot;
+    one piece of a tile's key range cut in four (some may be empty), which the workgroup
+    joins itself, into the output or, where the range has several pieces, into the run's
+    partial slot.  Places 8 and 9: the tile's first partial slot and number of pieces if the
+    kernel is to merge them itself (then the tile has no merge entry), else 0;
     ``big_items`` [n, 16] for longer segments: the first five the same, then the first rows
     of the item's further tiles (-1: none), ``rows_big`` rows per item; then the segment's
     first token, number of tokens and number of keys, and the first and end key of the walk
@@ -72,8 +80,12 @@ class AttentionPlan:
     # the most partial results that a merge item joins (under a static layout, whose kernel
     # launches are fixed while the plans change: the most that any of its plans could have)
     max_parts: int = 0
+    # some one-tile items ask the kernel to merge their tile's pieces itself (it needs counters)
+    merged_in_kernel: bool = False
 
     def __post_init__(self):
+        if len(self.items) and int(self.items[:, 9].max()) > 1:
+            self.merged_in_kernel = True
         if len(self.merges) and self.max_parts == 0:
             self.max_parts = int(self.merges[:, 3].max())
         self.cap_items = max(self.cap_items, len(self.items))
@@ -173,12 +185,14 @@ def _cut_long(seg_ids, rho0s, kv_b, kv_e, chunk, slots_per_tile, first_slot, seg
 def _cut_joined(seg_ids, rho0s, kv_b, kv_e, most_pieces, first_slot, seg_scalars):
     """Items and merge entries of one-tile items whose key ranges are cut into at most
     ``most_pieces`` pieces, one per workgroup, and every piece into four, one per wave (in
-    blocks of 32 keys, as evenly as they go; where a piece is short the last of the four are
+    blocks of 32 keys, as evenly as they go; where a piece is short some of the four are
     empty).  A piece's four items stand in a row and carry the piece's partial slot, or -1
-    where the range is one piece; the longest pieces come first."""
+    where the range is one piece; the longest pieces come first.  The pieces are merged by
+    the kernel itself (no merge entries) unless ``most_pieces`` allows more of them than it
+    takes."""
     n = len(seg_ids)
     if n == 0:
-        return np.zeros((0, 8), np.int32), np.zeros((0, 8), np.int32), first_slot
+        return np.zeros((0, SMALL_ITEM_INTS), np.int32), np.zeros((0, 8), np.int32), first_slot
     base = kv_b - kv_b % KEYS_PER_BLOCK
     blocks = -(-(kv_e - base) // KEYS_PER_BLOCK)
     n_pieces = np.clip((kv_e - base) // MIN_PIECE_KEYS, 1, most_pieces)
@@ -193,7 +207,7 @@ def _cut_joined(seg_ids, rho0s, kv_b, kv_e, most_pieces, first_slot, seg_scalars
     b = np.maximum(kv_b[tile_of][:, None], edge[:, :-1])
     e = np.minimum(kv_e[tile_of][:, None], edge[:, 1:])
     empty = b >= e
-    items = np.zeros((total, WAVES_PER_GROUP, 8), dtype=np.int32)
+    items = np.zeros((total, WAVES_PER_GROUP, SMALL_ITEM_INTS), dtype=np.int32)
     items[:, :, 0] = seg_ids[tile_of][:, None]
     items[:, :, 1] = rho0s[tile_of][:, None]
     items[:, :, 2] = np.where(empty, 0, b)
@@ -205,6 +219,10 @@ def _cut_joined(seg_ids, rho0s, kv_b, kv_e, most_pieces, first_slot, seg_scalars
     slots[split] = first_slot + np.arange(n_split)
     items[:, :, 4] = slots[:, None]
     cut = np.nonzero(n_pieces > 1)[0]
+    if most_pieces <= MERGED_IN_KERNEL:  # the kernel merges: the items say where and how many
+        items[:, :, 8] = np.where(split, slots[first_item[tile_of]], 0)[:, None]
+        items[:, :, 9] = np.where(split, n_pieces[tile_of], 0)[:, None]
+        cut = cut[:0]
     merges = np.zeros((len(cut), 8), dtype=np.int32)
     merges[:, 0] = seg_ids[cut]
     merges[:, 1] = rho0s[cut]
@@ -214,7 +232,7 @@ def _cut_joined(seg_ids, rho0s, kv_b, kv_e, most_pieces, first_slot, seg_scalars
     merges[:, 5:7] = seg_scalars[seg_ids[cut], :2]
     keys = np.where(empty, 0, e).max(axis=1) - b[:, 0]  # a piece's first wave always has keys
     order = np.argsort(-keys, kind="stable")
-    return items[order].reshape(total * WAVES_PER_GROUP, 8), merges, first_slot + n_split
+    return items[order].reshape(total * WAVES_PER_GROUP, SMALL_ITEM_INTS), merges, first_slot + n_split
 
 
 def _group_items(items: np.ndarray, piece: np.ndarray, group: int, seg_scalars: np.ndarray) -> np.ndarray:
@@ -306,23 +324,39 @@ def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: 
     return AttentionPlan(items, big_items, merges, slot, rows_big)
 
 
+_COUNTERS: dict = {}
+
+
+def _counters(device) -> torch.Tensor:
+    """The device's counters of the attention kernel: zero between its launches (the kernel
+    sets back what it counts), so one array serves every launch of a stream, recorded ones
+    included; launches that overlap on one device must not share it."""
+    device = torch.device(device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    if key not in _COUNTERS:
+        _COUNTERS[key] = torch.zeros(N_COUNTERS, dtype=torch.int32, device=device)
+    return _COUNTERS[key]
+
+
 def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, window):
     plan, items, big_items, merges, counts = plan_dev
     n_pages, n_kv, page_size, head_dim = kv.k.shape
     lib = library.attention_library(head_dim)
     n = ctx.n_tokens
     out = torch.empty((n, n_heads * head_dim), dtype=torch.bfloat16, device=q.device)
-    part_o = part_ml = None
-    if plan.cap_partials and plan.cap_merges:
+    part_o = part_ml = counters = None
+    if plan.cap_partials:
         part_o = torch.empty((plan.cap_partials, n_kv, 16, head_dim), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((plan.cap_partials, n_kv, 16, 2), dtype=torch.float32, device=q.device)
+    if plan.merged_in_kernel:
+        counters = _counters(q.device)
     P = ops._ptr
     rc = lib.hal_attention_mfma(
         P(q), q_row_stride, P(out), n_heads * head_dim,
         P(items), plan.cap_items, P(big_items), plan.cap_big, P(merges), plan.cap_merges, P(counts),
         P(ctx.seg_q_start), P(ctx.seg_q_len), P(ctx.seg_kv_len),
         P(group.block_table), group.block_table.shape[1], P(kv.k), P(kv.v), P(part_o), P(part_ml),
-        n_heads, n_kv, head_dim, page_size, 1 if getattr(kv, "tiled", False) else 0,
+        P(counters), N_COUNTERS, n_heads, n_kv, head_dim, page_size, 1 if getattr(kv, "tiled", False) else 0,
         ctypes.c_float(scale), window, plan.max_parts, ops._stream(),
     )
     ops._check(lib, rc)

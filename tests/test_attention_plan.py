@@ -30,13 +30,18 @@ def check_plan(plan, q_len, kv_len, group, window):
     assert plan.n_items % 4 == 0
     for r in range(0, plan.n_items, 4):
         run = plan.items[r : r + 4]
-        assert len(set(map(tuple, run[:, [0, 1, 4, 5, 6, 7]].tolist()))) == 1
+        assert len(set(map(tuple, run[:, [0, 1, 4, 5, 6, 7, 8, 9]].tolist()))) == 1 and (run[:, 10:] == 0).all()
         live = run[run[:, 3] > run[:, 2]]
         assert run[0, 3] > run[0, 2] and (live[1:, 2] == live[:-1, 3]).all() and (live[:-1, 3] % 32 == 0).all()
         assert (run[run[:, 3] <= run[:, 2], 2:4] == 0).all()
         blocks = -(-(live[:, 3] - live[:, 2] // 32 * 32) // 32)
         assert blocks.max() - blocks.min() <= 1 or len(live) < 4
-    for arr, is_big in ((plan.items, False), (plan.big_items[:, :8], True)):
+    in_kernel = {}  # (segment, tile) -> (first partial slot, pieces) that the items themselves name
+    for seg, rho0, first, n in plan.items[:, [0, 1, 8, 9]].tolist():
+        assert n != 1 and (n > 1 or first == 0)
+        if n > 1:
+            assert in_kernel.setdefault((seg, (rho0,)), (first, n)) == (first, n)
+    for arr, is_big in ((plan.items[:, :8], False), (plan.big_items[:, :8], True)):
         for seg, rho0, b, e, partial, *more in arr.tolist():
             if is_big and rho0 < 0:
                 assert (b, e, partial, more) == (0, 0, -1, [-1, -1, -1])
@@ -87,6 +92,12 @@ def check_plan(plan, q_len, kv_len, group, window):
         stride = per_item if len(tiles) > 1 or rows > 16 and per_item > 1 else 1
         slots = [p for _, _, p in pieces]
         assert slots == list(range(slots[0], slots[0] + stride * len(slots), stride))
+        if (seg, tiles) in in_kernel:  # merged by the attention kernel: no merge entry
+            assert in_kernel.pop((seg, tiles)) == (slots[0], len(slots)) and len(slots) <= 8
+            assert not [m for m in plan.merges.tolist() if m[0] == seg and m[1] == tiles[0]]
+            assert not used_slots & set(slots)
+            used_slots.update(slots)
+            continue
         for sub, t in enumerate(tiles):
             match = [m for m in plan.merges.tolist() if m[0] == seg and m[1] == t]
             assert match == [[seg, t, slots[0] + sub, len(slots), stride,
@@ -96,7 +107,8 @@ def check_plan(plan, q_len, kv_len, group, window):
             for sub in range(stride):
                 assert s0 + sub not in used_slots
                 used_slots.add(s0 + sub)
-    assert n_merges == plan.n_merges
+    assert n_merges == plan.n_merges and not in_kernel
+    assert plan.merged_in_kernel == bool((plan.items[:, 9] > 1).any())
     assert not used_slots or max(used_slots) < plan.n_partials
 
 
@@ -113,9 +125,10 @@ def test_every_row_and_key_is_covered_once(group, window, rows_big):
 def test_long_decode_is_split_and_prefill_is_not():
     # eight requests, eight key/value heads: four pieces each fill the 256 compute units
     plan = plan_items(np.array([1] * 8), np.array([8192] * 8), 4, 8, 0)
-    assert plan.n_merges == 8 and plan.n_items == 8 * 4 * 4 and plan.n_partials == 32 and plan.n_big == 0
-    assert (plan.merges[:, 3] == 4).all() and (plan.merges[:, 4] == 1).all()
-    assert plan.items[:4, 2:5].tolist() == [[0, 512, 0], [512, 1024, 0], [1024, 1536, 0], [1536, 2048, 0]]
+    assert plan.n_merges == 0 and plan.n_items == 8 * 4 * 4 and plan.n_partials == 32 and plan.n_big == 0
+    assert plan.merged_in_kernel and (plan.items[:, 9] == 4).all()  # the kernel merges a tile's four itself
+    assert plan.items[:4, [2, 3, 4, 8]].tolist() == [[0, 512, 0, 0], [512, 1024, 0, 0], [1024, 1536, 0, 0], [1536, 2048, 0, 0]]
+    assert sorted(set(plan.items[:, 8].tolist())) == [0, 4, 8, 12, 16, 20, 24, 28]
     plan = plan_items(np.array([2048]), np.array([2048]), 4, 8, 0)
     assert plan.n_merges == 0 and plan.n_big == 2048 * 4 // 64 and plan.n_items == 0
     # neighbouring tiles ride together
@@ -144,14 +157,30 @@ def test_the_pieces_of_decode_tokens_key_ranges():
     # no piece under 384 keys, whatever room there is
     assert plan_items(np.array([1]), np.array([767]), 4, 8, 0).n_items == 4
     plan = plan_items(np.array([1]), np.array([1200]), 4, 8, 0)
-    assert plan.n_items == 12 and plan.merges.tolist() == [[0, 0, 0, 3, 1, 0, 1, 0]]
+    assert plan.n_items == 12 and plan.items[:, 4].tolist() == [0] * 4 + [1] * 4 + [2] * 4
+    assert plan.merges.tolist() == [[0, 0, 0, 3, 1, 0, 1, 0]] and (plan.items[:, 8:10] == 0).all()  # (one tile could have 32 pieces)
+    plan = plan_items(np.array([1] * 4), np.array([1200, 50, 50, 50]), 4, 8, 0)
+    assert plan.n_items == 12 + 3 * 4 and plan.n_merges == 0 and (plan.items[:12, 8:10] == [0, 3]).all()
     # as many pieces as fill the compute units once, and none where the tiles alone do
     assert [pieces_per_tile(n, 8) for n in (1, 2, 3, 8, 12, 16, 24, 32, 64)] == [32, 16, 10, 4, 2, 2, 1, 1, 1]
     assert pieces_per_tile(1, 1) == 256 and pieces_per_tile(0, 8) == 256
     plan = plan_items(np.array([1] * 64), np.array([30000] * 64), 4, 8, 0)
     assert plan.n_items == 256 and plan.n_merges == 0
-    plan = plan_items(np.array([1]), np.array([131072]), 4, 8, 0)
-    assert plan.n_items == 128 and plan.merges[0, 3] == 32
+    plan = plan_items(np.array([1] * 4), np.array([131072] * 4), 4, 8, 0)
+    assert plan.n_items == 128 and (plan.items[:, 9] == 8).all() and plan.n_merges == 0
+    # more pieces than the attention kernel merges itself: they are the merge kernel's
+    plan = plan_items(np.array([1]), np.array([131072]), 4, 2, 0)
+    assert plan.n_items == 4 * 128 and not plan.merged_in_kernel and (plan.items[:, 8:] == 0).all()
+    assert plan.merges.tolist() == [[0, 0, 0, 128, 1, 0, 1, 0]]
+    for kv_heads in (1, 2, 8):
+        q_len, kv_len = np.array([1, 2, 1]), np.array([40000, 9000, 300])
+        check_plan(plan_items(q_len, kv_len, 4, kv_heads, 0), q_len, kv_len, 4, 0)
+        check_plan(plan_items(q_len, kv_len, 4, kv_heads, 5000), q_len, kv_len, 4, 5000)
+        q_len, kv_len = np.array([1, 2, 1, 1, 1]), np.array([40000, 9000, 300, 2000, 767])
+        plan = plan_items(q_len, kv_len, 4, kv_heads, 0)
+        assert plan.merged_in_kernel == (kv_heads == 8) and (plan.n_merges == 0) == (kv_heads == 8)
+        check_plan(plan, q_len, kv_len, 4, 0)
+        check_plan(plan_items(q_len, kv_len, 4, kv_heads, 5000), q_len, kv_len, 4, 5000)
     # a mixed step: the decode tokens' pieces do not depend on the prompt portion beside them
     mixed = plan_items(np.array([1, 700, 1]), np.array([5000, 700, 5000]), 4, 8, 0)
     alone = plan_items(np.array([1, 1]), np.array([5000, 5000]), 4, 8, 0)

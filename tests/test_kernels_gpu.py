@@ -422,22 +422,79 @@ def test_attention_mfma(gpu, H, K, D, segs):
 @pytest.mark.parametrize("H,K,D", SHAPES)
 def test_attention_mfma_pieces_of_decode_tokens(gpu, H, K, D):
     """Decode tokens against key ranges of one piece (joined in the workgroup, some of its four
-    quarters empty) and of several (joined there into partial results, then merged), at every
+    quarters empty) and of several (joined there into partial results, which the workgroup that
+    comes last merges), at every
     head size, with windows that start a range in the middle of a block."""
     segs = [(2000, 1), (900, 1), (40, 1), (1199, 2), (383, 1)]
     if 2 * (H // K) <= 16:  # every segment is one tile: three of the ranges are cut
         q_len, kv_len = np.array([n for _, n in segs]), np.array([b + n for b, n in segs])
         plan = attn_kernels.plan_items(q_len, kv_len, H // K, K, 0, attn_kernels.rows_per_big_item(D))
-        assert plan.n_big == 0 and sorted(plan.merges[:, 3].tolist()) == [2, 3, 5] and plan.n_items == 4 * 12
+        assert plan.n_big == 0 and plan.n_items == 4 * 12
+        if K * 5 * 8 >= 256:  # few enough pieces a tile that the attention kernel merges them itself
+            assert sorted(set(plan.items[:, 9].tolist())) == [0, 2, 3, 5] and plan.n_merges == 0
+        else:
+            assert sorted(plan.merges[:, 3].tolist()) == [2, 3, 5] and not plan.merged_in_kernel
     for page, window, tiled in ((16, 0, False), (64, 0, D % 32 == 0), (8, 37, False), (64, 1000, D % 32 == 0), (24, 601, False)):
         attention_case(gpu, "bfloat16", H, K, D, page, segs, window, seed=33, use="mfma", tiled=tiled)
 
 
+def test_attention_mfma_merges_in_the_kernel_the_same_every_time(gpu):
+    """Eight decode tokens against a few thousand keys each: every tile's key range has four
+    pieces, and the workgroup that finishes a tile last merges them.  Which one that is
+    varies from launch to launch; the result must not."""
+    H, K, D, page = 32, 8, 128, 64
+    lens = [3000, 4100, 2047, 3500, 1600, 4096, 2500, 3999]
+    rng = torch.Generator().manual_seed(70)
+    n_pages = sum(-(-n // page) for n in lens)
+    k_pages = (torch.randn((n_pages, K, page, D), generator=rng) * 0.5).to(torch.bfloat16).to(gpu)
+    v_pages = torch.randn((n_pages, K, D, page), generator=rng).to(torch.bfloat16).to(gpu)  # (values are kept transposed)
+    order = torch.randperm(n_pages, generator=rng).to(torch.int32)
+    width = max(-(-n // page) for n in lens)
+    bt = torch.full((len(lens), width), -1, dtype=torch.int32)
+    at = 0
+    for i, n in enumerate(lens):
+        bt[i, : -(-n // page)] = order[at : at + -(-n // page)]
+        at += -(-n // page)
+    q = torch.randn((len(lens), H * D), generator=rng).to(torch.bfloat16).to(gpu)
+    q_len, kv_len = np.ones(len(lens), dtype=np.int32), np.array(lens, dtype=np.int32)
+    plan = attn_kernels.plan_items(q_len, kv_len, H // K, K, 0, attn_kernels.rows_per_big_item(D))
+    assert plan.merged_in_kernel and plan.n_merges == 0 and (plan.items[:, 9] == 4).all()
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+
+    class Ctx:
+        n_tokens = len(lens)
+        seg_q_start = dev(np.arange(len(lens), dtype=np.int32))
+        seg_q_len = dev(q_len)
+        seg_kv_len = dev(kv_len)
+
+    class Group:
+        block_table = bt.to(gpu)
+
+    class KV:
+        k, v, tiled = k_pages, v_pages, False
+
+    plan_dev = attn_kernels.upload_plan(plan, gpu)
+    first = attn_kernels.attention_mfma(q, H * D, plan_dev, Ctx, Group, KV, H, D**-0.5, 0)
+    # against plain attention over the gathered keys
+    for i, n in enumerate(lens):
+        pages = bt[i, : -(-n // page)].long()
+        k = k_pages[pages].permute(0, 2, 1, 3).reshape(-1, K, D)[:n].float().cpu()
+        v = v_pages[pages].permute(0, 3, 1, 2).reshape(-1, K, D)[:n].float().cpu()
+        qi = q[i].float().cpu().view(H, D)
+        want = torch.stack([torch.softmax(k[:, h // (H // K)] @ qi[h] * D**-0.5, 0) @ v[:, h // (H // K)] for h in range(H)])
+        close(first[i].view(H, D), want, 1.2e-2, f"request {i}")
+    for _ in range(300):
+        again = attn_kernels.attention_mfma(q, H * D, plan_dev, Ctx, Group, KV, H, D**-0.5, 0)
+        assert torch.equal(again, first)
+    assert int(attn_kernels._counters(gpu).abs().sum()) == 0  # every count was set back
+
+
 def test_attention_mfma_split_keys(gpu):
-    # few rows and many keys: the key range is cut and merged
+    # few rows and many keys: the key range is cut and merged (so few tiles that a tile may have
+    # more pieces than the attention kernel merges itself: the merge kernel's work)
     segs = [(3000, 1), (1500, 2), (4000, 1)]
     plan = attn_kernels.plan_items(np.array([1, 2, 1]), np.array([3001, 1502, 4001]), 4, 2, 0)
-    assert plan.n_merges == 3 and plan.n_big == 0
+    assert plan.n_merges == 3 and plan.n_big == 0 and not plan.merged_in_kernel
     attention_case(gpu, "bfloat16", 8, 2, 128, 64, segs, 0, seed=40, use="mfma")
     attention_case(gpu, "bfloat16", 8, 2, 128, 16, segs, 1000, seed=41, use="mfma")
     # a short portion against a long context: tiles of 64 rows, cut and merged
