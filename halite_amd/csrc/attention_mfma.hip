@@ -766,20 +766,25 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     const int n_pieces = uniform(pre[9]);
     if (n_pieces > 1) {
       // What one workgroup writes and another reads in the same launch goes through loads and
-      // stores of device scope (each a dword, a lane's values 64 apart so that an instruction
-      // covers 256 consecutive bytes), which pass the caches that are not coherent between
-      // workgroups; the count is taken after the stores have completed.
+      // stores of device scope (sc1), which pass the caches that are not coherent between
+      // workgroups; the count is taken after the stores have completed.  A slot's sums lie in
+      // the order [16 dims][lane][4], so that an instruction covers a contiguous KiB.
       auto put = [](float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
       auto get = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+      constexpr int SC1 = 16;                // cache policy of a buffer access: device scope
+      constexpr int RAW_BUFFER = 0x00020000;  // descriptor word 3: 32-bit elements, no swizzle
+      auto slot_sums = [&](size_t slot) {
+        return __builtin_amdgcn_make_buffer_rsrc(part_o + slot * 16 * D, 0, 16 * D * 4, RAW_BUFFER);
+      };
       const int first_slot = uniform(pre[8]);
       int* counter = counters + (size_t)first_slot * K + g;
       if (wave == 0) {
         const size_t slot = (size_t)partial * K + g;
-        float* po = part_o + slot * 16 * D;
+        const auto to = slot_sums(slot);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) put(po + (dt * 4 + r) * HAL_WAVE + lane, o[0][dt][r]);
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o[0][dt]), to,
+                                                 (dt * HAL_WAVE + lane) * 16, 0, SC1);
         if (quad == 0) {
           float* pm = part_ml + (slot * 16 + col) * 2;
           put(pm, m[0]);
@@ -808,10 +813,11 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
           const size_t slot = (size_t)(first_slot + (i < n_pieces ? i : i0)) * K + g;
           pm[u] = get(part_ml + (slot * 16 + col) * 2);
           pl[u] = get(part_ml + (slot * 16 + col) * 2 + 1);
+          const auto from = slot_sums(slot);
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) po[u][dt][r] = get(part_o + slot * 16 * D + (dt * 4 + r) * HAL_WAVE + lane);
+            po[u][dt] = __builtin_bit_cast(
+                f32x4, __builtin_amdgcn_raw_buffer_load_b128(from, (dt * HAL_WAVE + lane) * 16, 0, SC1));
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
