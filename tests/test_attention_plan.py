@@ -185,3 +185,26 @@ def test_the_pieces_of_decode_tokens_key_ranges():
     mixed = plan_items(np.array([1, 700, 1]), np.array([5000, 700, 5000]), 4, 8, 0)
     alone = plan_items(np.array([1, 1]), np.array([5000, 5000]), 4, 8, 0)
     assert (mixed.items[:, 2:5] == alone.items[:, 2:5]).all() and mixed.n_big > 0
+
+
+def test_random_steps_are_covered():
+    """Random mixes of decode tokens and prompt portions, contexts from nothing to 200,000
+    keys, any head grouping and window: every plan passes the same checks."""
+    rng = np.random.default_rng(7)
+    for case in range(300):
+        n_seg = int(rng.integers(1, 40))
+        kinds = rng.integers(0, 4, n_seg)
+        q_len = np.where(kinds == 0, rng.integers(1, 4, n_seg), np.where(kinds == 1, 1, rng.integers(1, 600, n_seg)))
+        q_len = np.where(kinds == 3, 1, q_len).astype(np.int32)
+        before = np.where(rng.random(n_seg) < 0.3, 0, rng.integers(0, int(rng.choice([50, 900, 5000, 200000])), n_seg))
+        kv_len = (q_len + before).astype(np.int32)
+        group = int(rng.choice([1, 2, 3, 4, 8, 20]))
+        kv_heads = int(rng.choice([1, 2, 8]))
+        window = int(rng.choice([0, 0, 1, 37, 1000, 5000]))
+        rows_big = int(rng.choice([16, 32, 64]))
+        plan = plan_items(q_len, kv_len, group, kv_heads, window, rows_big)
+        try:
+            check_plan(plan, q_len, kv_len, group, window)
+        except AssertionError as e:
+            raise AssertionError(f"case {case}: q {q_len.tolist()} kv {kv_len.tolist()} group {group} kv heads {kv_heads} "
+                                 f"window {window} rows {rows_big}") from e
