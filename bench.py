@@ -222,7 +222,7 @@ def engine_workload(args) -> int:
     server = ServerConfig(
         kv_cache_num_tokens=pool, max_seqs_per_forward=len(lengths), max_tokens_per_forward=8192,
         chunked_prefill_size=chunk, max_prefill_tokens=8192, use_cudagraph=not args.no_graph,
-        cudagraph_max_batch_size=len(lengths), scheduling_steps_ahead=args.steps_ahead,
+        cudagraph_max_batch_size=len(lengths), cudagraph_step=1, scheduling_steps_ahead=args.steps_ahead,
     )
     t0 = time.perf_counter()
     runner = ModelRunner.from_random(cfg, seed=0, server_config=server, model_config=ModelConfig(dtype=args.dtype, context_len=8192))

@@ -29,6 +29,17 @@ class ServerConfig(BaseModel):
     use_cudagraph: StrictBool = False
     """Replay decode-only steps from a captured HIP graph."""
     cudagraph_max_batch_size: StrictInt = 64
+    """Largest decode batch that is replayed from a graph.  A graph here serves the batch
+    size it was recorded for and nothing is padded (the reference pads a batch up to the
+    next size it has a graph for, model_runner.py:160-166), so every size up to this one
+    gets a graph of its own, at its first use or ahead of time."""
+    cudagraph_step: StrictInt = Field(default=16, gt=0)
+    cudagraph_additonal_batch_size: tuple[StrictInt, ...] = ()
+    """The sizes whose graphs are recorded ahead of time
+    (``InferenceEngine.initialize(capture_graphs=True)``): the additional ones and every
+    multiple of the step up to the largest, as the reference lists its graph sizes
+    (model_runner.py:86-95; the option's name is spelled as there).  Other sizes are
+    recorded when a step first has them."""
 
     # -- tokainfer/types.py:65-190 -------------------------------------------
     page_size: StrictInt = Field(default=64, gt=0)

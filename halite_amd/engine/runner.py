@@ -217,15 +217,20 @@ class ModelRunner:
     def capture_graphs(self, batch_sizes=None) -> list[int]:
         """Records the decode graphs of the given batch sizes now instead of at their
         first use (the reference records its graphs when the engine is set up,
-        src/halite/transformers/infer/engine/model_runner.py:159-239).  Needs an idle
-        cache: every size is run once with one-token requests that are freed again.
-        Returns the sizes that have a graph afterwards."""
+        src/halite/transformers/infer/engine/model_runner.py:159-239); without sizes,
+        those that the server configuration lists (``cudagraph_additonal_batch_size`` and
+        the multiples of ``cudagraph_step``).  Needs an idle cache: every size is run
+        once with one-token requests that are freed again.  Returns the sizes that have
+        a graph afterwards."""
         if not self.graphs_allowed:
             return []
         if not self.cache.idle():
             raise RuntimeError("graphs are recorded ahead of time only while no request is live")
         most = min(self.server_config.cudagraph_max_batch_size, self.server_config.max_seqs_per_forward)
-        for b in sorted(set(batch_sizes) if batch_sizes is not None else range(1, most + 1)):
+        if batch_sizes is None:
+            cfg = self.server_config
+            batch_sizes = set(cfg.cudagraph_additonal_batch_size) | set(range(cfg.cudagraph_step, most + 1, cfg.cudagraph_step))
+        for b in sorted(set(batch_sizes)):
             entry = self._graphs.get(b)
             if b < 1 or b > most or (entry is not None and entry["graph"] is not None):
                 continue

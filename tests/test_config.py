@@ -170,6 +170,12 @@ def test_engine_options_and_overrides():
     assert s.page_size == 16 and s.max_tokens_per_forward == 512 and s.use_cudagraph is True
     assert s.max_prefill_tokens == 16384 and s.chunked_prefill_size == 8192  # the reference's defaults
     assert s.default_init_new_token_ratio == 0.7
+    # the reference's way to list graph sizes (infer/types.py:77-80), its spelling included
+    assert s.cudagraph_step == 16 and s.cudagraph_additonal_batch_size == ()
+    s = ServerConfig(**parse_overrides(["cudagraph_step=8", "cudagraph_additonal_batch_size=[1, 2, 4]"]))
+    assert s.cudagraph_step == 8 and s.cudagraph_additonal_batch_size == (1, 2, 4)
+    with pytest.raises(ValueError):
+        ServerConfig(cudagraph_step=0)
     with pytest.raises(ValueError):
         ServerConfig(page_size=0)
     with pytest.raises(ValueError):

@@ -332,11 +332,11 @@ def test_the_engine_serves_on_after_a_refused_or_failed_batch(models):
 
 
 def test_graphs_recorded_ahead_of_time(models):
-    """``initialize(capture_graphs=True)`` records the decode graph of every batch size while
-    the engine is idle; generation then replays them and gives the tokens of an engine
-    that records at first use."""
+    """``initialize(capture_graphs=True)`` records the decode graphs of the batch sizes that
+    the configuration lists while the engine is idle; generation then replays them and gives
+    the tokens of an engine that records at first use."""
     folder, pc, pw = models[("B", "bfloat16")]
-    server = ServerConfig(kv_cache_num_tokens=2048, max_seqs_per_forward=6, use_cudagraph=True)
+    server = ServerConfig(kv_cache_num_tokens=2048, max_seqs_per_forward=6, use_cudagraph=True, cudagraph_step=1)
     prompts = [tiny.random_tokens(tiny.TINY_B, n, 500 + n) for n in (3, 40, 17, 9)]
     batch = [(p, {"max_new_tokens": 10 + 2 * i, "temperature": 0.0}) for i, p in enumerate(prompts)]
     lazy = InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="bfloat16"))
@@ -349,6 +349,15 @@ def test_graphs_recorded_ahead_of_time(models):
     assert [r.output_ids for r in eager.infer_batch(batch)] == want
     assert runner.graph_replays > replays and sorted(runner._graphs) == [1, 2, 3, 4, 5, 6]
     assert runner.capture_graphs([2, 3]) == [1, 2, 3, 4, 5, 6]  # nothing to do
+    # the reference's way to list the sizes: multiples of a step, and additional ones; the
+    # other sizes get their graphs when a step first has them
+    some = InferenceEngine.from_pretrained(
+        folder, server.model_copy(update={"cudagraph_step": 4, "cudagraph_additonal_batch_size": (1, 6, 9)}),
+        ModelConfig(dtype="bfloat16"))
+    some.initialize(capture_graphs=True)
+    assert sorted(some.model_runner._graphs) == [1, 4, 6]  # (no more than six requests are live at a time)
+    assert [r.output_ids for r in some.infer_batch(batch)] == want
+    assert set(some.model_runner._graphs) >= {1, 2, 3, 4, 6}
     # without graphs there is nothing to record
     plain = InferenceEngine.from_pretrained(folder, ServerConfig(kv_cache_num_tokens=512), ModelConfig(dtype="bfloat16"))
     plain.initialize(capture_graphs=True)
