@@ -75,11 +75,35 @@ class ModelConfig(BaseModel):
 
     context_len: StrictInt | None = Field(default=None, gt=0)
     """Longest request; ``None`` takes the model's ``max_position_embeddings``."""
+    n_heads: StrictInt | None = Field(default=None, gt=0)
+    n_key_value_heads: StrictInt | None = Field(default=None, gt=0)
+    head_dim: StrictInt | None = Field(default=None, gt=0)
+    n_layers: StrictInt | None = Field(default=None, gt=0)
+    """The reference's engine is told these (infer/types.py:85-89, scripts/eval_task.py:148-154);
+    here the model says them, and what a caller states is only checked against it."""
+    tp_size: Literal[1] = 1
+    distributed: Literal[False] = False
     dtype: Literal["bfloat16", "float32"] = "bfloat16"
     kv_cache_dtype: Literal["auto"] = "auto"
     memory_fraction_static: float = Field(default=0.88, gt=0, le=1)
     gpu_id: StrictInt = 0
     device: str = "cuda"
+
+
+def check_stated_sizes(options: ModelConfig, n_layers: int, attention_sizes: list[tuple[int, int, int]]) -> None:
+    """Raises if sizes that a caller states in ``options`` (as the reference's callers do)
+    disagree with the model: ``n_layers`` runs, and ``(heads, key/value heads, head size)``
+    of every layer that has them."""
+    wrong = []
+    if options.n_layers is not None and options.n_layers != n_layers:
+        wrong.append(f"n_layers={options.n_layers} (the model runs {n_layers})")
+    for name, at in (("n_heads", 0), ("n_key_value_heads", 1), ("head_dim", 2)):
+        stated = getattr(options, name)
+        have = sorted({sizes[at] for sizes in attention_sizes})
+        if stated is not None and have != [stated]:
+            wrong.append(f"{name}={stated} (the model's layers have {', '.join(map(str, have)) or 'none'})")
+    if wrong:
+        raise ValueError("model options disagree with the model: " + "; ".join(wrong))
 
 
 def parse_overrides(pairs: list[str]) -> dict:

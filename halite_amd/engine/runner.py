@@ -17,7 +17,7 @@ import numpy as np
 import torch
 
 from ..cache import CacheManager, NoSpace
-from ..config.engine import ModelConfig, ServerConfig
+from ..config.engine import ModelConfig, ServerConfig, check_stated_sizes
 from ..config.registry import read_config
 from ..parts.decoder import Decoder
 from ..weights import fill_random, load_weights
@@ -71,6 +71,9 @@ class ModelRunner:
             st = mixer.state_need()
             if st:
                 state_needs[i] = st
+        check_stated_sizes(self.model_config, len(spec.order), [
+            (getattr(model.mixer_of_run(i).p, "n_heads", need.n_kv_heads), need.n_kv_heads, need.head_dim)
+            for i, need in needs.items()])
         page_size = self.server_config.page_size
         n_slots = self.server_config.max_seqs_per_forward
         num_pages = self._size_pool(needs, page_size, model.dtype)

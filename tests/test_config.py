@@ -184,6 +184,19 @@ def test_engine_options_and_overrides():
         ModelConfig(dtype="float16")
     with pytest.raises(ValueError, match="key=value"):
         parse_overrides(["page_size"])
+    # what the reference's callers tell its engine about the model (scripts/eval_task.py:148-154)
+    # is taken and checked against the model; several GPUs are not
+    from halite_amd.config.engine import check_stated_sizes
+
+    stated = ModelConfig(n_heads=6, n_key_value_heads=2, head_dim=48, n_layers=3, context_len=256)
+    check_stated_sizes(stated, 3, [(6, 2, 48)] * 3)
+    check_stated_sizes(ModelConfig(), 5, [(4, 4, 16), (8, 2, 32)])  # nothing stated, nothing to check
+    with pytest.raises(ValueError, match=r"n_layers=3 \(the model runs 4\).*head_dim=48 \(the model's layers have 32, 48\)"):
+        check_stated_sizes(stated, 4, [(6, 2, 48), (6, 2, 32)])
+    with pytest.raises(ValueError):
+        ModelConfig(tp_size=2)
+    with pytest.raises(ValueError):
+        ModelConfig(distributed=True)
 
 
 def test_command_line_takes_overrides_and_options_in_any_order():

@@ -364,6 +364,21 @@ def test_graphs_recorded_ahead_of_time(models):
     assert plain.model_runner._graphs == {}
 
 
+def test_stated_model_sizes_are_checked(models):
+    """The reference's callers tell its engine the model's sizes (scripts/eval_task.py:148-154);
+    here they are read from the model, and what a caller states must agree."""
+    folder, pc, pw = models[("B", "bfloat16")]
+    cfg = tiny.TINY_B
+    server = ServerConfig(kv_cache_num_tokens=256)
+    stated = dict(n_heads=cfg["num_attention_heads"], n_key_value_heads=cfg["num_key_value_heads"],
+                  head_dim=cfg.get("head_dim", cfg["hidden_size"] // cfg["num_attention_heads"]),
+                  n_layers=cfg["num_hidden_layers"], context_len=128)
+    engine = InferenceEngine.from_pretrained(folder, server, ModelConfig(**stated))
+    assert len(engine.infer_batch([([3, 4, 5], {"max_new_tokens": 2, "temperature": 0.0})])[0].output_ids[0]) == 2
+    with pytest.raises(ValueError, match="n_key_value_heads"):
+        InferenceEngine.from_pretrained(folder, server, ModelConfig(**dict(stated, n_key_value_heads=stated["n_key_value_heads"] + 1)))
+
+
 class LetterTokenizer:
     """Token t is the letter chr(97 + t % 26); no end-of-text token."""
 
