@@ -119,6 +119,26 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
     }
   }
 
+  // What the norm-preparing epilogue reads from memory beside the sums is asked for here too
+  // (a workgroup has at least 256 threads): behind the last product that trip to memory would
+  // be the kernel's tail (0.7 us of 16 on the o-proj and down products of a 4,096-wide model).
+  // PREP, element e = tid + i * threads: column c of the tile, row m
+  constexpr int PREPS = (MT * 256 + 255) / 256;
+  float prep_h[PREP ? PREPS : 1], prep_w[PREP ? PREPS : 1];
+  if constexpr (PREP) {
+#pragma unroll
+    for (int i = 0; i < PREPS; ++i) {
+      const int e = tid + i * (int)blockDim.x;
+      prep_h[i] = 0.f, prep_w[i] = 0.f;
+      if (e >= MT * 256) continue;
+      const int t = e / 256, c = (e % 256) / 16, m = t * 16 + e % 16, n = n_base + c;
+      if (n < N && m < M) {
+        prep_h[i] = ((const float*)C)[(size_t)m * ldc + n];
+        prep_w[i] = load_as_f32(nf.norm_w, nf.norm_w_dtype, n);
+      }
+    }
+  }
+
   f32x4 acc[SETS][NT][MT];
 #pragma unroll
   for (int s = 0; s < SETS; ++s)
@@ -311,18 +331,19 @@ __global__ void skinny_gemm_kernel(const bf16_t* __restrict__ X, int ldx,
   if constexpr (PREP) {
     // thread (column c of the tile, row m): h += product (rounded to bf16 first, as the
     // unfused way hands it on), the next norm's input, and h^2 for the row's sum
-    for (int e = tid; e < MT * 256; e += blockDim.x) {
+#pragma unroll
+    for (int i = 0; i < PREPS; ++i) {
+      const int e = tid + i * (int)blockDim.x;
+      if (e >= MT * 256) continue;
       const int t = e / 256, c = (e % 256) / 16, m = t * 16 + e % 16, n = n_base + c;
       const int idx = t * 256 + ((c / 4) * 16 + e % 16) * 4 + c % 4;
       float sq = 0.f;
       if (n < N && m < M) {
         float v = 0.f;
         for (int w = 0; w < slots; ++w) v += red[(size_t)w * TILE + idx];
-        float* hp = (float*)C + (size_t)m * ldc + n;
-        const float h = *hp + bf16_to_f32(f32_to_bf16(v));
-        *hp = h;
-        const float wn = load_as_f32(nf.norm_w, nf.norm_w_dtype, n);
-        nf.xw_out[(size_t)m * N + n] = f32_to_bf16(wn * bf16_to_f32(f32_to_bf16(h)));
+        const float h = prep_h[i] + bf16_to_f32(f32_to_bf16(v));
+        ((float*)C)[(size_t)m * ldc + n] = h;
+        nf.xw_out[(size_t)m * N + n] = f32_to_bf16(prep_w[i] * bf16_to_f32(f32_to_bf16(h)));
         sq = h * h;
       }
       row_sums[c][m] = sq;
@@ -370,6 +391,8 @@ static int launch_skinny(const bf16_t* X, int ldx, const bf16_t* W, const bf16_t
                          hipStream_t stream, RopeEpilogue rope = RopeEpilogue{},
                          NormFusion nf = NormFusion{}) {
   constexpr int SETS = GATED ? 2 : 1;
+  HAL_REQUIRE((FLAGS & SK_PREP) == 0 || waves >= 4,
+              "small-batch product: the norm-preparing epilogue takes at least four waves (%d)", waves);
   // LDS for the partial sums of all waves, or of a half, a quarter ... if that is too much
   const size_t per_wave = (size_t)SETS * NT * MT * 256 * sizeof(float);
   int slots = waves;
