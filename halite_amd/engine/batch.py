@@ -199,17 +199,8 @@ class StepContext:
         if self._dev is None:
             cap = None
             if self.static is not None:  # decode only: room for whatever the planner makes of these requests
-                tiles = self.n_segs * -(-(n_heads // n_kv_heads) // attention_kernels.ROWS_PER_ITEM)
-                most = attention_kernels.pieces_per_tile(tiles, n_kv_heads)
-                cap = plan.cap_items = attention_kernels.WAVES_PER_GROUP * tiles * most
-                # the launches are recorded once for all later plans: none of them cuts a key
-                # range into more pieces than this (into none at all where the tiles are many),
-                # and by this number the kernel merges the pieces itself or leaves them to the
-                # merge kernel
-                plan.cap_partials = tiles * most if most > 1 else 0
-                plan.cap_merges = tiles if most > attention_kernels.MERGED_IN_KERNEL else 0
-                plan.merged_in_kernel = 1 < most <= attention_kernels.MERGED_IN_KERNEL
-                plan.max_parts = most
+                attention_kernels.fix_room_for_decode(plan, self.n_segs, n_heads // n_kv_heads, n_kv_heads)
+                cap = plan.cap_items
             self._packer.add(plan.name + "_items", plan.items, None if cap is None else cap * attention_kernels.SMALL_ITEM_INTS)
             self._packer.add(plan.name + "_big", plan.big_items)
             self._packer.add(plan.name + "_merges", plan.merges, None if cap is None else plan.cap_merges * 8)

@@ -109,6 +109,22 @@ class AttentionPlan:
         return np.array([self.n_items, self.n_big, self.n_merges], dtype=np.int32)
 
 
+def fix_room_for_decode(plan: AttentionPlan, n_requests: int, group_size: int, n_kv_heads: int) -> None:
+    """Gives ``plan``, of a step of one token for each of ``n_requests`` requests, the room
+    that any such step's plan fits, whatever the requests' lengths, and says which way its
+    tiles' pieces are merged: what launches that are recorded once for all later steps of
+    this size need to know.  No plan cuts a key range into more pieces than
+    ``pieces_per_tile`` allows (into none at all where the tiles are many), and by that
+    number the attention kernel merges the pieces itself or leaves them to the merge kernel."""
+    tiles = n_requests * -(-group_size // ROWS_PER_ITEM)
+    most = pieces_per_tile(tiles, n_kv_heads)
+    plan.cap_items = WAVES_PER_GROUP * tiles * most
+    plan.cap_partials = tiles * most if most > 1 else 0
+    plan.cap_merges = tiles if most > MERGED_IN_KERNEL else 0
+    plan.merged_in_kernel = 1 < most <= MERGED_IN_KERNEL
+    plan.max_parts = most
+
+
 def mfma_supported(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
     return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and page_size % 8 == 0
 

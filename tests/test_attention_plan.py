@@ -208,3 +208,26 @@ def test_random_steps_are_covered():
         except AssertionError as e:
             raise AssertionError(f"case {case}: q {q_len.tolist()} kv {kv_len.tolist()} group {group} kv heads {kv_heads} "
                                  f"window {window} rows {rows_big}") from e
+
+
+def test_recorded_decode_steps_have_room_for_any_lengths():
+    """A decode step that is replayed from a graph has the launches and the room of the step
+    it was recorded with; whatever the requests' lengths later are, the plan fits that room
+    and merges its pieces the same way."""
+    from halite_amd.kernels.attention import fix_room_for_decode
+
+    rng = np.random.default_rng(3)
+    for case in range(400):
+        n = int(rng.integers(1, 70))
+        # (more than 16 heads to a key/value head make a token a long segment: such steps are not recorded)
+        group, kv_heads = int(rng.choice([1, 2, 4, 8, 16])), int(rng.choice([1, 2, 8]))
+        window = int(rng.choice([0, 0, 500]))
+        first = plan_items(np.ones(n, dtype=np.int32), np.ones(n, dtype=np.int32), group, kv_heads, window)
+        fix_room_for_decode(first, n, group, kv_heads)
+        kv_len = rng.integers(1, int(rng.choice([40, 2000, 200000])), n).astype(np.int32)
+        plan = plan_items(np.ones(n, dtype=np.int32), kv_len, group, kv_heads, window)
+        assert plan.n_big == 0 and plan.n_items <= first.cap_items and plan.n_items % 4 == 0
+        assert plan.n_merges <= first.cap_merges and plan.n_partials <= first.cap_partials
+        assert plan.max_parts <= first.max_parts
+        if plan.n_partials:  # some range is cut: by the kernel itself or by the merge kernel, as recorded
+            assert plan.merged_in_kernel == first.merged_in_kernel and (plan.n_merges > 0) == (first.cap_merges > 0)
