@@ -141,7 +141,7 @@ def _tiles(seg_q_len, seg_kv_len, group_size, window, rows_per_tile, pick):
     ql = np.asarray(seg_q_len, dtype=np.int64)
     kl = np.asarray(seg_kv_len, dtype=np.int64)
     rows = ql * group_size
-    chosen = np.nonzero(pick(rows) & (rows > 0))[0] if len(ql) else np.zeros(0, dtype=np.int64)
+    chosen = np.nonzero(pick(rows, ql) & (rows > 0))[0] if len(ql) else np.zeros(0, dtype=np.int64)
     if len(chosen) == 0:
         z = np.zeros(0, dtype=np.int64)
         return z, z, z, z
@@ -311,16 +311,19 @@ def _group_tiles(seg_ids, rho0s, kv_b, kv_e, per_item: int):
 
 def plan_items(seg_q_len, seg_kv_len, group_size: int, n_kv_heads: int, window: int,
                rows_big: int = 64) -> AttentionPlan:
-    """Cuts the step's query rows into tiles of 16 rows.  A segment of at most 16 rows
-    (decode tokens) gives one-tile items, four to a workgroup, which takes a piece of the
-    tile's key range; a longer segment gives items of ``rows_big / 16`` tiles that share the
-    keys a wave loads.  Where there are too few items to fill the GPU, a key range is cut
+    """Cuts the step's query rows into tiles of 16 rows.  A segment of at most 16 rows or
+    of one token (decode tokens) gives one-tile items, four to a workgroup, which takes a
+    piece of the tile's key range; a longer segment gives items of ``rows_big / 16`` tiles
+    that share the keys a wave loads.  Where there are too few items to fill the GPU, a key range is cut
     into pieces whose partial results are merged."""
     ql = np.asarray(seg_q_len, dtype=np.int64).reshape(-1)
     seg_scalars = np.stack((np.cumsum(ql) - ql, ql, np.asarray(seg_kv_len, dtype=np.int64).reshape(-1)), axis=1)
     per_item = max(1, rows_big // ROWS_PER_ITEM)
-    small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: (r <= ROWS_PER_ITEM) | (per_item == 1))
-    big = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r: (r > ROWS_PER_ITEM) & (per_item > 1))
+    # (a single token is never a long segment, however many heads share its keys: a decode
+    # step then has one-tile items only, whose room is known before the lengths are)
+    short = lambda r, q: (r <= ROWS_PER_ITEM) | (q == 1) | (per_item == 1)
+    small = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, short)
+    big = _tiles(seg_q_len, seg_kv_len, group_size, window, ROWS_PER_ITEM, lambda r, q: ~short(r, q))
     items, merges_s, slot = _cut_joined(*small, pieces_per_tile(len(small[0]), n_kv_heads), 0, seg_scalars)
     more = None
     if len(big[0]):

@@ -50,7 +50,7 @@ def check_plan(plan, q_len, kv_len, group, window):
                 assert (b, e) == (0, 0)
                 continue
             rows = q_len[seg] * group
-            assert (rows > 16 and per_item > 1) == is_big
+            assert (rows > 16 and q_len[seg] > 1 and per_item > 1) == is_big
             assert 0 <= b < e <= kv_len[seg]
             tiles = tuple([rho0] + [m for m in more[: per_item - 1] if m >= 0]) if is_big else (rho0,)
             if not is_big:  # the segment's first token, tokens and keys ride along
@@ -74,7 +74,7 @@ def check_plan(plan, q_len, kv_len, group, window):
             lo = t_lo if lo is None else min(lo, t_lo)
             hi = t_hi if hi is None else max(hi, t_hi)
         pieces.sort()
-        if len(tiles) == 1 and (rows <= 16 or per_item == 1):  # the quarters of a piece share its slot
+        if len(tiles) == 1 and (rows <= 16 or q_len[seg] == 1 or per_item == 1):  # the quarters of a piece share its slot
             whole = []
             for b, e, p in pieces:
                 if whole and whole[-1][2] == p and (p >= 0 or whole[-1][1] == b):
@@ -89,7 +89,7 @@ def check_plan(plan, q_len, kv_len, group, window):
         if len(pieces) == 1:
             assert pieces[0][2] == -1
             continue
-        stride = per_item if len(tiles) > 1 or rows > 16 and per_item > 1 else 1
+        stride = per_item if len(tiles) > 1 or rows > 16 and q_len[seg] > 1 and per_item > 1 else 1
         slots = [p for _, _, p in pieces]
         assert slots == list(range(slots[0], slots[0] + stride * len(slots), stride))
         if (seg, tiles) in in_kernel:  # merged by the attention kernel: no merge entry
@@ -219,8 +219,7 @@ def test_recorded_decode_steps_have_room_for_any_lengths():
     rng = np.random.default_rng(3)
     for case in range(400):
         n = int(rng.integers(1, 70))
-        # (more than 16 heads to a key/value head make a token a long segment: such steps are not recorded)
-        group, kv_heads = int(rng.choice([1, 2, 4, 8, 16])), int(rng.choice([1, 2, 8]))
+        group, kv_heads = int(rng.choice([1, 2, 4, 8, 16, 20, 40])), int(rng.choice([1, 2, 8]))
         window = int(rng.choice([0, 0, 500]))
         first = plan_items(np.ones(n, dtype=np.int32), np.ones(n, dtype=np.int32), group, kv_heads, window)
         fix_room_for_decode(first, n, group, kv_heads)

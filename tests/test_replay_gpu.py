@@ -431,3 +431,28 @@ def test_a_decode_graph_serves_key_ranges_of_one_piece_and_of_several(dtype, tmp
     rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
     assert sorted(runner._graphs) == [2] and runner.graph_replays >= 56
     replay.compare(rows, ref, TOL[dtype])
+
+
+def test_twenty_heads_to_a_key_value_head_decode_from_a_graph(tmp_path):
+    """More than 16 heads share a key/value head: a token's rows are two tiles, and a decode
+    step still has one-tile items only, so it is recorded and replayed like any other; its
+    key ranges are cut into pieces (40 tiles and key/value heads: six a tile at most) that
+    the attention kernel merges itself."""
+    cfg = dict(tiny.TINY_A, hidden_size=320, num_attention_heads=20, num_key_value_heads=1, head_dim=16,
+               intermediate_size=96, num_hidden_layers=2, vocab_size=331, max_position_embeddings=2048)
+    weights = tiny.random_weights(cfg, seed=5, std=0.06)
+    a, b = tiny.random_tokens(cfg, 1300, 90), tiny.random_tokens(cfg, 60, 91)
+    folder = str(tmp_path / "model")
+    tiny.write_model_folder(folder, cfg, weights, torch.bfloat16)
+    pc, pw = plain_llama.read_model_folder(folder)
+    ref = {"a": plain_llama.forward(pc, pw, a), "b": plain_llama.forward(pc, pw, b)}
+    trace = [{"step": 0, "entries": [{"id": "a", "tokens": a[:1250], "want": []}, {"id": "b", "tokens": b[:20], "want": []}], "end": []}]
+    for i in range(40):
+        trace.append({"step": len(trace), "entries": [{"id": "a", "tokens": [a[1250 + i]], "want": [0]},
+                                                       {"id": "b", "tokens": [b[20 + i]], "want": [0]}], "end": []})
+    trace[-1]["end"] = ["a", "b"]
+    server = ServerConfig(kv_cache_num_tokens=1536, page_size=64, max_seqs_per_forward=4, use_cudagraph=True)
+    runner = ModelRunner.from_pretrained(folder, server, ModelConfig(dtype="bfloat16"))
+    rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
+    assert sorted(runner._graphs) == [2] and runner.graph_replays >= 36
+    replay.compare(rows, ref, TOL["bfloat16"])
