@@ -455,10 +455,21 @@ def test_attention_mfma_merges_in_the_kernel_the_same_every_time(gpu):
     for i, n in enumerate(lens):
         bt[i, : -(-n // page)] = order[at : at + -(-n // page)]
         at += -(-n // page)
-    q = torch.randn((len(lens), H * D), generator=rng).to(torch.bfloat16).to(gpu)
+    q = torch.randn((len(lens), H * D), generator=rng).to(torch.bfloat16)
+    # one key in the third of the first request's four pieces gets most of the weight: a piece
+    # that is dropped, or merged with a wrong maximum, shows
+    far = 1700
+    far_page, far_off = int(bt[0, far // page]), far % page
+    k_pages[far_page, :, far_off, :] = 0
+    k_pages[far_page, :, far_off, 1] = 8.0
+    v_pages[far_page, :, :, far_off] = 3.0
+    q[0].view(H, D)[:, 1] = 12.0
+    q = q.to(gpu)
     q_len, kv_len = np.ones(len(lens), dtype=np.int32), np.array(lens, dtype=np.int32)
     plan = attn_kernels.plan_items(q_len, kv_len, H // K, K, 0, attn_kernels.rows_per_big_item(D))
     assert plan.merged_in_kernel and plan.n_merges == 0 and (plan.items[:, 9] == 4).all()
+    holds_far = plan.items[(plan.items[:, 0] == 0) & (plan.items[:, 2] <= far) & (far < plan.items[:, 3])]
+    assert len(holds_far) == 1 and holds_far[0, 4] - holds_far[0, 8] == 2  # the third piece's slot
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
 
     class Ctx:
@@ -483,6 +494,8 @@ def test_attention_mfma_merges_in_the_kernel_the_same_every_time(gpu):
         qi = q[i].float().cpu().view(H, D)
         want = torch.stack([torch.softmax(k[:, h // (H // K)] @ qi[h] * D**-0.5, 0) @ v[:, h // (H // K)] for h in range(H)])
         close(first[i].view(H, D), want, 1.2e-2, f"request {i}")
+        if i == 0:
+            assert float(want.abs().min()) > 0.5  # the far key decides
     for _ in range(300):
         again = attn_kernels.attention_mfma(q, H * D, plan_dev, Ctx, Group, KV, H, D**-0.5, 0)
         assert torch.equal(again, first)
