@@ -78,17 +78,18 @@ def generate(args) -> int:
         from ..config import parse_config
 
         with open(args.random) as f:
-            _, cfg = parse_config(json.load(f))
+            arch, cfg = parse_config(json.load(f))
     else:
-        _, cfg = read_config(args.model)
+        arch, cfg = read_config(args.model)
     prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
     if args.prompt_file:
         with open(args.prompt_file) as f:
             prompts += [json.loads(line) for line in f if line.strip()]
     if args.prompt_lens:
         gen = torch.Generator().manual_seed(args.prompt_seed)
+        vocab_size = arch.to_spec(cfg).vocab_size  # (the configuration's own key for it is the architecture's business)
         for n in args.prompt_lens.split(","):
-            prompts.append(torch.randint(0, cfg.vocab_size, (int(n),), generator=gen).tolist())
+            prompts.append(torch.randint(0, vocab_size, (int(n),), generator=gen).tolist())
     if not prompts:
         raise SystemExit("no prompts: give --prompt-ids, --prompt-file or --prompt-lens")
 

@@ -26,6 +26,16 @@ class ConfigError(ValueError):
 
 @dataclass(frozen=True)
 class Architecture:
+    """What the framework asks of an architecture.
+
+    ``config_cls`` is a pydantic model of the architecture's ``config.json``.  Beside its
+    own keys it must have the field ``architectures`` (a list whose first entry is
+    ``name``: what a model folder is recognised by, and what the random-weights mode
+    writes).  It may have ``stop_token_ids`` (token ids that end a request unless it asks
+    to ignore them) and a method ``to_json_dict()`` (the ``config.json`` to write, if
+    ``model_dump(exclude_none=True)`` is not it).  Nothing else of it is read outside
+    ``to_spec`` and ``weight_map``, which are the architecture's own."""
+
     name: str
     config_cls: type[BaseModel]
     to_spec: Callable[[BaseModel], ModelSpec]
@@ -38,6 +48,15 @@ ARCHITECTURES: dict[str, Architecture] = {}
 
 
 def register_architecture(arch: Architecture) -> Architecture:
+    fields = getattr(arch.config_cls, "model_fields", None)
+    if fields is None or "architectures" not in fields:
+        raise ConfigError(
+            f"architecture {arch.name!r}: its configuration class must be a pydantic model with "
+            "the field 'architectures'"
+        )
+    for optional in ("to_json_dict",):
+        if hasattr(arch.config_cls, optional) and not callable(getattr(arch.config_cls, optional)):
+            raise ConfigError(f"architecture {arch.name!r}: {optional} of its configuration class is not a method")
     ARCHITECTURES[arch.name] = arch
     return arch
 

@@ -208,7 +208,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
   const int j_first = walk_begin & ~31;
   // PAGE32: page numbers are looked up (scalar loads) well before the loads that need them
   auto page_at = [&](int j0) {
-    if constexpr (PAGE32) return uniform(bt[(j0 < walk_end ? j0 : j_first) >> page_shift]);
+    // (an entry of a page that a window has passed is -1: never an address)
+    if constexpr (PAGE32) return max(uniform(bt[(j0 < walk_end ? j0 : j_first) >> page_shift]), 0);
     else return 0;
   };
   // with LDS: the pages of this half's first three steps are asked for here, so that they

@@ -71,9 +71,8 @@ class ModelRunner:
             st = mixer.state_need()
             if st:
                 state_needs[i] = st
-        check_stated_sizes(self.model_config, len(spec.order), [
-            (getattr(model.mixer_of_run(i).p, "n_heads", need.n_kv_heads), need.n_kv_heads, need.head_dim)
-            for i, need in needs.items()])
+        sizes = [model.mixer_of_run(i).attention_sizes() for i in range(len(spec.order))]
+        check_stated_sizes(self.model_config, len(spec.order), [s for s in sizes if s is not None])
         page_size = self.server_config.page_size
         n_slots = self.server_config.max_seqs_per_forward
         num_pages = self._size_pool(needs, page_size, model.dtype)
@@ -299,14 +298,19 @@ class ModelRunner:
         if ahead is None:  # a step that was put together ahead has its pages already
             self.cache.reserve(spans)
         logits = None
-        if graph_step:
-            logits = self._step_graph(segments, ahead)
-        if logits is None:
-            ctx = StepContext(segments, self.cache, self.device, self._staging)
-            for run in self.model.runs:
-                self.model.mixer_of_run(run.index).prepare(ctx, run)
-            self._feed_tokens(ctx)
-            logits = self.model.forward(ctx)
+        try:
+            if graph_step:
+                logits = self._step_graph(segments, ahead)
+            if logits is None:
+                ctx = StepContext(segments, self.cache, self.device, self._staging)
+                for run in self.model.runs:
+                    self.model.mixer_of_run(run.index).prepare(ctx, run)
+                self._feed_tokens(ctx)
+                logits = self.model.forward(ctx)
+        except BaseException:
+            # a step that stops half-way may leave pieces counted that nobody merged
+            attention_kernels.reset_counters(self.device)
+            raise
         for slot, new_len in spans:
             self.cache.advance(slot, new_len)
         if graph_step:

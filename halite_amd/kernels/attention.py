@@ -30,7 +30,7 @@ BIG_ITEM_INTS = 16  # an item of the kernel for long segments: 8, then what its 
 # reads a second, so an even share each counts for more than many waves: measured), and no
 # piece shorter than this many keys (below, a second piece and the merge cost more than the
 # shorter walk saves).
-COMPUTE_UNITS = 256
+COMPUTE_UNITS = 256  # of the MI355X; the device that runs is asked (`compute_units`)
 MIN_PIECE_KEYS = 384
 # Up to this many pieces a tile the attention kernel merges the partial results itself (the
 # workgroup that finishes a tile last does, in the same launch: 1 to 3 us less than a merge
@@ -40,10 +40,25 @@ MERGED_IN_KERNEL = 8
 N_COUNTERS = 1 << 14  # one per (tile that the kernel merges, key/value head); a tile has pieces only while these are few
 
 
+_compute_units: int | None = None
+
+
+def compute_units() -> int:
+    """Compute units of the device that runs the kernels, asked once (without a device,
+    as where the planner is tested: the MI355X's)."""
+    global _compute_units
+    if _compute_units is None:
+        if torch.cuda.is_available():
+            _compute_units = int(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count)
+        else:
+            _compute_units = COMPUTE_UNITS
+    return _compute_units
+
+
 def pieces_per_tile(n_tiles: int, n_kv_heads: int) -> int:
     """Into how many pieces, at most, the key range of each of ``n_tiles`` one-tile items
     is cut (every piece is one workgroup per key/value head)."""
-    return max(1, COMPUTE_UNITS // max(1, n_tiles * n_kv_heads))
+    return max(1, compute_units() // max(1, n_tiles * n_kv_heads))
 
 
 @dataclass
@@ -223,11 +238,14 @@ def _cut_joined(seg_ids, rho0s, kv_b, kv_e, most_pieces, first_slot, seg_scalars
     b = np.maximum(kv_b[tile_of][:, None], edge[:, :-1])
     e = np.minimum(kv_e[tile_of][:, None], edge[:, 1:])
     empty = b >= e
+    # (an empty item names the piece's first key twice: the kernel asks for the page of an
+    # item's first key before it knows whether the item has any, and under a window the
+    # pages before the piece may have been given back)
     items = np.zeros((total, WAVES_PER_GROUP, SMALL_ITEM_INTS), dtype=np.int32)
     items[:, :, 0] = seg_ids[tile_of][:, None]
     items[:, :, 1] = rho0s[tile_of][:, None]
-    items[:, :, 2] = np.where(empty, 0, b)
-    items[:, :, 3] = np.where(empty, 0, e)
+    items[:, :, 2] = np.where(empty, b[:, :1], b)
+    items[:, :, 3] = np.where(empty, b[:, :1], e)
     items[:, :, 5:8] = seg_scalars[seg_ids[tile_of]][:, None, :]
     split = n_pieces[tile_of] > 1
     n_split = int(split.sum())
@@ -355,6 +373,23 @@ def _counters(device) -> torch.Tensor:
     if key not in _COUNTERS:
         _COUNTERS[key] = torch.zeros(N_COUNTERS, dtype=torch.int32, device=device)
     return _COUNTERS[key]
+
+
+def reset_counters(device) -> None:
+    """Sets the device's counters back to zero (a kernel on the current stream): after a
+    step that raised, whose attention kernels may have counted pieces that nobody merged."""
+    device = torch.device(device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    if key in _COUNTERS:
+        _COUNTERS[key].zero_()
+
+
+def counters_idle(device) -> bool:
+    """Whether every counter is zero, as it is between launches (a check for tests; it
+    waits for the device)."""
+    device = torch.device(device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    return key not in _COUNTERS or int(_COUNTERS[key].abs().sum()) == 0
 
 
 def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, window):

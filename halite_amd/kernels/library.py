@@ -164,12 +164,24 @@ def _filter(stderr: str) -> str:
     )
 
 
+def _check_device() -> None:
+    """The kernels use instructions and LDS sizes of gfx950 alone; another GPU is refused
+    here rather than met by a code object that does not load."""
+    import torch
+
+    if torch.cuda.is_available():
+        name = torch.cuda.get_device_properties(torch.cuda.current_device()).gcnArchName
+        if not name.startswith(ARCH):
+            raise KernelLibraryError(f"the HIP kernels are written for {ARCH} (MI355X); this GPU is {name}")
+
+
 def load_library(name: str, sources: list[str], defines: dict[str, int] | None = None) -> ctypes.CDLL:
     defines = defines or {}
     key = name + repr(sorted(defines.items()))
     with _lock:
         if key in _loaded:
             return _loaded[key]
+        _check_device()
         path = build_library(name, sources, defines)
         try:
             lib = ctypes.CDLL(path)

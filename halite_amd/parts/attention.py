@@ -97,6 +97,9 @@ class Attention(Mixer):
                     steps = -(-p.hidden_size // 32)
                     self.t_q = self.t_qkv[: (n_q // 16) * steps * 512]
 
+    def attention_sizes(self):
+        return self.p.n_heads, self.p.n_kv_heads, self.p.head_dim
+
     def cache_need(self):
         return PagedKVNeed(self.p.n_kv_heads, self.p.head_dim, self.p.window)
 

@@ -129,6 +129,12 @@ class Mixer(Part):
     takes_normed_rows: ClassVar[bool] = False
     folds_next_norm: ClassVar[bool] = False
 
+    def attention_sizes(self) -> tuple[int, int, int] | None:
+        """(query heads, key/value heads, head size) if the mixer has such sizes, for the
+        check of sizes that a caller states beside the model (``ModelConfig.n_heads`` and
+        its like); None if it has none."""
+        return None
+
     def prepare(self, ctx: "StepContext", run: RunBinding) -> None:
         """Called for every run before the step's arrays go to the device; a mixer
         may add host-built arrays of its own to that one copy."""
@@ -195,6 +201,10 @@ class Embedding(Part):
 
 
 class Head(Part):
+    def bind(self, embedding: "Embedding") -> None:
+        """Called once, before ``finalize``, with the model's embedding: a head that shares
+        tensors with it (tied weights) takes them here."""
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 

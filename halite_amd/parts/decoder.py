@@ -86,8 +86,7 @@ class Decoder:
         return self.layers[self.spec.order[index].layer].mixer
 
     def finalize(self):
-        if getattr(self.head.p, "tied", False):
-            self.head.tie(self.embedding)
+        self.head.bind(self.embedding)
         for part in self.named_parts().values():
             part.finalize()
 

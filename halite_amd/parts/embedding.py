@@ -51,8 +51,9 @@ class LinearHead(Head):
             return {}
         return {"weight": ParamDecl((self.p.vocab_size, self.p.size))}
 
-    def tie(self, embedding: TokenEmbedding):
-        self.weight = embedding.weight
+    def bind(self, embedding):
+        if self.p.tied:
+            self.weight = embedding.weight
 
     def finalize(self):
         self.t_weight = None

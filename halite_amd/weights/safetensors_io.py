@@ -125,15 +125,15 @@ class ModelFiles:
             raise SafetensorsError(f"{folder}: no model.safetensors and no model.safetensors.index.json")
         if problems:
             raise SafetensorsError(f"{folder}: " + "; ".join(problems))
-        by_file = {}
+        names_in = {}  # path of a file -> the names of its tensors
         for p in paths:
             sf = SafetensorsFile(p)
             self.files.append(sf)
-            by_file[os.path.basename(p)] = sf
-            for name in sf.names():
+            names_in[p] = set(sf.names())
+            for name in names_in[p]:
                 self.where[name] = sf
-        for name, shard in shard_of.items():
-            if name not in by_file[shard].names():
+        for name, shard in shard_of.items():  # (a shard may be named with a subfolder)
+            if name not in names_in[os.path.join(folder, shard)]:
                 self.notes.append(f"the index lists {name} in {shard}, which does not hold it")
 
     def names(self):

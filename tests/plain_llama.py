@@ -103,13 +103,18 @@ def rotate_interleaved(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor):
 # --------------------------------------------------------------------------
 
 
-def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, round_to=None) -> torch.Tensor:
     """``weight * (x32 * rsqrt(mean(x32^2) + eps)).type_as(x)``.
+
+    With ``round_to`` the model's element type is that one: the normalised row is rounded to
+    it before the weight multiplies it (the ``type_as``), and so is the product.
 
     src/halite/nn/normalization.py:43-57
     """
     x32 = x.to(torch.float32)
     normed = x32 * torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + eps)
+    if round_to is not None:
+        return (weight * normed.to(round_to).float()).to(round_to).float()
     return weight * normed.type_as(x)
 
 
@@ -202,11 +207,20 @@ def rope_frequencies_of(config: dict) -> torch.Tensor:
     return inv_freq
 
 
-def forward(config: dict, weights: dict, ids, position_offset: int = 0) -> torch.Tensor:
+def forward(config: dict, weights: dict, ids, position_offset: int = 0, round_to=None) -> torch.Tensor:
     """Logits ``[n, vocab]`` (float32) of one whole token sequence.
 
     The order in a layer is norm, q/k/v, rotation, attention, out, add, norm,
     gate/up, silu*mul, down, add.
+
+    ``round_to`` (``torch.bfloat16``): a model whose element type is that one, emulated in
+    float32: the result of every product, the rotated queries and keys, the attention's
+    output, the activation and the norms' results are rounded to it; the norms' statistics,
+    the rotation, the softmax and the residual sum stay float32 (the parts that are 32-bit
+    whatever the model's type: src/halite/nn/normalization.py:43-57,
+    src/halite/transformers/position.py:294-300, src/halite/transformers/attention.py:708).
+    The arithmetic inside a product stays float32.  It says how far a model of that type may
+    lie from 32-bit arithmetic through the number format alone.
     src/halite/transformers/block.py:56-74 (``x + module(pre_norm(x))``),
     src/halite/transformers/infer/attention.py:157-172,
     src/halite/transformers/infer/transformer.py:82-114
@@ -223,25 +237,34 @@ def forward(config: dict, weights: dict, ids, position_offset: int = 0) -> torch
     cos, sin = rotation_table(
         torch.arange(n) + position_offset, rope_frequencies_of(config)
     )
+    def r(t):
+        return t if round_to is None else t.to(round_to).float()
+
     h = embed(ids, weights["model.embed_tokens.weight"])
     for i in range(config["num_hidden_layers"]):
         p = f"model.layers.{i}."
-        x = rms_norm(h, weights[p + "input_layernorm.weight"], eps)
-        q = (x @ weights[p + "self_attn.q_proj.weight"].T).view(n, n_heads, head_dim)
-        k = (x @ weights[p + "self_attn.k_proj.weight"].T).view(n, n_kv, head_dim)
-        v = (x @ weights[p + "self_attn.v_proj.weight"].T).view(n, n_kv, head_dim)
-        q = rotate(q, cos, sin)
-        k = rotate(k, cos, sin)
-        a = causal_attention(q, k, v).reshape(n, n_heads * head_dim)
-        h = h + a @ weights[p + "self_attn.o_proj.weight"].T
-        x = rms_norm(h, weights[p + "post_attention_layernorm.weight"], eps)
-        h = h + gated_feed_forward(
-            x,
-            weights[p + "mlp.gate_proj.weight"],
-            weights[p + "mlp.up_proj.weight"],
-            weights[p + "mlp.down_proj.weight"],
-        )
-    h = rms_norm(h, weights["model.norm.weight"], eps)
+        x = rms_norm(h, weights[p + "input_layernorm.weight"], eps, round_to)
+        q = r(x @ weights[p + "self_attn.q_proj.weight"].T).view(n, n_heads, head_dim)
+        k = r(x @ weights[p + "self_attn.k_proj.weight"].T).view(n, n_kv, head_dim)
+        v = r(x @ weights[p + "self_attn.v_proj.weight"].T).view(n, n_kv, head_dim)
+        q = r(rotate(q, cos, sin))
+        k = r(rotate(k, cos, sin))
+        a = r(causal_attention(q, k, v)).reshape(n, n_heads * head_dim)
+        h = h + r(a @ weights[p + "self_attn.o_proj.weight"].T)
+        x = rms_norm(h, weights[p + "post_attention_layernorm.weight"], eps, round_to)
+        if round_to is None:
+            f = gated_feed_forward(
+                x,
+                weights[p + "mlp.gate_proj.weight"],
+                weights[p + "mlp.up_proj.weight"],
+                weights[p + "mlp.down_proj.weight"],
+            )
+        else:  # the same formula with the activation and the result rounded
+            gate = x @ weights[p + "mlp.gate_proj.weight"].T
+            up = x @ weights[p + "mlp.up_proj.weight"].T
+            f = r(r(up * (gate * torch.sigmoid(gate))) @ weights[p + "mlp.down_proj.weight"].T)
+        h = h + f
+    h = rms_norm(h, weights["model.norm.weight"], eps, round_to)
     if config.get("tie_word_embeddings", False):
         head = weights["model.embed_tokens.weight"]
     else:

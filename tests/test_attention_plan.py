@@ -33,7 +33,8 @@ def check_plan(plan, q_len, kv_len, group, window):
         assert len(set(map(tuple, run[:, [0, 1, 4, 5, 6, 7, 8, 9]].tolist()))) == 1 and (run[:, 10:] == 0).all()
         live = run[run[:, 3] > run[:, 2]]
         assert run[0, 3] > run[0, 2] and (live[1:, 2] == live[:-1, 3]).all() and (live[:-1, 3] % 32 == 0).all()
-        assert (run[run[:, 3] <= run[:, 2], 2:4] == 0).all()
+        # an empty quarter names the piece's first key twice: a key whose page is held
+        assert (run[run[:, 3] <= run[:, 2], 2:4] == run[0, 2]).all()
         blocks = -(-(live[:, 3] - live[:, 2] // 32 * 32) // 32)
         assert blocks.max() - blocks.min() <= 1 or len(live) < 4
     in_kernel = {}  # (segment, tile) -> (first partial slot, pieces) that the items themselves name
@@ -47,7 +48,9 @@ def check_plan(plan, q_len, kv_len, group, window):
                 assert (b, e, partial, more) == (0, 0, -1, [-1, -1, -1])
                 continue
             if not is_big and b == e:  # an empty quarter of a short piece
-                assert (b, e) == (0, 0)
+                pos0 = kv_len[seg] - q_len[seg]
+                first_seen = 0 if window <= 0 else max(0, pos0 + rho0 // group - window + 1)
+                assert first_seen <= b < kv_len[seg]  # inside the window: its page is held
                 continue
             rows = q_len[seg] * group
             assert (rows > 16 and q_len[seg] > 1 and per_item > 1) == is_big

@@ -209,3 +209,27 @@ def test_command_line_takes_overrides_and_options_in_any_order():
     assert over == {"sampling": {"max_new_tokens": 4}, "server": {"page_size": 16}, "model": {"dtype": "float32"}}
     with pytest.raises(SystemExit):
         split_overrides(["foo=1"])
+
+
+def test_an_architecture_must_bring_what_the_framework_reads_of_its_configuration():
+    """``architectures`` is the one field that generic code reads of a configuration class;
+    a class without it is refused when it is registered, not when a folder is written."""
+    from pydantic import BaseModel
+
+    from halite_amd.config.registry import ARCHITECTURES, Architecture, ConfigError, register_architecture
+
+    class Nameless(BaseModel):
+        width: int
+
+    with pytest.raises(ConfigError, match="architectures"):
+        register_architecture(Architecture("NamelessLM", Nameless, lambda c: None, lambda c: {}))
+    assert "NamelessLM" not in ARCHITECTURES
+
+    class Named(BaseModel):
+        architectures: list[str]
+        width: int
+
+    try:
+        assert register_architecture(Architecture("NamedLM", Named, lambda c: None, lambda c: {})).name == "NamedLM"
+    finally:
+        ARCHITECTURES.pop("NamedLM", None)

@@ -367,6 +367,13 @@ def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use, tiled=Fal
     for i, t in enumerate(tables):
         bt[i, : len(t)] = t
     k_pages, v_pages = torch.cat(kps), torch.cat(vps)
+    if window:
+        # pages that the window of a segment's first new token has passed are given back in
+        # the engine; here their entries name a page of NaN, so that a kernel that uses one shows
+        k_pages = torch.cat((k_pages, torch.full_like(k_pages[:1], float("nan"))))
+        v_pages = torch.cat((v_pages, torch.full_like(v_pages[:1], float("nan"))))
+        for i, (before, new) in enumerate(segs):
+            bt[i, : max(0, before - window + 1) // page] = k_pages.shape[0] - 1
     if tiled:
         k_pages, v_pages = to_tiled(k_pages, v_pages)
     k_pages, v_pages, is_tiled = k_pages.to(gpu), v_pages.to(gpu), tiled

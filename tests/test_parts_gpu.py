@@ -649,7 +649,7 @@ TOY_MIX = dict(architectures=["ToyMixForCausalLM"], width=64, vocab=211, kinds=[
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_toy_architecture_from_its_config_file_to_generated_tokens(gpu, dtype, tmp_path):
+def test_a_toy_architecture_from_its_config_file_to_generated_tokens(gpu, dtype, tmp_path, capsys):
     """An architecture of its own (config keys, layer kinds that differ from layer to layer,
     tensor names) is registered here; the framework's folder writer, loader, engine,
     scheduler and sampler then serve it as they serve the built-in one."""
@@ -693,6 +693,17 @@ def test_a_toy_architecture_from_its_config_file_to_generated_tokens(gpu, dtype,
                 row = logits[len(p) - 1 + j]
                 assert float(row.max() - row[tok]) <= margin * max(1.0, float(row.abs().max())), (len(p), j)
         assert engine.stats.prefill_tokens >= sum(len(p) for p in prompts) and engine.model_runner.cache.idle()
+        # the command line draws random prompts from the toy's vocabulary, which its
+        # configuration calls by a name of its own
+        from halite_amd.cli import generate as command_line
+
+        capsys.readouterr()
+        status = command_line.main(["--model", folder, "--prompt-lens", "9,4", "--prompt-seed", "2", "sampling.temperature=0",
+                                    "sampling.max_new_tokens=3", f"model.dtype={dtype}", "server.kv_cache_num_tokens=256",
+                                    "server.max_seqs_per_forward=4"])
+        lines = [json.loads(line) for line in capsys.readouterr().out.strip().split("\n")]
+        assert status == 0 and [len(r["input_ids"]) for r in lines] == [9, 4]
+        assert all(0 <= t < 211 for r in lines for t in r["input_ids"] + r["output_ids"][0])
         # the loader's one error speaks the toy's tensor names
         from safetensors import safe_open
         from safetensors.torch import save_file

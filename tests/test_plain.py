@@ -233,8 +233,99 @@ def test_model_shift_invariance_and_causality():
     assert torch.allclose(a, b, atol=2e-5)  # only distances count
     c = P.forward(cfg, w, ids[:8])
     assert torch.allclose(a[:8], c, atol=1e-5)  # a prefix's logits do not see the rest
-    # tied head: the logits are hidden @ embedding^T
-    assert "lm_head.weight" not in w
+    # tied head: the logits are hidden @ embedding^T.  Another table handed in as a head is
+    # not looked at, and the logits follow the embedding table's rows
+    decoy = dict(w)
+    decoy["lm_head.weight"] = torch.randn_like(w["model.embed_tokens.weight"])
+    assert torch.equal(P.forward(cfg, decoy, ids), a)
+    swapped = dict(w)
+    table = w["model.embed_tokens.weight"].clone()
+    unused = [t for t in range(cfg["vocab_size"]) if t not in ids][:2]
+    table[unused] = table[unused[::-1]]  # two rows that no token of the input reads
+    swapped["model.embed_tokens.weight"] = table
+    d = P.forward(cfg, swapped, ids)
+    assert torch.equal(d[:, unused], a[:, unused[::-1]]) and not torch.equal(d[:, unused], a[:, unused])
+    # the same weights read as untied: the other table is the head then
+    assert not torch.allclose(P.forward(dict(cfg, tie_word_embeddings=False), decoy, ids), a, atol=1e-3)
+
+
+def library_model(cfg, w, ids):
+    """The whole model once more, from library routines alone and in the reference's own
+    formulation where it has one: ``F.embedding``, ``F.rms_norm``, ``F.linear``, the rotation
+    as a product of complex numbers (src/halite/transformers/position.py:140-167, 294-300),
+    ``F.scaled_dot_product_attention`` with ``is_causal`` and ``enable_gqa``
+    (src/halite/transformers/attention.py:600-609), ``F.silu``; a sub-block is
+    ``input + module(pre_norm(input))`` (src/halite/transformers/block.py:56-74), the last
+    norm and the head follow the last block (src/halite/transformers/infer/transformer.py:
+    105-112).  For configurations with ``rope_interleaved``."""
+    n = len(ids)
+    H, K = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    D = cfg.get("head_dim") or cfg["hidden_size"] // H
+    eps, width = cfg["rms_norm_eps"], (cfg["hidden_size"],)
+    freq = 1.0 / cfg["rope_theta"] ** (torch.arange(0, D, 2, dtype=torch.float32) / D)
+    sc = cfg.get("rope_scaling")
+    if sc is not None:  # the two-where form of src/halite/transformers/position.py:264-284
+        orig, factor = sc["original_max_position_embeddings"], sc["factor"]
+        lo, hi = sc["low_freq_factor"], sc["high_freq_factor"]
+        wl = 2 * math.pi / freq
+        first = torch.where(wl > orig / lo, freq / factor, freq)
+        smooth = (orig / wl - lo) / (hi - lo)
+        freq = torch.where(~(wl < orig / hi) & ~(wl > orig / lo), (1 - smooth) * first / factor + smooth * first, first)
+    ang = torch.outer(torch.arange(n, dtype=torch.float32), freq)
+    cis = torch.polar(torch.ones_like(ang), ang).unsqueeze(1)
+
+    def rotate(x):
+        return torch.view_as_real(torch.view_as_complex(x.float().reshape(n, -1, D // 2, 2)) * cis).flatten(-2)
+
+    h = F.embedding(torch.as_tensor(ids), w["model.embed_tokens.weight"])
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        x = F.rms_norm(h, width, w[p + "input_layernorm.weight"], eps)
+        q = rotate(F.linear(x, w[p + "self_attn.q_proj.weight"]).view(n, H, D))
+        k = rotate(F.linear(x, w[p + "self_attn.k_proj.weight"]).view(n, K, D))
+        v = F.linear(x, w[p + "self_attn.v_proj.weight"]).view(n, K, D)
+        a = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
+                                           is_causal=True, enable_gqa=True)[0].transpose(0, 1).reshape(n, H * D)
+        h = h + F.linear(a, w[p + "self_attn.o_proj.weight"])
+        x = F.rms_norm(h, width, w[p + "post_attention_layernorm.weight"], eps)
+        h = h + F.linear(F.silu(F.linear(x, w[p + "mlp.gate_proj.weight"])) * F.linear(x, w[p + "mlp.up_proj.weight"]),
+                         w[p + "mlp.down_proj.weight"])
+    head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
+    return F.linear(F.rms_norm(h, width, w["model.norm.weight"], eps), head)
+
+
+def rows_for_half_split(cfg, w):
+    """The same model stored for the half-split pairing: the rows of every head of the
+    query and key matrices reordered [0, 2, 4, ..., 1, 3, 5, ...]."""
+    D = cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_attention_heads"]
+    perm = torch.cat((torch.arange(0, D, 2), torch.arange(1, D, 2)))
+    out = dict(w)
+    for name, t in w.items():
+        if name.endswith(("q_proj.weight", "k_proj.weight")):
+            out[name] = t.view(-1, D, t.shape[1])[:, perm].reshape(t.shape)
+    return out
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_model_against_library_routines(name):
+    """Pins every formula and the order of a block at once: the plain implementation
+    against a model made of library routines (an outside model library is not used as a
+    yardstick here: model code of installed packages is no source for this repository).
+    Then the half-split pairing, which model folders are stored for, against the adjacent
+    one on the reordered rows."""
+    cfg = dict({"A": tiny.TINY_A, "B": tiny.TINY_B, "C": tiny.TINY_C}[name], rope_interleaved=True)
+    w = tiny.random_weights(cfg, 21, std=0.08)
+    for n, seed in ((1, 1), (37, 2), (cfg["max_position_embeddings"] // 2, 3)):
+        ids = tiny.random_tokens(cfg, n, seed)
+        want = library_model(cfg, w, ids)
+        got = P.forward(cfg, w, ids)
+        assert float((got - want).abs().max()) <= 1e-5 * max(1.0, float(want.abs().max())), (name, n)
+        half = P.forward(dict(cfg, rope_interleaved=False), rows_for_half_split(cfg, w), ids)
+        assert float((half - want).abs().max()) <= 1e-5 * max(1.0, float(want.abs().max())), (name, n)
+    # what the comparison would catch: a residual taken after the norm, a norm left out
+    broken = dict(w)
+    broken["model.norm.weight"] = torch.ones_like(w["model.norm.weight"])
+    assert float((P.forward(cfg, broken, ids) - want).abs().max()) > 1e-3
 
 
 def test_norm_weight_position_matters():
@@ -285,3 +376,23 @@ def test_sample_token_greedy_and_draw():
         counts[P.sample_token(logits, {"temperature": 1.0, "seed": 9}, i)[0]] += 1
     want = torch.softmax(logits, -1) * 3000
     assert ((counts - want).abs() < 4 * want.sqrt() + 5).all()
+
+
+def test_rounding_mode_rounds_where_it_says():
+    """``round_to`` emulates a model of that element type: float32 changes nothing, bfloat16
+    moves the logits by about its precision per rounding, and what is rounded is what the
+    docstring lists (a product's result: one layer's q, k, v are on the bfloat16 grid)."""
+    cfg = tiny.TINY_C
+    w = {k: v.to(torch.bfloat16).float() for k, v in tiny.random_weights(cfg, 5, std=0.06).items()}
+    ids = tiny.random_tokens(cfg, 40, 3)
+    exact = P.forward(cfg, w, ids)
+    assert torch.equal(P.forward(cfg, w, ids, round_to=torch.float32), exact)
+    rounded = P.forward(cfg, w, ids, round_to=torch.bfloat16)
+    err = float((rounded - exact).abs().max()) / float(exact.abs().max())
+    assert 1e-4 < err < 2e-2, err
+    x = torch.randn(5, cfg["hidden_size"])
+    weight = w["model.norm.weight"]
+    y = P.rms_norm(x, weight, 1e-6, torch.bfloat16)
+    assert torch.equal(y, y.to(torch.bfloat16).float())
+    inner = (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16).float()
+    assert torch.equal(y, (weight * inner).to(torch.bfloat16).float())  # rounded before the weight, as type_as does

@@ -44,8 +44,8 @@ def folders(tmp_path_factory):
     return out
 
 
-def make_runner(folder, dtype, tokens, page_size=64):
-    server = ServerConfig(kv_cache_num_tokens=tokens, page_size=page_size, max_seqs_per_forward=8)
+def make_runner(folder, dtype, tokens, page_size=64, **server_options):
+    server = ServerConfig(kv_cache_num_tokens=tokens, page_size=page_size, max_seqs_per_forward=8, **server_options)
     return ModelRunner.from_pretrained(folder, server, ModelConfig(dtype=dtype))
 
 
@@ -77,6 +77,28 @@ def test_schedules(folders, name, page, schedule, dtype):
     assert sum(len(v) for v in rows.values()) > 0
     replay.compare(rows, ref, TOL[dtype])
     assert runner.cache.idle()
+
+
+@pytest.mark.parametrize("schedule", list(SCHEDULES))
+@pytest.mark.parametrize("name,page", [("B", 16), ("B", 64), ("C", 64)])
+def test_schedules_on_row_major_weights(folders, name, page, schedule, monkeypatch):
+    """bfloat16 without the second, tiled copy of the matrices (a model too large for it, or
+    ``decode_weight_copy="off"``): steps of few tokens then take the norm, the products on
+    the row-major matrices and the rotation as kernels of their own, none of the fused ones."""
+    from halite_amd.kernels import ops
+
+    fused = []
+    for fn in ("qkv_rope_append", "gemm_bf16_skinny_norm"):
+        monkeypatch.setattr(ops, fn, lambda *a, _n=fn, **kw: fused.append(_n))
+    folder, requests, ref = folders[(name, "bfloat16")]
+    trace = SCHEDULES[schedule](requests)
+    runner = make_runner(folder, "bfloat16", replay.peak_tokens(trace, page), page, decode_weight_copy="off")
+    assert not runner.model.build.tiled_weights
+    for g in runner.cache.groups:
+        g.storage.fill_(float("nan"))
+    rows = replay.collect(trace, replay.run_trace(runner, trace), CONFIGS[name]["vocab_size"])
+    replay.compare(rows, ref, TOL["bfloat16"])
+    assert runner.cache.idle() and not fused
 
 
 def test_bfloat16_run_of_a_folder_stored_in_float32(folders):
@@ -173,8 +195,11 @@ def test_cuts_agree_with_each_other(folders, dtype):
 def test_small_pages_and_other_page_sizes(folders, dtype):
     folder, requests, ref = folders[("A", dtype)]
     trace = replay.mixed(requests, seed=3)
-    for page in ([1, 4, 8, 16] if dtype == "float32" else [8, 16, 32]):
+    # (bfloat16 pages of 1 and 4 tokens: the plain attention kernel on a bfloat16 cache)
+    for page in ([1, 4, 8, 16] if dtype == "float32" else [1, 4, 8, 16, 32]):
         runner = make_runner(folder, dtype, replay.peak_tokens(trace, page), page)
+        for g in runner.cache.groups:
+            g.storage.fill_(float("nan"))
         rows = replay.collect(trace, replay.run_trace(runner, trace), 256)
         replay.compare(rows, ref, TOL[dtype])
 
@@ -357,11 +382,12 @@ LLAMA_8B_LAYERS = dict(
 )
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_layers_of_the_8b_shape(dtype, tmp_path):
+@pytest.mark.parametrize("dtype,weight_copy", [("float32", "auto"), ("bfloat16", "auto"), ("bfloat16", "off")])
+def test_layers_of_the_8b_shape(dtype, weight_copy, tmp_path):
     """Two layers with every size of Llama-3.1-8B (width 4096, 32 heads over 8 groups of
     128, feed-forward 14336, vocabulary 128256, llama3 frequency scaling), weights
-    N(0, 0.02): the kernels at the sizes that the benchmark runs."""
+    N(0, 0.02): the kernels at the sizes that the benchmark runs; in bfloat16 with and
+    without the tiled copy of the matrices (without: the way of the 70B shape)."""
     cfg = LLAMA_8B_LAYERS
     weights = tiny.random_weights(cfg, seed=11, std=0.02)
     requests = {f"r{i}": tiny.random_tokens(cfg, n, 70 + i) for i, n in enumerate([70, 9, 200, 33])}
@@ -372,12 +398,66 @@ def test_layers_of_the_8b_shape(dtype, tmp_path):
     ref = {rid: plain_llama.forward(pc, pw, toks) for rid, toks in requests.items()}
     del pw
     runner = None
-    for make in (replay.tail_one_by_one, replay.portions, replay.mixed):
+    for make in (replay.whole, replay.tail_one_by_one, replay.portions, replay.mixed):
         trace = make(requests)
         del runner
-        runner = make_runner(folder, dtype, replay.peak_tokens(trace))
+        runner = make_runner(folder, dtype, replay.peak_tokens(trace), decode_weight_copy=weight_copy)
+        assert runner.model.build.tiled_weights == (dtype == "bfloat16" and weight_copy == "auto")
         rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
         replay.compare(rows, ref, TOL[dtype])
+
+
+def test_eight_layers_of_the_8b_shape_within_the_bounds_of_the_number_format():
+    """At depth the bfloat16 engine's distance from float32 arithmetic is measured against
+    that of the plain implementation rounding to bfloat16 at the same places, under all
+    four schedules; float32 against 1e-4.  ``tests/full_depth_equality.py`` states the
+    bounds and runs the same with all 32 layers."""
+    import full_depth_equality
+
+    lines, missed = full_depth_equality.run(8, [70, 9, 150, 33])
+    assert not missed, "\n".join(missed + lines)
+
+
+def test_the_pool_is_sized_from_free_memory(folders, monkeypatch):
+    """Without ``kv_cache_num_tokens`` the pool takes what the reference's formula gives
+    (src/halite/transformers/infer/engine/model_runner.py:117-131: free memory less the
+    share of the whole that ``memory_fraction_static`` keeps back, over the bytes of a
+    cached token), capped at what ``max_seqs_per_forward`` requests of the context length
+    could hold; and the engine generates with it."""
+    from halite_amd.engine.engine import InferenceEngine
+
+    folder, requests, ref = folders[("B", "bfloat16")]
+    cfg = tiny.TINY_B
+    per_token = 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * cfg["num_hidden_layers"] * 2  # keys and values, bf16
+    GiB = 1 << 30
+    total, fraction, page = 4 * GiB, 0.88, 16
+    free = int(total * (1 - fraction)) + 300_000  # what the formula leaves: 300,000 bytes
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (free, total))
+    server = ServerConfig(kv_cache_num_tokens=None, page_size=page, max_seqs_per_forward=64)
+    runner = ModelRunner.from_pretrained(folder, server, ModelConfig(dtype="bfloat16", memory_fraction_static=fraction))
+    usable = free - total * (1 - fraction)
+    reference_tokens = int(usable // per_token)
+    assert runner.cache.num_pages == int(usable // (per_token * page)) and runner.cache.num_pages > 40
+    # (a page number is reserved, and the pool holds whole pages)
+    assert reference_tokens - 2 * page < runner.cache.token_capacity <= reference_tokens
+    assert runner.cache.token_capacity == runner.max_total_tokens == (runner.cache.num_pages - 1) * page
+    engine = InferenceEngine(runner)
+    toks = requests["r1"]
+    out = engine.infer_batch([(0, toks[:30], {"max_new_tokens": 4, "temperature": 0.0})])[0].output_ids[0]
+    assert len(out) == 4
+    logits = plain_llama.forward(*plain_llama.read_model_folder(folder), toks[:30] + out)
+    for j, tok in enumerate(out):  # the plain implementation's best token, or within rounding of it
+        row = logits[29 + j]
+        assert float(row.max() - row[tok]) <= TOL["bfloat16"] * max(1.0, float(row.abs().max()))
+    # plenty of memory: the cap
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (3 * GiB, total))
+    capped = ModelRunner.from_pretrained(folder, ServerConfig(kv_cache_num_tokens=None, page_size=page, max_seqs_per_forward=8),
+                                         ModelConfig(dtype="bfloat16", memory_fraction_static=fraction))
+    assert capped.cache.num_pages == 8 * (cfg["max_position_embeddings"] // page) + 1
+    # none: an error that says so
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (int(total * (1 - fraction)), total))
+    with pytest.raises(RuntimeError, match="no device memory is left"):
+        ModelRunner.from_pretrained(folder, server, ModelConfig(dtype="bfloat16", memory_fraction_static=fraction))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

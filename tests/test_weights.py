@@ -163,7 +163,7 @@ def test_random_mode_writes_a_loadable_folder(tmp_path, raw):
         f.close()
 
 
-def _two_shards(folder, raw, w, drop_from_shard=None):
+def _two_shards(folder, raw, w, drop_from_shard=None, second_in=""):
     """The folder's tensors in two files and an index, as large models are stored."""
     from safetensors.torch import save_file as pkg_save
 
@@ -173,12 +173,14 @@ def _two_shards(folder, raw, w, drop_from_shard=None):
     names = list(w)
     first = {n: w[n].contiguous() for n in names[::2]}
     second = {n: w[n].contiguous() for n in names[1::2]}
+    second_name = os.path.join(second_in, "model-00002-of-00002.safetensors")  # (an index may name a subfolder)
+    os.makedirs(os.path.join(folder, second_in), exist_ok=True)
     index = {"metadata": {}, "weight_map": {**{n: "model-00001-of-00002.safetensors" for n in first},
-                                            **{n: "model-00002-of-00002.safetensors" for n in second}}}
+                                            **{n: second_name for n in second}}}
     if drop_from_shard is not None:
         first.pop(drop_from_shard, None), second.pop(drop_from_shard, None)
     pkg_save(first, os.path.join(folder, "model-00001-of-00002.safetensors"))
-    pkg_save(second, os.path.join(folder, "model-00002-of-00002.safetensors"))
+    pkg_save(second, os.path.join(folder, second_name))
     with open(os.path.join(folder, "model.safetensors.index.json"), "w") as f:
         json.dump(index, f)
 
@@ -221,3 +223,13 @@ def test_a_missing_shard_and_a_tensor_missing_from_its_shard_are_named(tmp_path)
     assert "the index lists model.layers.1.mlp.up_proj.weight in model-0000" in str(e.value)
     with pytest.raises(WeightError, match="no model.safetensors and no model.safetensors.index.json"):
         load_weights(model, arch.weight_map(cfg), str(tmp_path / "nothing"))
+    # a shard that the index names with a subfolder: found, and named so where it lacks a tensor
+    deep = str(tmp_path / "deep")
+    _two_shards(deep, raw, w, second_in="part2")
+    load_weights(model, arch.weight_map(cfg), deep)
+    assert torch.equal(model.head.weight, w["lm_head.weight"])
+    deep_lacks = str(tmp_path / "deep_lacks")
+    _two_shards(deep_lacks, raw, w, drop_from_shard=list(w)[1], second_in="part2")
+    with pytest.raises(WeightError) as e:
+        load_weights(model, arch.weight_map(cfg), deep_lacks)
+    assert f"the index lists {list(w)[1]} in part2/model-00002" in str(e.value)
