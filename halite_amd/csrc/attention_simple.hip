@@ -1,17 +1,22 @@
 // Paged attention, the plain way: float32 arithmetic on the vector units throughout, any
-// head size that is a multiple of 2 up to 512, any page size, any number of heads and
+// head size that is a multiple of 4 up to 512, any page size, any number of heads and
 // groups, float32 or bf16 storage.  It is the whole attention of the 32-bit path and the
 // fallback of the bf16 path for shapes that the matrix-core kernel refuses.
 //
-// A workgroup of up to four waves serves one (token, query head).  The row's keys, from the
-// start of its window to its own position, go in blocks of 64; wave w takes the blocks w,
-// w + waves, ... and keeps a running maximum, denominator and weighted sum of its own, and
-// at the end the waves' results are joined in wave order by the log-sum-exp rule.  A row's
-// result therefore depends on the row's own position and request alone, not on the batch.
-// Within a block a lane is a key for the scores (the block's keys lie in LDS, transposed on
-// the way in, so that global loads are contiguous and a lane walks its key's dimensions in
-// order) and a dimension for the weighted sum (the block's values in LDS likewise, a lane
-// walks the keys in order).
+// A workgroup of four waves serves up to 16 rows that share their keys: a few neighbouring
+// tokens of one request times the query heads of one key/value head, so the keys and values
+// are read once for all of them.  It walks the keys in blocks of 64 (32 for heads above
+// 256), always cut at multiples of the block size counted from the request's first key:
+// all threads bring a block's keys [key][D] and values [D][key] into LDS together (the next
+// block's loads are in flight while this one is worked on), then wave w takes the rows w,
+// w + 4, ...: a lane is a key for the scores and a dimension for the weighted sum.
+//
+// A row's keys are summed in pieces of 512: a piece starts from nothing, and the pieces'
+// sums are joined in the order of the keys by the log-sum-exp rule.  Where a step has few
+// rows (decoding) every piece is a workgroup of its own and a second kernel joins them;
+// where it has many, one workgroup walks all of a row's pieces and joins as it goes.  Both
+// do the same arithmetic in the same order, so a row's result depends on the row's own
+// position, window and request alone: not on the batch, and not on which way was taken.
 //
 // scores, mask, softmax and weighted sum as in
 // src/halite/transformers/attention.py:647-714; the causal rule for a portion that
@@ -20,238 +25,436 @@
 #include "hal_common.h"
 #include "hal_api.h"
 
-#define SIMPLE_MAX_ACC 8  // head sizes up to 64 * 8
-#define SIMPLE_MAX_WAVES 4
-
-// floats of LDS that one wave needs: a tile of 64 keys x D (rows padded by one) that holds
-// the keys and then the values of a block, and the block's 64 probabilities
-static inline size_t simple_wave_floats(int D) { return (size_t)HAL_WAVE * (D + 1) + D + HAL_WAVE; }
+#define PLAIN_THREADS 256
+#define PLAIN_WAVES 4
+#define PLAIN_PIECE 512     // keys of a piece
+#define PLAIN_MAX_ROWS 16   // rows of a workgroup, four to a wave at most
+#define PLAIN_PAD 4         // floats between two rows of a tile: 16-byte rows, no bank conflicts
 
 // LDS that one lane of a wave writes and another reads: the wave's LDS operations are done
 // in the order they were issued; this keeps the compiler from moving them across
-__device__ __forceinline__ void simple_wave_sync() {
+__device__ __forceinline__ void plain_wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// R: 64-wide pieces of a head (head sizes up to 64 * R)
-template <typename T, int R>
-__global__ void __launch_bounds__(SIMPLE_MAX_WAVES * HAL_WAVE)
-attention_simple_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__ out,
-                        int out_row_stride, const int* __restrict__ positions,
-                        const int* __restrict__ token_seg, const int* __restrict__ block_table,
-                        int bt_stride, const T* __restrict__ k_pages,
-                        const T* __restrict__ v_pages, int H, int K, int D, int page_size,
-                        int n_pages, float scale, int window) {
+// The join of two partial softmax sums, (M, L, A) with (m, l, a): one definition for the
+// kernel that walks and the kernel that merges, written without contraction so that both
+// compile to the same operations.
+__device__ __forceinline__ void plain_join_weights(float M, float m, float& M_new, float& w_old, float& w_new) {
+  M_new = fmaxf(M, m);
+  w_old = (M == -INFINITY) ? 0.f : expf(M - M_new);
+  w_new = (m == -INFINITY) ? 0.f : expf(m - M_new);
+}
+__device__ __forceinline__ float plain_join(float A, float w_old, float a, float w_new) {
+  return __fadd_rn(__fmul_rn(A, w_old), __fmul_rn(a, w_new));
+}
+
+static inline size_t plain_lds_floats(int D, int keys, int rows) {
+  return (size_t)keys * (D + PLAIN_PAD) + (size_t)D * (keys + PLAIN_PAD) + (size_t)rows * D +
+         (size_t)PLAIN_WAVES * keys + (size_t)2 * 2 * keys;  // tiles, rows, probabilities, places
+}
+
+// R: 64-wide pieces of a head (head sizes up to 64 * R); KEYS: keys of a block.
+// Grid: x = groups of `tq` tokens, y = key/value head times chunk of 16 heads of its group,
+// z = piece (split) or 1.
+template <typename T, int R, int KEYS>
+__global__ void __launch_bounds__(PLAIN_THREADS)
+attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__ out,
+                       int out_row_stride, const int* __restrict__ positions,
+                       const int* __restrict__ token_seg, const int* __restrict__ block_table,
+                       int bt_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+                       float* __restrict__ part, int n_tokens, int H, int K, int D, int page_size,
+                       int n_pages, float scale, int window, int tq, int chunks, int split,
+                       int max_pieces, int page_shift, int cw_shift) {
+  constexpr int NV = KEYS * R / 16;  // 16-byte vectors of a tile that a thread brings
+  constexpr int ROWS_MOST = R == 8 ? PLAIN_WAVES : PLAIN_MAX_ROWS;  // (the largest heads: a row a wave)
+  constexpr int RW = ROWS_MOST / PLAIN_WAVES;                       // rows of a wave
   extern __shared__ float smem[];
-  const int n_waves = blockDim.x / HAL_WAVE;
-  const int lane = threadIdx.x % HAL_WAVE;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / HAL_WAVE);
-  float* q_s = smem;  // [D], shared by the waves
-  float* mine = smem + D + (size_t)wave * ((size_t)HAL_WAVE * (D + 1) + D + HAL_WAVE);
-  float* tile = mine;                                  // keys [64][D + 1], then values [D][65]
-  float* p_s = mine + (size_t)HAL_WAVE * (D + 1) + D;  // [64]  (D * 65 <= 64 * (D + 1) + D)
+  const int tid = threadIdx.x;
+  const int lane = tid % HAL_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / HAL_WAVE);
+  const int KS = D + PLAIN_PAD, VS = KEYS + PLAIN_PAD;
+  float* k_tile = smem;                                // [KEYS][D + pad]
+  float* v_tile = k_tile + (size_t)KEYS * KS;           // [D][KEYS + pad]
+  float* q_rows = v_tile + (size_t)D * VS;              // [rows][D]
+  float* p_mine = q_rows + (size_t)ROWS_MOST * D + (size_t)wave * KEYS;  // [KEYS] per wave
+  int2* key_place = (int2*)(q_rows + (size_t)ROWS_MOST * D + (size_t)PLAIN_WAVES * KEYS);  // [2][KEYS]
 
-  const int t = blockIdx.x, h = blockIdx.y;
-  const int g = h / (H / K);
+  const int G = H / K;
+  const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+  const int heads_here = min(ROWS_MOST, G - chunk * ROWS_MOST);  // heads of this chunk
+  const int h_first = g * G + chunk * ROWS_MOST;
+  const int t_first = blockIdx.x * tq;
+  const int t_end = min(n_tokens, t_first + tq);
+  const int dv = D / 4;  // 16-byte vectors of a key's row
+
+  // the tokens of the group go in runs of one request; each run is a walk of its own
+  for (int ta = t_first; ta < t_end;) {
+    const int seg = token_seg[ta];
+    int tb = ta + 1;
+    while (tb < t_end && token_seg[tb] == seg) ++tb;
+    int p_max = -1, lo_min = 0x7fffffff;
+    for (int t = ta; t < tb; ++t) {
+      const int p = positions[t];
+      const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+      p_max = max(p_max, p);
+      lo_min = min(lo_min, lo);
+    }
+    const int* bt = block_table + (size_t)seg * bt_stride;
+    const int n_rows = (tb - ta) * heads_here;
+    // the keys this workgroup walks for the run
+    int j_begin = lo_min / KEYS * KEYS, j_end = p_max + 1;
+    if (split) {
+      j_begin = max(j_begin, (int)blockIdx.z * PLAIN_PIECE);
+      j_end = min(j_end, ((int)blockIdx.z + 1) * PLAIN_PIECE);
+    }
+    if (j_begin >= j_end) {  // (the same for every thread)
+      ta = tb;
+      continue;
+    }
+
+    __syncthreads();  // the walk before is done with the tiles and the rows
+    for (int e = tid; e < n_rows * dv; e += PLAIN_THREADS) {
+      const int r = e / dv, i = (e % dv) * 4;
+      const T* qp = q + (size_t)(ta + r / heads_here) * q_row_stride + (size_t)(h_first + r % heads_here) * D + i;
+      float v[4];
+      load4(qp, v);
+      store4(q_rows + (size_t)r * D + i, v);
+    }
+
+    // this wave's rows: r = wave + 4 * rr
+    int row_p[RW], row_lo[RW];
+    float M[RW], L[RW], A[RW][R];    // the pieces so far
+    float m[RW], l[RW], acc[RW][R];  // the piece at hand
+#pragma unroll
+    for (int rr = 0; rr < RW; ++rr) {
+      const int r = wave + PLAIN_WAVES * rr;
+      const int p = r < n_rows ? positions[ta + r / heads_here] : -1;
+      row_p[rr] = p;
+      row_lo[rr] = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+      M[rr] = m[rr] = -INFINITY;
+      L[rr] = l[rr] = 0.f;
+#pragma unroll
+      for (int c = 0; c < R; ++c) A[rr][c] = acc[rr][c] = 0.f;
+    }
+
+    // A block's keys and values on their way to LDS.  Where a key lies (its page's part for
+    // this key/value head, its slot) is looked up once per key, by the block's first threads,
+    // two blocks ahead, and left in LDS.  Keys outside [lo_min, p_max] are not read (their
+    // pages may not be held) and count as zero; a hole in the block table inside that range
+    // gives NaN keys, so that it shows.  Of the keys, thread `tid` brings vector c of the
+    // rows r0, r0 + rows_per_pass, ...; of the values, four keys of a dimension each time.
+    auto look_up = [&](int j0, int buf) {
+      if (tid < KEYS) {
+        const int j = j0 + tid;
+        int2 where = make_int2(-2, 0);  // not read
+        if (j >= lo_min && j <= p_max) {
+          const int pg = page_shift >= 0 ? j >> page_shift : j / page_size;
+          const int page = bt[pg];
+          where.y = j - pg * page_size;
+          where.x = (page >= 0 && page < n_pages) ? page * K + g : -1;  // -1: a hole
+        }
+        key_place[buf * KEYS + tid] = where;
+      }
+    };
+    float kreg[NV][4], vreg[NV][4];
+    const int kc = tid & ((1 << cw_shift) - 1), kr0 = tid >> cw_shift, rows_per_pass = PLAIN_THREADS >> cw_shift;
+    auto fetch = [&](int buf) {
+      const int2* place = key_place + buf * KEYS;
+#pragma unroll
+      for (int u = 0; u < NV; ++u) {
+        kreg[u][0] = kreg[u][1] = kreg[u][2] = kreg[u][3] = 0.f;
+        vreg[u][0] = vreg[u][1] = vreg[u][2] = vreg[u][3] = 0.f;
+        const int row = kr0 + u * rows_per_pass;
+        if (row < KEYS && kc < dv) {
+          const int2 w = place[row];
+          if (w.x >= 0) load4(k_pages + ((size_t)w.x * page_size + w.y) * D + kc * 4, kreg[u]);
+          else if (w.x == -1) kreg[u][0] = kreg[u][1] = kreg[u][2] = kreg[u][3] = __uint_as_float(0x7fc00000u);
+        }
+        const int e = tid + u * PLAIN_THREADS;
+        const int d = e / (KEYS / 4), jj = (e % (KEYS / 4)) * 4;
+        if (d < D) {
+          if (page_size % 4 == 0) {  // the four keys lie side by side in one page
+            const int2 w = place[jj];
+            if (w.x >= 0) {
+              load4(v_pages + ((size_t)w.x * D + d) * page_size + w.y, vreg[u]);
+              if (place[jj + 3].x < 0) {  // (some of the four are outside the range: their slots may hold anything)
+#pragma unroll
+                for (int x = 1; x < 4; ++x)
+                  if (place[jj + x].x < 0) vreg[u][x] = 0.f;
+              }
+            } else {  // the range may begin among the four
+#pragma unroll
+              for (int x = 1; x < 4; ++x) {
+                const int2 wx = place[jj + x];
+                if (wx.x >= 0) vreg[u][x] = to_f32(v_pages[((size_t)wx.x * D + d) * page_size + wx.y]);
+              }
+            }
+          } else {
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+              const int2 wx = place[jj + x];
+              if (wx.x >= 0) vreg[u][x] = to_f32(v_pages[((size_t)wx.x * D + d) * page_size + wx.y]);
+            }
+          }
+        }
+      }
+    };
+    auto commit = [&]() {
+#pragma unroll
+      for (int u = 0; u < NV; ++u) {
+        const int row = kr0 + u * rows_per_pass;
+        if (row < KEYS && kc < dv) store4(k_tile + (size_t)row * KS + kc * 4, kreg[u]);
+        const int e = tid + u * PLAIN_THREADS;
+        const int d = e / (KEYS / 4), jj = (e % (KEYS / 4)) * 4;
+        if (d < D) store4(v_tile + (size_t)d * VS + jj, vreg[u]);
+      }
+    };
+
+    look_up(j_begin, 0);
+    look_up(j_begin + KEYS, 1);
+    __syncthreads();
+    fetch(0);
+    int buf = 0;
+    for (int j0 = j_begin; j0 < j_end; j0 += KEYS, buf ^= 1) {
+      __syncthreads();  // every wave has read the block before
+      commit();
+      look_up(j0 + 2 * KEYS, buf);
+      if (j0 + KEYS < j_end) fetch(buf ^ 1);
+      __syncthreads();
+      const bool piece_ends = (j0 + KEYS) % PLAIN_PIECE == 0 || j0 + KEYS >= j_end;
+#pragma unroll
+      for (int rr = 0; rr < RW; ++rr) {
+        const int r = wave + PLAIN_WAVES * rr;
+        const bool have_row = r < n_rows;  // (the same for the whole wave)
+        const int p = row_p[rr], lo = row_lo[rr];
+        if (have_row && j0 <= p && j0 + KEYS > lo) {  // the block holds keys of this row
+          // ---- scores: a lane is a key ----
+          const int j = j0 + lane;
+          const bool valid = lane < KEYS && j >= lo && j <= p;
+          float s = -INFINITY;
+          if (lane < KEYS) {
+            const float* kr = k_tile + (size_t)lane * KS;
+            const float* qr = q_rows + (size_t)r * D;
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+            for (int i = 0; i < D; i += 4) {
+              const float4 kk = *(const float4*)(kr + i);
+              const float4 qq = *(const float4*)(qr + i);
+              d0 = fmaf(kk.x, qq.x, d0);
+              d1 = fmaf(kk.y, qq.y, d1);
+              d2 = fmaf(kk.z, qq.z, d2);
+              d3 = fmaf(kk.w, qq.w, d3);
+            }
+            if (valid) s = ((d0 + d1) + (d2 + d3)) * scale;
+          }
+          const float m_new = fmaxf(m[rr], wave_max(s));
+          // (a NaN score makes every sum NaN, as it must; m_new is -inf only if no key is valid)
+          const float alpha = (m[rr] == -INFINITY) ? 0.f : expf(m[rr] - m_new);
+          const float pj = valid ? expf(s - m_new) : 0.f;
+          l[rr] = l[rr] * alpha + wave_sum(pj);
+          m[rr] = m_new;
+          if (lane < KEYS) p_mine[lane] = pj;
+          plain_wave_sync();
+          // ---- weighted sum: a lane is a dimension ----
+#pragma unroll
+          for (int c = 0; c < R; ++c) {
+            const int d = lane + c * HAL_WAVE;
+            if (d < D) {
+              const float* vr = v_tile + (size_t)d * VS;
+              float t0 = 0.f, t1 = 0.f;
+#pragma unroll 4
+              for (int jj = 0; jj < KEYS; jj += 4) {
+                const float4 vv = *(const float4*)(vr + jj);
+                const float4 pp = *(const float4*)(p_mine + jj);
+                t0 = fmaf(pp.x, vv.x, t0);
+                t1 = fmaf(pp.y, vv.y, t1);
+                t0 = fmaf(pp.z, vv.z, t0);
+                t1 = fmaf(pp.w, vv.w, t1);
+              }
+              acc[rr][c] = __fadd_rn(__fmul_rn(acc[rr][c], alpha), __fadd_rn(t0, t1));
+            }
+          }
+          plain_wave_sync();  // before the next row's probabilities overwrite these
+        }
+        if (have_row && piece_ends) {
+          // Only pieces that hold keys of the row count (the others would join as nothing,
+          // but where pieces are workgroups of their own nobody computes them).
+          const int pc = j0 / PLAIN_PIECE;
+          const bool mine = pc >= lo / PLAIN_PIECE && pc <= p / PLAIN_PIECE;
+          const bool only_piece = lo / PLAIN_PIECE == p / PLAIN_PIECE;
+          if (mine && split && !only_piece) {
+            float* dst = part + (((size_t)(ta + r / heads_here) * H + h_first + r % heads_here) * max_pieces + pc) * (D + 2);
+#pragma unroll
+            for (int c = 0; c < R; ++c) {
+              const int d = lane + c * HAL_WAVE;
+              if (d < D) dst[d] = acc[rr][c];
+            }
+            if (lane == 0) {
+              dst[D] = m[rr];
+              dst[D + 1] = l[rr];
+            }
+          } else if (mine) {
+            float M_new, w_old, w_new;
+            plain_join_weights(M[rr], m[rr], M_new, w_old, w_new);
+            L[rr] = plain_join(L[rr], w_old, l[rr], w_new);
+            M[rr] = M_new;
+#pragma unroll
+            for (int c = 0; c < R; ++c) A[rr][c] = plain_join(A[rr][c], w_old, acc[rr][c], w_new);
+          }
+          m[rr] = -INFINITY;
+          l[rr] = 0.f;
+#pragma unroll
+          for (int c = 0; c < R; ++c) acc[rr][c] = 0.f;
+        }
+      }
+    }
+
+    // rows whose pieces were all joined here are done
+#pragma unroll
+    for (int rr = 0; rr < RW; ++rr) {
+      const int r = wave + PLAIN_WAVES * rr;
+      const int p = row_p[rr], lo = row_lo[rr];
+      const bool only_piece = lo / PLAIN_PIECE == p / PLAIN_PIECE;
+      if (r >= n_rows || (split && !(only_piece && (int)blockIdx.z == p / PLAIN_PIECE))) continue;
+      T* op = out + (size_t)(ta + r / heads_here) * out_row_stride + (size_t)(h_first + r % heads_here) * D;
+      const float inv = 1.0f / L[rr];
+#pragma unroll
+      for (int c = 0; c < R; ++c) {
+        const int d = lane + c * HAL_WAVE;
+        if (d < D) op[d] = from_f32<T>(__fmul_rn(A[rr][c], inv));
+      }
+    }
+    ta = tb;
+  }
+}
+
+// The pieces of a row, joined in the order of the keys: one wave per (token, head) whose
+// keys lie in more than one piece.
+template <typename T, int R>
+__global__ void __launch_bounds__(HAL_WAVE)
+attention_plain_merge_kernel(T* __restrict__ out, int out_row_stride, const int* __restrict__ positions,
+                             const float* __restrict__ part, int H, int D, int window, int max_pieces) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int p = positions[t];
-  const int seg = token_seg[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-  const int* bt = block_table + (size_t)seg * bt_stride;
-
-  const T* qp = q + (size_t)t * q_row_stride + (size_t)h * D;
-  for (int i = threadIdx.x; i < D; i += blockDim.x) q_s[i] = to_f32(qp[i]);
-  __syncthreads();
-
-  float m = -INFINITY, l = 0.f;
-  float acc[R];
+  const int first = lo / PLAIN_PIECE, last = p / PLAIN_PIECE;
+  if (first == last) return;  // written by the piece's own workgroup
+  float M = -INFINITY, L = 0.f, A[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) acc[r] = 0.f;
-
-  for (int j0 = lo + wave * HAL_WAVE; j0 <= p; j0 += n_waves * HAL_WAVE) {
-    const int j = j0 + lane;
-    const bool valid = j <= p;
-    const int n_valid = (p - j0 + 1) < HAL_WAVE ? (p - j0 + 1) : HAL_WAVE;
-    // this lane's key: where it lies (a hole in the block table must show)
-    long long base = -1;
-    int off = 0;
-    if (valid) {
-      const long long page = bt[j / page_size];
-      off = j % page_size;
-      if (page >= 0 && page < n_pages) base = page * K + g;
-    }
-    // the block's keys into LDS, the lanes along the dimensions; eight keys' loads are
-    // issued before the first is stored, so that the trips to memory overlap
-    constexpr int KEYS_AT_ONCE = R <= 2 ? 16 : (R <= 4 ? 8 : 4);
-    for (int jj0 = 0; jj0 < n_valid; jj0 += KEYS_AT_ONCE) {
-      float kv[KEYS_AT_ONCE][R];
+  for (int c = 0; c < R; ++c) A[c] = 0.f;
+  for (int pc = first; pc <= last; ++pc) {
+    const float* src = part + (((size_t)t * H + h) * max_pieces + pc) * (D + 2);
+    float M_new, w_old, w_new;
+    plain_join_weights(M, src[D], M_new, w_old, w_new);
+    L = plain_join(L, w_old, src[D + 1], w_new);
+    M = M_new;
 #pragma unroll
-      for (int u = 0; u < KEYS_AT_ONCE; ++u) {
-        const int jj = jj0 + u < n_valid ? jj0 + u : n_valid - 1;
-        const int b_lo = __builtin_amdgcn_readlane((int)(base & 0xffffffffll), jj);
-        const int b_hi = __builtin_amdgcn_readlane((int)(base >> 32), jj);
-        const long long b = ((long long)b_hi << 32) | (unsigned int)b_lo;
-        const int o = __builtin_amdgcn_readlane(off, jj);
-        const T* kp = k_pages + ((size_t)(b < 0 ? 0 : b) * page_size + o) * D;  // (a hole: any row)
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const int i = lane + r * HAL_WAVE;
-          kv[u][r] = i < D ? to_f32(kp[i]) : 0.f;
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < KEYS_AT_ONCE; ++u) {
-        if (jj0 + u >= n_valid) break;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const int i = lane + r * HAL_WAVE;
-          if (i < D) tile[(size_t)(jj0 + u) * (D + 1) + i] = kv[u][r];
-        }
-      }
-    }
-    simple_wave_sync();  // the rows are written by other lanes than the one that reads them
-    float s = -INFINITY;
-    if (valid) {
-      if (base >= 0) {
-        const float* kr = tile + (size_t)lane * (D + 1);
-        float dot = 0.f;
-        for (int i = 0; i < D; ++i) dot += q_s[i] * kr[i];
-        s = dot * scale;
-      } else {
-        s = __uint_as_float(0x7fc00000u);
-      }
-    }
-    const float m_tile = wave_max(s);
-    const float m_new = fmaxf(m, m_tile);
-    const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
-    const float pj = valid ? expf(s - m_new) : 0.f;
-    l = l * alpha + wave_sum(pj);
-    m = m_new;
-    simple_wave_sync();  // every lane has read its key's row
-    p_s[lane] = pj;
-    // the block's values into the same tile, [dimension][key], the lanes along the keys
-    // (every lane has read its key's row by now: a wave runs in step)
-    {
-      const bool have = valid && base >= 0;
-      const T* vp = v_pages + (size_t)(have ? base : 0) * D * page_size + off;
-      for (int i0 = 0; i0 < D; i0 += 32) {  // 32 dimensions' loads at a time
-        float vv[32];
-#pragma unroll
-        for (int u = 0; u < 32; ++u) {
-          const int i = i0 + u < D ? i0 + u : D - 1;
-          vv[u] = to_f32(vp[(size_t)i * page_size]);
-        }
-#pragma unroll
-        for (int u = 0; u < 32; ++u)
-          if (i0 + u < D) tile[(size_t)(i0 + u) * (HAL_WAVE + 1) + lane] = have ? vv[u] : 0.f;
-      }
-    }
-    simple_wave_sync();
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int i = lane + r * HAL_WAVE;
-      if (i < D) {
-        const float* vr = tile + (size_t)i * (HAL_WAVE + 1);
-        float a = acc[r] * alpha;
-        for (int jj = 0; jj < n_valid; ++jj) a += p_s[jj] * vr[jj];
-        acc[r] = a;
-      }
-    }
-    simple_wave_sync();  // before the next block's keys overwrite the tile
-  }
-
-  // join the waves' results in wave order: every wave leaves (m, l, sums) in its own LDS,
-  // the first wave adds them up
-  __syncthreads();
-  if (lane == 0) {
-    p_s[0] = m;
-    p_s[1] = l;
-  }
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int i = lane + r * HAL_WAVE;
-    if (i < D) tile[i] = acc[r];
-  }
-  __syncthreads();
-  if (wave != 0) return;
-  const size_t per_wave = (size_t)HAL_WAVE * (D + 1) + D + HAL_WAVE;
-  float m_all = -INFINITY;
-  for (int w = 0; w < n_waves; ++w) m_all = fmaxf(m_all, smem[D + w * per_wave + (size_t)HAL_WAVE * (D + 1) + D]);
-  float l_all = 0.f;
-  float tot[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) tot[r] = 0.f;
-  for (int w = 0; w < n_waves; ++w) {
-    const float* theirs = smem + D + w * per_wave;
-    const float mw = theirs[(size_t)HAL_WAVE * (D + 1) + D], lw = theirs[(size_t)HAL_WAVE * (D + 1) + D + 1];
-    const float wgt = mw == -INFINITY ? 0.f : expf(mw - m_all);
-    l_all += wgt * lw;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int i = lane + r * HAL_WAVE;
-      if (i < D) tot[r] += wgt * theirs[i];
+    for (int c = 0; c < R; ++c) {
+      const int d = lane + c * HAL_WAVE;
+      if (d < D) A[c] = plain_join(A[c], w_old, src[d], w_new);
     }
   }
   T* op = out + (size_t)t * out_row_stride + (size_t)h * D;
-  const float inv = 1.0f / l_all;
+  const float inv = 1.0f / L;
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int i = lane + r * HAL_WAVE;
-    if (i < D) op[i] = from_f32<T>(tot[r] * inv);
+  for (int c = 0; c < R; ++c) {
+    const int d = lane + c * HAL_WAVE;
+    if (d < D) op[d] = from_f32<T>(__fmul_rn(A[c], inv));
   }
+}
+
+// How `hal_attention_simple` cuts a step of `n_tokens` tokens whose longest key range is
+// `max_kv_len`: tokens per workgroup, whether pieces are workgroups of their own, the
+// pieces' number and the floats of partial sums that the caller must bring then.
+extern "C" int hal_attention_simple_plan(int n_tokens, int H, int K, int D, int max_kv_len, int* tq,
+                                         int* split, int* max_pieces, long long* part_floats) {
+  HAL_REQUIRE(n_tokens >= 0 && H > 0 && K > 0 && D > 0 && H % K == 0 && max_kv_len >= 0,
+              "hal_attention_simple_plan: bad sizes T=%d H=%d K=%d D=%d keys=%d", n_tokens, H, K, D, max_kv_len);
+  const int G = H / K;
+  const int rows_most = D > 256 ? PLAIN_WAVES : PLAIN_MAX_ROWS;
+  const int chunks = (G + rows_most - 1) / rows_most;
+  int together = G >= rows_most ? 1 : rows_most / G;  // tokens whose rows fill a workgroup
+  const long long groups = ((long long)n_tokens + together - 1) / together * K * chunks;
+  const int pieces = max(1, (max_kv_len + PLAIN_PIECE - 1) / PLAIN_PIECE);
+  // few workgroups: a token each, and a piece each
+  *split = (groups < 512 && pieces > 1) ? 1 : 0;
+  *tq = *split ? 1 : together;
+  *max_pieces = pieces;
+  *part_floats = *split ? (long long)n_tokens * H * pieces * (D + 2) : 0;
+  return 0;
 }
 
 extern "C" int hal_attention_simple(const void* q, int q_row_stride, void* out,
                                     int out_row_stride, int dtype, const int* positions,
                                     const int* token_seg, const int* block_table, int bt_stride,
-                                    const void* k_pages, const void* v_pages, int n_tokens, int H,
-                                    int K, int D, int page_size, int n_pages, float scale,
-                                    int window, hipStream_t stream) {
+                                    const void* k_pages, const void* v_pages, float* part,
+                                    int n_tokens, int H, int K, int D, int page_size, int n_pages,
+                                    float scale, int window, int max_kv_len, hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && H > 0 && K > 0 && D > 0 && page_size > 0 && n_pages > 0,
               "hal_attention_simple: bad sizes T=%d H=%d K=%d D=%d page=%d pages=%d", n_tokens, H,
               K, D, page_size, n_pages);
   HAL_REQUIRE(H % K == 0, "hal_attention_simple: %d query heads are not a multiple of %d kv heads",
               H, K);
-  HAL_REQUIRE(D <= HAL_WAVE * SIMPLE_MAX_ACC, "hal_attention_simple: head size %d > %d", D,
-              HAL_WAVE * SIMPLE_MAX_ACC);
-  HAL_REQUIRE(H <= 65535, "hal_attention_simple: %d heads exceed the grid limit", H);
-  HAL_REQUIRE(window >= 0, "hal_attention_simple: window %d", window);
+  HAL_REQUIRE(D % 4 == 0 && D <= 512, "hal_attention_simple: head size %d is not a multiple of 4 up to 512", D);
+  HAL_REQUIRE(window >= 0 && max_kv_len >= 0, "hal_attention_simple: window %d, keys %d", window, max_kv_len);
+  HAL_REQUIRE(q_row_stride % 4 == 0 && out_row_stride % 4 == 0,
+              "hal_attention_simple: rows of %d and %d elements are not multiples of 4", q_row_stride, out_row_stride);
   if (n_tokens == 0) return 0;
-  // as many waves as fit the LDS of a CU with their tiles, four at most
-  int waves = SIMPLE_MAX_WAVES;
-  while (waves > 1 && ((size_t)D + waves * simple_wave_floats(D)) * sizeof(float) > 150 * 1024) waves /= 2;
-  const size_t smem = ((size_t)D + waves * simple_wave_floats(D)) * sizeof(float);
+  int tq, split, max_pieces;
+  long long part_floats;
+  if (hal_attention_simple_plan(n_tokens, H, K, D, max_kv_len, &tq, &split, &max_pieces, &part_floats)) return 1;
+  HAL_REQUIRE(!split || part != nullptr, "hal_attention_simple: %lld floats of partial sums are needed", part_floats);
+  const int G = H / K;
+  const int rows_most = D > 256 ? PLAIN_WAVES : PLAIN_MAX_ROWS;
+  const int chunks = (G + rows_most - 1) / rows_most;
+  const int keys = D > 256 ? 32 : 64;
+  const size_t smem = plain_lds_floats(D, keys, rows_most) * sizeof(float);
   HAL_REQUIRE(smem <= 160 * 1024, "hal_attention_simple: head size %d needs %zu bytes of LDS", D, smem);
-  dim3 grid(n_tokens, H);
-#define SIMPLE_LAUNCH(T_, R_)                                                                        \
+  const long long gy = (long long)K * chunks;
+  HAL_REQUIRE(gy <= 65535 && max_pieces <= 65535, "hal_attention_simple: %lld head chunks or %d pieces exceed the grid limit", gy, max_pieces);
+  int page_shift = -1;  // pages of a power of two need no division
+  for (int b = 0; b < 31; ++b)
+    if (page_size == (1 << b)) page_shift = b;
+  int cw_shift = 0;  // a key's row of D / 4 vectors goes to the next power of two of threads
+  while ((1 << cw_shift) < D / 4) ++cw_shift;
+  HAL_REQUIRE((long long)n_pages * K < (1ll << 31), "hal_attention_simple: %d pages of %d heads exceed the index range", n_pages, K);
+  dim3 grid((n_tokens + tq - 1) / tq, (unsigned)gy, split ? max_pieces : 1);
+  dim3 merge_grid(n_tokens, H);
+#define PLAIN_LAUNCH(T_, R_, KEYS_)                                                                  \
   do {                                                                                              \
     static bool raised = false; /* more than 64 KB of LDS has to be asked for, once per kernel */    \
     if (!raised) {                                                                                  \
-      HAL_CHECK_HIP(hipFuncSetAttribute((const void*)attention_simple_kernel<T_, R_>,               \
+      HAL_CHECK_HIP(hipFuncSetAttribute((const void*)attention_plain_kernel<T_, R_, KEYS_>,         \
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));   \
       raised = true;                                                                                \
     }                                                                                               \
-    hipLaunchKernelGGL((attention_simple_kernel<T_, R_>), grid, dim3(waves * HAL_WAVE), smem, stream, \
-                       (const T_*)q, q_row_stride, (T_*)out, out_row_stride, positions, token_seg,  \
-                       block_table, bt_stride, (const T_*)k_pages, (const T_*)v_pages, H, K, D,      \
-                       page_size, n_pages, scale, window);                                          \
+    hipLaunchKernelGGL((attention_plain_kernel<T_, R_, KEYS_>), grid, dim3(PLAIN_THREADS), smem,     \
+                       stream, (const T_*)q, q_row_stride, (T_*)out, out_row_stride, positions,      \
+                       token_seg, block_table, bt_stride, (const T_*)k_pages, (const T_*)v_pages,    \
+                       part, n_tokens, H, K, D, page_size, n_pages, scale, window, tq, chunks,       \
+                       split, max_pieces, page_shift, cw_shift);                                     \
+    if (split)                                                                                      \
+      hipLaunchKernelGGL((attention_plain_merge_kernel<T_, R_>), merge_grid, dim3(HAL_WAVE), 0,      \
+                         stream, (T_*)out, out_row_stride, positions, part, H, D, window,            \
+                         max_pieces);                                                                \
   } while (0)
-#define SIMPLE_BY_SIZE(T_)                   \
-  do {                                       \
-    if (D <= 64) SIMPLE_LAUNCH(T_, 1);       \
-    else if (D <= 128) SIMPLE_LAUNCH(T_, 2); \
-    else if (D <= 256) SIMPLE_LAUNCH(T_, 4); \
-    else SIMPLE_LAUNCH(T_, 8);               \
+#define PLAIN_BY_SIZE(T_)                       \
+  do {                                          \
+    if (D <= 64) PLAIN_LAUNCH(T_, 1, 64);       \
+    else if (D <= 128) PLAIN_LAUNCH(T_, 2, 64); \
+    else if (D <= 256) PLAIN_LAUNCH(T_, 4, 64); \
+    else PLAIN_LAUNCH(T_, 8, 32);               \
   } while (0)
   if (dtype == HAL_F32)
-    SIMPLE_BY_SIZE(float);
+    PLAIN_BY_SIZE(float);
   else if (dtype == HAL_BF16)
-    SIMPLE_BY_SIZE(bf16_t);
+    PLAIN_BY_SIZE(bf16_t);
   else
     return hal_fail("hal_attention_simple: unknown dtype %d", dtype);
-#undef SIMPLE_BY_SIZE
-#undef SIMPLE_LAUNCH
+#undef PLAIN_BY_SIZE
+#undef PLAIN_LAUNCH
   HAL_LAUNCH_CHECK();
   return 0;
 }

@@ -326,9 +326,12 @@ def attention_simple(
     n_heads: int,
     scale: float,
     window: int = 0,
+    max_kv_len: int | None = None,
 ):
-    """Paged attention, one wavefront per (token, head); ``q`` holds the query
-    heads at the start of rows of ``q_row_stride`` elements."""
+    """Paged attention in float32 arithmetic; ``q`` holds the query heads at the start of
+    rows of ``q_row_stride`` elements.  ``max_kv_len``: the most keys that a request of the
+    step has (what the block table could hold if it is not given); it decides how the step
+    is cut into workgroups, never a result."""
     lib = library.core_library()
     _dev(q, positions, token_seg, block_table, k_pages, v_pages)
     _i32(positions, "positions"), _i32(token_seg, "token_seg"), _i32(block_table, "block_table")
@@ -338,13 +341,19 @@ def attention_simple(
     _need(k_pages.dtype == q.dtype and v_pages.dtype == q.dtype, "attention: cache dtype")
     _need(q.numel() >= n * q_row_stride and q_row_stride >= n_heads * head_dim, "attention: q rows")
     out = torch.empty((n, n_heads * head_dim), dtype=q.dtype, device=q.device)
+    if max_kv_len is None:
+        max_kv_len = block_table.shape[1] * page_size
+    tq, split, pieces, floats = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_longlong()
+    _check(lib, lib.hal_attention_simple_plan(n, n_heads, n_kv, head_dim, max_kv_len, ctypes.byref(tq),
+                                              ctypes.byref(split), ctypes.byref(pieces), ctypes.byref(floats)))
+    part = torch.empty(floats.value, dtype=torch.float32, device=q.device) if floats.value else None
     _check(
         lib,
         lib.hal_attention_simple(
             _ptr(q), q_row_stride, _ptr(out), n_heads * head_dim, dtype_code(q.dtype),
             _ptr(positions), _ptr(token_seg), _ptr(block_table), block_table.shape[1],
-            _ptr(k_pages), _ptr(v_pages), n, n_heads, n_kv, head_dim, page_size, n_pages,
-            ctypes.c_float(scale), window, _stream(),
+            _ptr(k_pages), _ptr(v_pages), _ptr(part), n, n_heads, n_kv, head_dim, page_size, n_pages,
+            ctypes.c_float(scale), window, max_kv_len, _stream(),
         ),
     )
     return out
