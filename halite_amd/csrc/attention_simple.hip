@@ -15,8 +15,11 @@
 // sums are joined in the order of the keys by the log-sum-exp rule.  Where a step has few
 // rows (decoding) every piece is a workgroup of its own and a second kernel joins them;
 // where it has many, one workgroup walks all of a row's pieces and joins as it goes.  Both
-// do the same arithmetic in the same order, so a row's result depends on the row's own
-// position, window and request alone: not on the batch, and not on which way was taken.
+// do the same arithmetic in the same order, and every sum over keys is cut at fixed
+// multiples counted from the request's first key, so a row's result depends on the row's
+// own position, window and request alone, not on what else the step holds.  (The kernel
+// has two builds, blocks of 32 keys for steps of few tokens and of 64 for the others: the
+// same row differs between them by rounding.)
 //
 // scores, mask, softmax and weighted sum as in
 // src/halite/transformers/attention.py:647-714; the causal rule for a portion that
@@ -28,7 +31,6 @@
 #define PLAIN_THREADS 256
 #define PLAIN_WAVES 4
 #define PLAIN_PIECE 512     // keys of a piece
-#define PLAIN_MAX_ROWS 16   // rows of a workgroup, four to a wave at most
 #define PLAIN_PAD 4         // floats between two rows of a tile: 16-byte rows, no bank conflicts
 
 // LDS that one lane of a wave writes and another reads: the wave's LDS operations are done
@@ -37,6 +39,44 @@ __device__ __forceinline__ void plain_wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Maximum and sum over the wave on the vector unit itself (data-parallel moves within a row
+// of 16 lanes, then the swaps of register halves between rows): a shuffle would be a trip
+// through the LDS hardware each, six in a row that the wave waits for.
+template <int CTRL>
+__device__ __forceinline__ float plain_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ void plain_swap_16(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void plain_swap_32(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float plain_wave_max(float v) {
+  v = fmaxf(v, plain_dpp<0xB1>(v));   // lanes 1 apart (quad_perm 1,0,3,2)
+  v = fmaxf(v, plain_dpp<0x4E>(v));   // 2 apart (quad_perm 2,3,0,1)
+  v = fmaxf(v, plain_dpp<0x141>(v));  // the mirrored half row
+  v = fmaxf(v, plain_dpp<0x140>(v));  // the mirrored row
+  float a = v, b = v;
+  plain_swap_16(a, b);
+  v = fmaxf(a, b);
+  a = b = v;
+  plain_swap_32(a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float plain_wave_sum(float v) {
+  v += plain_dpp<0xB1>(v);
+  v += plain_dpp<0x4E>(v);
+  v += plain_dpp<0x141>(v);
+  v += plain_dpp<0x140>(v);
+  float a = v, b = v;
+  plain_swap_16(a, b);
+  v = a + b;
+  a = b = v;
+  plain_swap_32(a, b);
+  return a + b;
 }
 
 // The join of two partial softmax sums, (M, L, A) with (m, l, a): one definition for the
@@ -56,11 +96,16 @@ static inline size_t plain_lds_floats(int D, int keys, int rows) {
          (size_t)PLAIN_WAVES * keys + (size_t)2 * 2 * keys;  // tiles, rows, probabilities, places
 }
 
-// R: 64-wide pieces of a head (head sizes up to 64 * R); KEYS: keys of a block.
-// Grid: x = groups of `tq` tokens, y = key/value head times chunk of 16 heads of its group,
-// z = piece (split) or 1.
-template <typename T, int R, int KEYS>
-__global__ void __launch_bounds__(PLAIN_THREADS)
+// R: 64-wide pieces of a head (head sizes up to 64 * R); KEYS: keys of a block; RW: rows of
+// a wave (a workgroup has 4 RW rows at most).  Steps of few tokens run RW = 1 with blocks of
+// 32 keys (less LDS and fewer registers, so four workgroups share a compute unit and one's
+// loads fly while the others compute), the others RW = 4 with blocks of 64.
+// Grid: x = groups of `tq` tokens, y = key/value head times chunk of 4 RW heads of its
+// group, z = piece (split) or 1.
+// (the build for few tokens is held to the registers that let four workgroups share a
+// compute unit, where its LDS allows as many)
+template <typename T, int R, int KEYS, int RW>
+__global__ void __launch_bounds__(PLAIN_THREADS, (RW == 1 && R <= 2) ? 4 : 1)
 attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__ out,
                        int out_row_stride, const int* __restrict__ positions,
                        const int* __restrict__ token_seg, const int* __restrict__ block_table,
@@ -69,8 +114,7 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
                        int n_pages, float scale, int window, int tq, int chunks, int split,
                        int max_pieces, int page_shift, int cw_shift) {
   constexpr int NV = KEYS * R / 16;  // 16-byte vectors of a tile that a thread brings
-  constexpr int ROWS_MOST = R == 8 ? PLAIN_WAVES : PLAIN_MAX_ROWS;  // (the largest heads: a row a wave)
-  constexpr int RW = ROWS_MOST / PLAIN_WAVES;                       // rows of a wave
+  constexpr int ROWS_MOST = RW * PLAIN_WAVES;
   extern __shared__ float smem[];
   const int tid = threadIdx.x;
   const int lane = tid % HAL_WAVE;
@@ -146,15 +190,26 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
     // pages may not be held) and count as zero; a hole in the block table inside that range
     // gives NaN keys, so that it shows.  Of the keys, thread `tid` brings vector c of the
     // rows r0, r0 + rows_per_pass, ...; of the values, four keys of a dimension each time.
-    auto look_up = [&](int j0, int buf) {
+    // (the entry of the block table is asked for in one step of the walk and put down in
+    // the next, when the wave waits for its loads anyway)
+    int asked_page = 0, asked_slot = -1;
+    auto ask_place = [&](int j0) {
+      asked_slot = -1;
       if (tid < KEYS) {
         const int j = j0 + tid;
-        int2 where = make_int2(-2, 0);  // not read
         if (j >= lo_min && j <= p_max) {
           const int pg = page_shift >= 0 ? j >> page_shift : j / page_size;
-          const int page = bt[pg];
-          where.y = j - pg * page_size;
-          where.x = (page >= 0 && page < n_pages) ? page * K + g : -1;  // -1: a hole
+          asked_page = bt[pg];
+          asked_slot = j - pg * page_size;
+        }
+      }
+    };
+    auto put_place = [&](int buf) {
+      if (tid < KEYS) {
+        int2 where = make_int2(-2, 0);  // not read
+        if (asked_slot >= 0) {
+          where.y = asked_slot;
+          where.x = (asked_page >= 0 && asked_page < n_pages) ? asked_page * K + g : -1;  // -1: a hole
         }
         key_place[buf * KEYS + tid] = where;
       }
@@ -213,16 +268,20 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
       }
     };
 
-    look_up(j_begin, 0);
-    look_up(j_begin + KEYS, 1);
+    ask_place(j_begin);
+    put_place(0);
+    ask_place(j_begin + KEYS);
+    put_place(1);
     __syncthreads();
     fetch(0);
+    ask_place(j_begin + 2 * KEYS);
     int buf = 0;
     for (int j0 = j_begin; j0 < j_end; j0 += KEYS, buf ^= 1) {
       __syncthreads();  // every wave has read the block before
       commit();
-      look_up(j0 + 2 * KEYS, buf);
+      put_place(buf);  // of the block after the next
       if (j0 + KEYS < j_end) fetch(buf ^ 1);
+      ask_place(j0 + 3 * KEYS);
       __syncthreads();
       const bool piece_ends = (j0 + KEYS) % PLAIN_PIECE == 0 || j0 + KEYS >= j_end;
 #pragma unroll
@@ -231,15 +290,20 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
         const bool have_row = r < n_rows;  // (the same for the whole wave)
         const int p = row_p[rr], lo = row_lo[rr];
         if (have_row && j0 <= p && j0 + KEYS > lo) {  // the block holds keys of this row
-          // ---- scores: a lane is a key ----
-          const int j = j0 + lane;
-          const bool valid = lane < KEYS && j >= lo && j <= p;
+          // ---- scores: a lane is a key (blocks of 32: the two halves of the wave take a
+          // half of the dimensions each, where that is a whole number of vectors) ----
+          const int key_lane = lane % KEYS;
+          const int j = j0 + key_lane;
+          const bool valid = j >= lo && j <= p;
           float s = -INFINITY;
-          if (lane < KEYS) {
-            const float* kr = k_tile + (size_t)lane * KS;
-            const float* qr = q_rows + (size_t)r * D;
+          {
+            const bool halves = KEYS == 32 && D % 8 == 0;  // (the same for every lane)
+            const int n = halves ? D / 2 : D, from = halves ? (lane / 32) * (D / 2) : 0;
+            const float* kr = k_tile + (size_t)key_lane * KS + from;
+            const float* qr = q_rows + (size_t)r * D + from;
             float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
-            for (int i = 0; i < D; i += 4) {
+#pragma unroll 4
+            for (int i = 0; i < n; i += 4) {
               const float4 kk = *(const float4*)(kr + i);
               const float4 qq = *(const float4*)(qr + i);
               d0 = fmaf(kk.x, qq.x, d0);
@@ -247,13 +311,20 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
               d2 = fmaf(kk.z, qq.z, d2);
               d3 = fmaf(kk.w, qq.w, d3);
             }
-            if (valid) s = ((d0 + d1) + (d2 + d3)) * scale;
+            float dot = (d0 + d1) + (d2 + d3);
+            if constexpr (KEYS == 32) {
+              if (!halves && lane >= 32) dot = 0.f;  // (the upper half did the lower half's work again)
+              float other = dot;
+              plain_swap_32(dot, other);  // (one of the two is this lane's, the other its partner's)
+              dot = dot + other;
+            }
+            if (valid) s = dot * scale;
           }
-          const float m_new = fmaxf(m[rr], wave_max(s));
+          const float m_new = fmaxf(m[rr], plain_wave_max(s));
           // (a NaN score makes every sum NaN, as it must; m_new is -inf only if no key is valid)
           const float alpha = (m[rr] == -INFINITY) ? 0.f : expf(m[rr] - m_new);
-          const float pj = valid ? expf(s - m_new) : 0.f;
-          l[rr] = l[rr] * alpha + wave_sum(pj);
+          const float pj = (valid && lane < KEYS) ? expf(s - m_new) : 0.f;  // (a key counts once)
+          l[rr] = l[rr] * alpha + plain_wave_sum(pj);
           m[rr] = m_new;
           if (lane < KEYS) p_mine[lane] = pj;
           plain_wave_sync();
@@ -369,11 +440,12 @@ attention_plain_merge_kernel(T* __restrict__ out, int out_row_stride, const int*
 // `max_kv_len`: tokens per workgroup, whether pieces are workgroups of their own, the
 // pieces' number and the floats of partial sums that the caller must bring then.
 extern "C" int hal_attention_simple_plan(int n_tokens, int H, int K, int D, int max_kv_len, int* tq,
-                                         int* split, int* max_pieces, long long* part_floats) {
+                                         int* split, int* rows_per_wave, int* max_pieces,
+                                         long long* part_floats) {
   HAL_REQUIRE(n_tokens >= 0 && H > 0 && K > 0 && D > 0 && H % K == 0 && max_kv_len >= 0,
               "hal_attention_simple_plan: bad sizes T=%d H=%d K=%d D=%d keys=%d", n_tokens, H, K, D, max_kv_len);
   const int G = H / K;
-  const int rows_most = D > 256 ? PLAIN_WAVES : PLAIN_MAX_ROWS;
+  const int rows_most = D > 256 ? PLAIN_WAVES : 4 * PLAIN_WAVES;
   const int chunks = (G + rows_most - 1) / rows_most;
   int together = G >= rows_most ? 1 : rows_most / G;  // tokens whose rows fill a workgroup
   const long long groups = ((long long)n_tokens + together - 1) / together * K * chunks;
@@ -381,6 +453,8 @@ extern "C" int hal_attention_simple_plan(int n_tokens, int H, int K, int D, int 
   // few workgroups: a token each, and a piece each
   *split = (groups < 512 && pieces > 1) ? 1 : 0;
   *tq = *split ? 1 : together;
+  // a token whose heads are at most four: a row a wave
+  *rows_per_wave = (*tq == 1 && G <= PLAIN_WAVES) || D > 256 ? 1 : 4;
   *max_pieces = pieces;
   *part_floats = *split ? (long long)n_tokens * H * pieces * (D + 2) : 0;
   return 0;
@@ -402,14 +476,14 @@ extern "C" int hal_attention_simple(const void* q, int q_row_stride, void* out,
   HAL_REQUIRE(q_row_stride % 4 == 0 && out_row_stride % 4 == 0,
               "hal_attention_simple: rows of %d and %d elements are not multiples of 4", q_row_stride, out_row_stride);
   if (n_tokens == 0) return 0;
-  int tq, split, max_pieces;
+  int tq, split, rw, max_pieces;
   long long part_floats;
-  if (hal_attention_simple_plan(n_tokens, H, K, D, max_kv_len, &tq, &split, &max_pieces, &part_floats)) return 1;
+  if (hal_attention_simple_plan(n_tokens, H, K, D, max_kv_len, &tq, &split, &rw, &max_pieces, &part_floats)) return 1;
   HAL_REQUIRE(!split || part != nullptr, "hal_attention_simple: %lld floats of partial sums are needed", part_floats);
   const int G = H / K;
-  const int rows_most = D > 256 ? PLAIN_WAVES : PLAIN_MAX_ROWS;
+  const int rows_most = rw * PLAIN_WAVES;
   const int chunks = (G + rows_most - 1) / rows_most;
-  const int keys = D > 256 ? 32 : 64;
+  const int keys = rw == 1 ? 32 : 64;
   const size_t smem = plain_lds_floats(D, keys, rows_most) * sizeof(float);
   HAL_REQUIRE(smem <= 160 * 1024, "hal_attention_simple: head size %d needs %zu bytes of LDS", D, smem);
   const long long gy = (long long)K * chunks;
@@ -422,15 +496,15 @@ extern "C" int hal_attention_simple(const void* q, int q_row_stride, void* out,
   HAL_REQUIRE((long long)n_pages * K < (1ll << 31), "hal_attention_simple: %d pages of %d heads exceed the index range", n_pages, K);
   dim3 grid((n_tokens + tq - 1) / tq, (unsigned)gy, split ? max_pieces : 1);
   dim3 merge_grid(n_tokens, H);
-#define PLAIN_LAUNCH(T_, R_, KEYS_)                                                                  \
+#define PLAIN_LAUNCH(T_, R_, KEYS_, RW_)                                                                  \
   do {                                                                                              \
     static bool raised = false; /* more than 64 KB of LDS has to be asked for, once per kernel */    \
     if (!raised) {                                                                                  \
-      HAL_CHECK_HIP(hipFuncSetAttribute((const void*)attention_plain_kernel<T_, R_, KEYS_>,         \
+      HAL_CHECK_HIP(hipFuncSetAttribute((const void*)attention_plain_kernel<T_, R_, KEYS_, RW_>,         \
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));   \
       raised = true;                                                                                \
     }                                                                                               \
-    hipLaunchKernelGGL((attention_plain_kernel<T_, R_, KEYS_>), grid, dim3(PLAIN_THREADS), smem,     \
+    hipLaunchKernelGGL((attention_plain_kernel<T_, R_, KEYS_, RW_>), grid, dim3(PLAIN_THREADS), smem,     \
                        stream, (const T_*)q, q_row_stride, (T_*)out, out_row_stride, positions,      \
                        token_seg, block_table, bt_stride, (const T_*)k_pages, (const T_*)v_pages,    \
                        part, n_tokens, H, K, D, page_size, n_pages, scale, window, tq, chunks,       \
@@ -440,12 +514,17 @@ extern "C" int hal_attention_simple(const void* q, int q_row_stride, void* out,
                          stream, (T_*)out, out_row_stride, positions, part, H, D, window,            \
                          max_pieces);                                                                \
   } while (0)
-#define PLAIN_BY_SIZE(T_)                       \
-  do {                                          \
-    if (D <= 64) PLAIN_LAUNCH(T_, 1, 64);       \
-    else if (D <= 128) PLAIN_LAUNCH(T_, 2, 64); \
-    else if (D <= 256) PLAIN_LAUNCH(T_, 4, 64); \
-    else PLAIN_LAUNCH(T_, 8, 32);               \
+#define PLAIN_BY_ROWS(T_, R_)                    \
+  do {                                           \
+    if (rw == 1) PLAIN_LAUNCH(T_, R_, 32, 1);    \
+    else PLAIN_LAUNCH(T_, R_, 64, 4);            \
+  } while (0)
+#define PLAIN_BY_SIZE(T_)                        \
+  do {                                           \
+    if (D <= 64) PLAIN_BY_ROWS(T_, 1);           \
+    else if (D <= 128) PLAIN_BY_ROWS(T_, 2);     \
+    else if (D <= 256) PLAIN_BY_ROWS(T_, 4);     \
+    else PLAIN_LAUNCH(T_, 8, 32, 1);             \
   } while (0)
   if (dtype == HAL_F32)
     PLAIN_BY_SIZE(float);
@@ -454,6 +533,7 @@ extern "C" int hal_attention_simple(const void* q, int q_row_stride, void* out,
   else
     return hal_fail("hal_attention_simple: unknown dtype %d", dtype);
 #undef PLAIN_BY_SIZE
+#undef PLAIN_BY_ROWS
 #undef PLAIN_LAUNCH
   HAL_LAUNCH_CHECK();
   return 0;

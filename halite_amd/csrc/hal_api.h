@@ -40,7 +40,7 @@ int hal_rope_append(void* qkv, int dtype, int row_stride, const int* positions,
 // `hal_attention_simple_plan` says how the step is cut; if `split`, `part` must bring
 // `part_floats` floats for the pieces' partial sums.
 int hal_attention_simple_plan(int n_tokens, int H, int K, int D, int max_kv_len, int* tq, int* split,
-                              int* max_pieces, long long* part_floats);
+                              int* rows_per_wave, int* max_pieces, long long* part_floats);
 int hal_attention_simple(const void* q, int q_row_stride, void* out, int out_row_stride,
                          int dtype, const int* positions, const int* token_seg,
                          const int* block_table, int bt_stride, const void* k_pages,

@@ -343,9 +343,9 @@ def attention_simple(
     out = torch.empty((n, n_heads * head_dim), dtype=q.dtype, device=q.device)
     if max_kv_len is None:
         max_kv_len = block_table.shape[1] * page_size
-    tq, split, pieces, floats = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_longlong()
-    _check(lib, lib.hal_attention_simple_plan(n, n_heads, n_kv, head_dim, max_kv_len, ctypes.byref(tq),
-                                              ctypes.byref(split), ctypes.byref(pieces), ctypes.byref(floats)))
+    tq, split, rows, pieces, floats = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_longlong()
+    _check(lib, lib.hal_attention_simple_plan(n, n_heads, n_kv, head_dim, max_kv_len, ctypes.byref(tq), ctypes.byref(split),
+                                              ctypes.byref(rows), ctypes.byref(pieces), ctypes.byref(floats)))
     part = torch.empty(floats.value, dtype=torch.float32, device=q.device) if floats.value else None
     _check(
         lib,
