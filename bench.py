@@ -191,9 +191,9 @@ def probe_gpu(torch) -> dict:
     }
 
 
-def engine_workload(args) -> int:
+def engine_workload(args) -> dict:
     """The two further workloads: requests through the scheduler (entry point, prompt
-    portions, decoding, sampling), one JSON line.
+    portions, decoding, sampling); returns the record of one.
 
     ``mixed3b``: Llama-3.2-3B shape, 32 requests with prompt lengths uniform in 64..4096,
     prompts cut into portions of 512 tokens, 256 new tokens each.
@@ -290,8 +290,9 @@ def engine_workload(args) -> int:
         "graphs_recorded_before": graphs_before,
         "weights_gb": round(runner.model.param_bytes() / 1e9, 2),
     }
-    print(json.dumps(record), flush=True)
-    return 0
+    del engine
+    runner.release()
+    return record
 
 
 def main() -> int:
@@ -317,12 +318,16 @@ def main() -> int:
                     help="how the decode steps sample (the contract's line is greedy)")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b"],
                     help="decode8b: the headline line; the others run requests through the scheduler")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="leave out what the default line adds beyond the contract's points: contexts of 32,768, "
+                         "the 32-bit points and the 3B requests through the scheduler")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
     if args.workload != "decode8b":
-        return engine_workload(args)
+        print(json.dumps(engine_workload(args)), flush=True)
+        return 0
 
     import numpy as np
     import torch
@@ -336,23 +341,27 @@ def main() -> int:
     n_layers = args.layers or full.num_hidden_layers
     cfg = full.model_copy(update={"num_hidden_layers": n_layers})
     context = args.context or 8192  # the benchmark's context; the model itself goes to 131,072
-    elt = 2 if args.dtype == "bfloat16" else 4
+    dtype = args.dtype  # (the 32-bit points of the default line run the same functions once more)
+    elt = 2 if dtype == "bfloat16" else 4
+    extras = dtype == "bfloat16" and not (args.no_points or args.no_extras or args.prefill_only)
+    LONG = 32768  # the further context of the default line
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     if args.dtype == "float32" and not args.no_points:
         batches = sorted({1, args.batch})  # the 32-bit path is for exactness: fewer, shorter points
     if args.prefill_only:
         batches, context = [1], max(4096, args.prefill_tokens + 64)
     # (batch, context at the end of decoding) of every point beyond the headline
-    more = [(16, context), (32, context), (128, context), (8, 32768), (1, 131072)] if args.more_points else []
-    pool_tokens = max([b * (context + 64) for b in batches] + [b * (c + 64) for b, c in more]) + 4096
-    longest = max([context] + [c for _, c in more] + ([16384 + 64] if args.more_points else []))
+    more = [(16, context), (32, context), (128, context), (8, 32768), (1, 131072), (8, 131072)] if args.more_points else []
+    pool_tokens = max([b * (context + 64) for b in batches] + [b * (c + 64) for b, c in more]
+                      + ([32 * (LONG + 64)] if extras else [])) + 4096
+    longest = max([context] + [c for _, c in more] + ([16384 + 64] if args.more_points else []) + ([LONG + 64] if extras else []))
     runner = ModelRunner.from_random(
         cfg, seed=0,
         server_config=ServerConfig(kv_cache_num_tokens=pool_tokens,
-                                   max_seqs_per_forward=max(batches + [b for b, _ in more]) + 1,
+                                   max_seqs_per_forward=max(batches + [b for b, _ in more] + ([32] if extras else [])) + 1,
                                    max_tokens_per_forward=16384, use_cudagraph=not args.no_graph,
-                                   cudagraph_max_batch_size=max(batches + [b for b, _ in more])),
-        model_config=ModelConfig(dtype=args.dtype, context_len=longest),
+                                   cudagraph_max_batch_size=max(batches + [b for b, _ in more] + ([32] if extras else []))),
+        model_config=ModelConfig(dtype=dtype, context_len=longest),
     )
     sampler = Sampler(runner.device)
     greedy = SamplingParams(temperature=0.0)
@@ -363,16 +372,24 @@ def main() -> int:
 
     EXTRA_MARKED = 8
 
-    def decode_run(batch: int, steps: int, warmup: int, end_context: int = context, families: bool = False):
+    def decode_run(batch: int, steps: int, warmup: int, end_context: int = context, families: bool = False,
+                   keep: list | None = None, reuse: list | None = None):
         """Prefills ``batch`` prompts so that the contexts end at ``end_context`` after
         the last timed step, then times ``steps`` decode steps.  Returns the seconds, the
         mean number of cached tokens of a step, the GPU's share of the time (events around
-        every step) and, if asked for, the families' times of one more, eager step."""
+        every step) and, if asked for, the families' times of one more, eager step.
+        ``keep``: a list that takes the requests (slot, last token) instead of their being
+        freed; ``reuse``: such requests, of which the first ``batch`` go on decoding from
+        where they are (the others are freed) instead of new prompts."""
         prompt_len = end_context - steps - warmup - (2 + EXTRA_MARKED if families else 0)
-        slots = [runner.admit() for _ in range(batch)]
-        last = []
+        if reuse is not None:
+            for s, _ in reuse[batch:]:
+                runner.free(s)
+            slots, last = [s for s, _ in reuse[:batch]], [t for _, t in reuse[:batch]]
+        else:
+            slots, last = [runner.admit() for _ in range(batch)], []
         t_said = time.perf_counter()
-        for i_slot, s in enumerate(slots):
+        for i_slot, s in enumerate(slots if reuse is None else []):
             if time.perf_counter() - t_said > 30:  # a long set-up says that it is alive
                 sync()
                 print(f"[bench] batch {batch}: prompt {i_slot} of {batch} ...", file=sys.stderr, flush=True)
@@ -433,8 +450,11 @@ def main() -> int:
                 fam = f.totals_ms()
             finally:
                 runner.graphs_allowed = graph
-        for s in slots:
-            runner.free(s)
+        if keep is not None:
+            keep.extend(zip(slots, last))
+        else:
+            for s in slots:
+                runner.free(s)
         return dt, kv_tokens, gpu_s, fam
 
     def prefill_run(T=args.prefill_tokens, families: bool = False, portion: int = 0):
@@ -461,7 +481,7 @@ def main() -> int:
                 times.append(time.perf_counter() - t0)
             runner.free(s)
         t = min(times[1:])
-        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+        peak = PEAK_FLOPS["bf16" if dtype == "bfloat16" else "fp32"]
         out = {
             "value": round(T / t, 1),
             "tokens": T,
@@ -509,7 +529,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "dtype": "bf16" if dtype == "bfloat16" else "fp32",
         "data": "synthetic: seeded uniform-random token ids, random weights N(0, 0.02)",
         "config": {
             "model": "Llama-3.1-8B shape",
@@ -565,8 +585,8 @@ def main() -> int:
                 points[f"decode_b{b}_frac"] = frac_of(b, context, n_steps, seconds, cached)
         # the other reading of the decode points: prompts of 512 tokens, as the benchmark
         # configuration words its decode workload (the reference publishes no figures)
-        for b in ((1, 8, 64) if args.dtype == "bfloat16" else (1, 8)):
-            n_steps = max(8, args.steps // 2) if args.dtype == "bfloat16" else 4
+        for b in ((1, 8, 64) if dtype == "bfloat16" else (1, 8)):
+            n_steps = max(8, args.steps // 2) if dtype == "bfloat16" else 4
             seconds, cached, _, _ = decode_run(b, n_steps, args.warmup, end_context=512 + n_steps + args.warmup)
             points[f"decode_p512_b{b}"] = round(b * n_steps / seconds, 2)
             points[f"decode_p512_b{b}_frac"] = frac_of(b, 0, n_steps, seconds, cached)
@@ -593,6 +613,56 @@ def main() -> int:
         record["prefill"]["frac_of_measured_gemm"] = round(
             prefill_flops(cfg, n_layers, record["prefill"]["tokens"]) / (record["prefill"]["ms"] * 1e-3)
             / (record["probe"]["gemm_8192_tflops"] * 1e12), 4)
+    if extras:
+        # -- further sizes: 32 requests whose contexts end near 32,768, then 16 of them --
+        t_extra = time.perf_counter()
+        n_steps = max(8, args.steps // 4)
+        held = []
+        seconds, cached, _, _ = decode_run(32, n_steps, 4, end_context=LONG - n_steps - 4, keep=held)
+        points[f"decode_b32_ctx{LONG}"] = round(32 * n_steps / seconds, 2)
+        points[f"decode_b32_ctx{LONG}_frac"] = frac_of(32, LONG, n_steps, seconds, cached)
+        seconds, cached, _, _ = decode_run(16, n_steps, 4, end_context=LONG, reuse=held)
+        points[f"decode_b16_ctx{LONG}"] = round(16 * n_steps / seconds, 2)
+        points[f"decode_b16_ctx{LONG}_frac"] = frac_of(16, LONG, n_steps, seconds, cached)
+        extra = prefill_run(LONG)
+        points[f"prefill_{LONG}"] = extra["value"]
+        points[f"prefill_{LONG}_frac"] = extra["frac"]
+        print(f"[bench] context {LONG}: decode batch 32 {points[f'decode_b32_ctx{LONG}']} tok/s, batch 16 "
+              f"{points[f'decode_b16_ctx{LONG}']} tok/s, prefill {extra['value']} tok/s "
+              f"({time.perf_counter() - t_extra:.0f} s)", file=sys.stderr, flush=True)
+        # -- the 32-bit path: the same functions on a model of float32 --
+        t_extra = time.perf_counter()
+        runner.release()
+        dtype, elt = "float32", 4
+        runner = ModelRunner.from_random(
+            cfg, seed=0,
+            server_config=ServerConfig(kv_cache_num_tokens=args.batch * (context + 64) + 4096, max_seqs_per_forward=args.batch + 1,
+                                       max_tokens_per_forward=16384, use_cudagraph=not args.no_graph,
+                                       cudagraph_max_batch_size=args.batch),
+            model_config=ModelConfig(dtype=dtype, context_len=context + 64),
+        )
+        n_steps = 8
+        seconds, cached, _, _ = decode_run(args.batch, n_steps, 2)
+        points[f"decode_b{args.batch}_fp32"] = round(args.batch * n_steps / seconds, 2)
+        points[f"decode_b{args.batch}_fp32_ms"] = round(seconds / n_steps * 1e3, 3)
+        points[f"decode_b{args.batch}_fp32_frac"] = frac_of(args.batch, context, n_steps, seconds, cached)
+        extra = prefill_run()
+        points[f"prefill_{extra['tokens']}_fp32"] = extra["value"]
+        points[f"prefill_{extra['tokens']}_fp32_frac"] = extra["frac"]
+        print(f"[bench] float32: decode batch {args.batch} {points[f'decode_b{args.batch}_fp32_ms']} ms/step, prefill "
+              f"{extra['value']} tok/s ({time.perf_counter() - t_extra:.0f} s)", file=sys.stderr, flush=True)
+        runner.release()
+        dtype, elt = args.dtype, 2
+        # -- requests through the scheduler: the 3B shape, 32 requests of mixed lengths --
+        args.workload = "mixed3b"
+        w = engine_workload(args)
+        record["workloads"] = {"mixed3b": {
+            "value": w["value"], "unit": "generated tok/s", "seconds": w["seconds"], "steps": w["steps"],
+            "mean_tokens_per_step": w["mean_tokens_per_step"], "retractions": w["retractions"],
+            "total_tokens_per_second": w["total_tokens_per_second"], "requests": w["config"]["global_batch"],
+            "prompt_tokens": w["config"]["prompt_tokens"], "new_tokens_each": w["config"]["new_tokens_each"],
+            "prefill_portion": w["config"]["prefill_portion"], "layers": w["config"]["layers"],
+        }}
     print(json.dumps(record), flush=True)
     return 0
 
