@@ -6,7 +6,8 @@
 // Two kernels.  The tiled one (any M): each output element is one chain of K multiply-adds
 // in index order.  The one for at most 16 rows (decode steps), which the tiled one serves
 // at 1/64 to 1/4 of its tile: a wave takes a few columns of the output, its lanes take
-// every 64th group of four k each, and the lanes' partial sums are added in a fixed tree.
+// every 64th group of four k each (the rows of A come through LDS, shared by the workgroup's
+// four waves), and the lanes' partial sums are added in a fixed tree.
 // In both a token's result depends on its own row alone, not on what else is in the batch;
 // between the two the order of the additions differs, i.e. the last bits may.
 #include "hal_common.h"
@@ -79,34 +80,61 @@ __global__ void __launch_bounds__(256)
 gemm_f32_skinny_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
                        float* __restrict__ C, int ldc, int M, int N, int K) {
   static_assert(MB * NC == HAL_WAVE, "one output per lane");
-  const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
+  // The rows of A go through LDS in pieces of CH k, brought by all four waves together (a
+  // wave that read them itself would ask memory for as many bytes of A as of W); the next
+  // piece is on its way to registers while this one is worked on.
+  constexpr int CH = 8192 / MB;                // k of a piece: 32 KB of LDS
+  constexpr int AV = MB * CH / 4 / 256;        // 16-byte vectors of a piece per thread
+  __shared__ __align__(16) float a_s[MB][CH];
+  const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
   const int n0 = (blockIdx.x * 4 + wave) * NC;
-  if (n0 >= N) return;
+  const bool have_columns = n0 < N;  // (a wave without columns still helps with A)
   const float* wrow[NC];
 #pragma unroll
   for (int c = 0; c < NC; ++c) wrow[c] = W + (size_t)(n0 + c < N ? n0 + c : N - 1) * ldw;
   float v[MB * NC];
 #pragma unroll
   for (int i = 0; i < MB * NC; ++i) v[i] = 0.f;
-  for (int k = lane * 4; k < K; k += HAL_WAVE * 4) {  // K is a multiple of 4
-    float4 w[NC], a[MB];
+  float4 a_next[AV];
+  auto ask_piece = [&](int k0) {  // vector e of the piece: row e / (CH/4), k0 + 4 (e % (CH/4))
 #pragma unroll
-    for (int c = 0; c < NC; ++c) w[c] = *(const float4*)(wrow[c] + k);
+    for (int u = 0; u < AV; ++u) {
+      const int e = tid + u * 256, m = e / (CH / 4), k = k0 + (e % (CH / 4)) * 4;
+      a_next[u] = (m < M && k < K) ? *(const float4*)(A + (size_t)m * lda + k) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  ask_piece(0);
+  for (int k0 = 0; k0 < K; k0 += CH) {
+    __syncthreads();  // the piece before is read
 #pragma unroll
-    for (int m = 0; m < MB; ++m)
-      a[m] = m < M ? *(const float4*)(A + (size_t)m * lda + k) : float4{0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < AV; ++u) {
+      const int e = tid + u * 256;
+      *(float4*)&a_s[e / (CH / 4)][(e % (CH / 4)) * 4] = a_next[u];
+    }
+    if (k0 + CH < K) ask_piece(k0 + CH);
+    __syncthreads();
+    if (!have_columns) continue;
+    const int k_end = k0 + CH < K ? k0 + CH : K;
+    for (int k = k0 + lane * 4; k < k_end; k += HAL_WAVE * 4) {  // K is a multiple of 4
+      float4 w[NC], a[MB];
 #pragma unroll
-    for (int m = 0; m < MB; ++m)
+      for (int c = 0; c < NC; ++c) w[c] = *(const float4*)(wrow[c] + k);
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        float s = v[m * NC + c];
-        s = fmaf(a[m].x, w[c].x, s);
-        s = fmaf(a[m].y, w[c].y, s);
-        s = fmaf(a[m].z, w[c].z, s);
-        s = fmaf(a[m].w, w[c].w, s);
-        v[m * NC + c] = s;
-      }
+      for (int m = 0; m < MB; ++m) a[m] = *(const float4*)&a_s[m][k - k0];
+#pragma unroll
+      for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          float s = v[m * NC + c];
+          s = fmaf(a[m].x, w[c].x, s);
+          s = fmaf(a[m].y, w[c].y, s);
+          s = fmaf(a[m].z, w[c].z, s);
+          s = fmaf(a[m].w, w[c].w, s);
+          v[m * NC + c] = s;
+        }
+    }
   }
+  if (!have_columns) return;
 #pragma unroll
   for (int half = HAL_WAVE / 2; half >= 1; half /= 2) {
     const bool upper = (lane & half) != 0;
