@@ -16,15 +16,15 @@ import sys
 import numpy as np
 import torch
 
-from ..parts.base import PagedKVNeed, StateNeed
-from .pages import CacheGroup, LayerPages, NoSpace, PagePool, tiled_layout
+from ..parts.base import PagedNeed, StateNeed
+from .pages import CacheGroup, NoSpace, PagePool
 from .slots import SlotAllocator, StateStore
 
 
 class CacheManager:
     def __init__(
         self,
-        needs: dict[int, PagedKVNeed],
+        needs: dict[int, PagedNeed],
         borrowed: dict[int, int] | None = None,
         state_needs: dict[int, dict[str, StateNeed]] | None = None,
         *,
@@ -44,7 +44,7 @@ class CacheManager:
         self.device = torch.device(device)
         self.groups: list[CacheGroup] = []
         self.group_of_run: dict[int, int] = {}
-        by_need: dict[PagedKVNeed, CacheGroup] = {}
+        by_need: dict[PagedNeed, CacheGroup] = {}
         for run in sorted(needs):
             need = needs[run]
             if need not in by_need:
@@ -58,20 +58,22 @@ class CacheManager:
             if owner not in self.group_of_run:
                 raise ValueError(f"run {run} borrows the cache of run {owner}, which owns none")
             self.group_of_run[run] = self.group_of_run[owner]
-        self._pages: dict[int, LayerPages] = {}
+        # what a run's mixer finds in ``run.kv``: the need says which tensors a page number
+        # stands for and binds them; a run's tensors lie one after the other in the group's
+        # storage, each ``[pages, *shape]``
+        self._pages: dict[int, object] = {}
         for g in self.groups:
-            k, d = g.need.n_kv_heads, g.need.head_dim
+            shapes = g.need.page_tensors(page_size)
+            sizes = {name: int(np.prod(shape)) for name, shape in shapes.items()}
             if allocate:
-                g.storage = torch.zeros(
-                    (len(g.runs), 2, num_pages, k * page_size * d), dtype=dtype, device=self.device
-                )
+                g.storage = torch.zeros((len(g.runs), num_pages * sum(sizes.values())), dtype=dtype, device=self.device)
             for i, run in enumerate(g.runs):
-                if allocate:
-                    kp = g.storage[i, 0].view(num_pages, k, page_size, d)
-                    vp = g.storage[i, 1].view(num_pages, k, d, page_size)
-                else:
-                    kp = vp = None
-                self._pages[run] = LayerPages(g.group_id, kp, vp, tiled_layout(dtype, d, page_size))
+                tensors, at = {}, 0
+                for name, shape in shapes.items():
+                    n = num_pages * sizes[name]
+                    tensors[name] = g.storage[i, at : at + n].view(num_pages, *shape) if allocate else None
+                    at += n
+                self._pages[run] = g.need.bind(g.group_id, tensors, page_size, dtype)
         for run, owner in self.borrowed.items():
             self._pages[run] = self._pages[owner]
         self.slots = SlotAllocator(n_slots)
@@ -81,9 +83,9 @@ class CacheManager:
 
     # -- sizes ------------------------------------------------------------------
     @staticmethod
-    def bytes_per_page(needs: dict[int, PagedKVNeed], page_size: int, dtype: torch.dtype) -> int:
+    def bytes_per_page(needs: dict[int, PagedNeed], page_size: int, dtype: torch.dtype) -> int:
         """Bytes that one page number costs over all groups and runs."""
-        return sum(2 * n.n_kv_heads * n.head_dim * page_size * dtype.itemsize for n in needs.values())
+        return sum(int(np.prod(shape)) * dtype.itemsize for n in needs.values() for shape in n.page_tensors(page_size).values())
 
     @property
     def token_capacity(self) -> int:
@@ -94,7 +96,7 @@ class CacheManager:
         run out of, which the largest integer stands for."""
         return min((g.pool.available for g in self.groups), default=sys.maxsize)
 
-    def layer_pages(self, run: int) -> LayerPages | None:
+    def layer_pages(self, run: int):
         return self._pages.get(run)
 
     def state_of_run(self, run: int) -> dict[str, torch.Tensor]:
@@ -105,8 +107,7 @@ class CacheManager:
         manager serves no step afterwards."""
         for g in self.groups:
             g.storage = None
-        for pages in self._pages.values():
-            pages.k = pages.v = None
+        self._pages = {}  # (whoever took a run's pages from ``layer_pages`` lets go of them too)
         self.state.tensors = {}
 
     # -- requests -----------------------------------------------------------------

@@ -17,7 +17,7 @@ from dataclasses import dataclass, field
 
 import torch
 
-from ..parts.base import PagedKVNeed
+from ..parts.base import PagedNeed
 
 
 class NoSpace(Exception):
@@ -94,14 +94,14 @@ class LayerPages:
 @dataclass
 class CacheGroup:
     group_id: int
-    need: PagedKVNeed
+    need: PagedNeed  # (its ``window`` is all that the bookkeeping below reads)
     runs: list[int]  # indices of the runs that own a cache in this group
     page_size: int
     pool: PagePool
     # per live slot: page number for every logical page, -1 where none is held
     tables: dict[int, list[int]] = field(default_factory=dict)
     released: dict[int, int] = field(default_factory=dict)
-    storage: torch.Tensor | None = None  # [runs, 2, pages, K * page_size * D]
+    storage: torch.Tensor | None = None  # [runs, pages * elements of a page]: a run's tensors one after the other
 
     def first_needed_page(self, next_position: int) -> int:
         """Logical pages before this one are out of reach of every query at

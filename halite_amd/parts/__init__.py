@@ -15,6 +15,7 @@ from .base import (
     Mixer,
     Norm,
     PagedKVNeed,
+    PagedNeed,
     ParamDecl,
     Part,
     PositionEncoding,
@@ -28,6 +29,6 @@ from .decoder import Decoder
 __all__ = [
     "ARRANGEMENTS", "EMBEDDINGS", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITIONS",
     "Arrangement", "BuildContext", "Decoder", "Embedding", "FeedForward", "Head", "Mixer", "Norm",
-    "PagedKVNeed", "ParamDecl", "Part", "PositionEncoding", "RotaryPositionEncoding", "RunBinding", "StateNeed",
+    "PagedKVNeed", "PagedNeed", "ParamDecl", "Part", "PositionEncoding", "RotaryPositionEncoding", "RunBinding", "StateNeed",
     "register_arrangement",
 ]

@@ -35,15 +35,47 @@ class ParamDecl:
     integer: bool = False
 
 
+class PagedNeed:
+    """Something of every token, kept in pages.  What a mixer's ``cache_need`` returns is a
+    frozen dataclass of this kind: runs whose needs are equal share one group of pages (one
+    block table per request for all of them).  The cache manager reads three things of a need:
+
+    * ``window`` (an attribute; ``None``: every token's page is kept while the request lives;
+      else the tokens a query looks back, itself included, so that pages are given back once
+      every later query has passed them);
+    * ``page_tensors(page_size)``: name -> shape of one page, the tensors a run keeps per page
+      number, all of the cache's element type;
+    * ``bind(group_id, tensors, page_size, dtype)``: what the run's mixer finds in ``run.kv``,
+      made of those tensors (each ``[pages, *shape]``).
+    """
+
+    window: int | None = None
+
+    def page_tensors(self, page_size: int) -> dict[str, tuple[int, ...]]:
+        raise NotImplementedError
+
+    def bind(self, group_id: int, tensors: dict[str, torch.Tensor | None], page_size: int, dtype: torch.dtype):
+        raise NotImplementedError
+
+
 @dataclass(frozen=True)
-class PagedKVNeed:
-    """Keys and values of every token, kept in pages.  Runs whose needs are equal
-    share one group of pages; ``window`` (tokens a query looks back, itself
-    included) lets pages be given back once every later query has passed them."""
+class PagedKVNeed(PagedNeed):
+    """Keys and values of every token: keys ``[K, page_size, D]`` and values, transposed,
+    ``[K, D, page_size]`` per page (or the same bytes in the matrix-core attention kernel's
+    order, see ``cache.pages.tiled_layout``); ``run.kv`` is a ``cache.pages.LayerPages``."""
 
     n_kv_heads: int
     head_dim: int
     window: int | None = None
+
+    def page_tensors(self, page_size: int) -> dict[str, tuple[int, ...]]:
+        k, d = self.n_kv_heads, self.head_dim
+        return {"k": (k, page_size, d), "v": (k, d, page_size)}
+
+    def bind(self, group_id, tensors, page_size, dtype):
+        from ..cache.pages import LayerPages, tiled_layout
+
+        return LayerPages(group_id, tensors["k"], tensors["v"], tiled_layout(dtype, self.head_dim, page_size))
 
 
 @dataclass(frozen=True)
@@ -109,7 +141,7 @@ class Part:
     def finalize(self) -> None:
         """Called once after the tensors are filled."""
 
-    def cache_need(self) -> PagedKVNeed | None:
+    def cache_need(self) -> PagedNeed | None:
         return None
 
     def state_need(self) -> dict[str, StateNeed]:

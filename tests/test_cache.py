@@ -1,10 +1,12 @@
 import random
+from dataclasses import dataclass
 
 import numpy as np
 import pytest
+import torch
 
 from halite_amd.cache import CacheManager, NoSlot, NoSpace, PagePool
-from halite_amd.parts.base import PagedKVNeed, StateNeed
+from halite_amd.parts.base import PagedKVNeed, PagedNeed, StateNeed
 
 FULL = PagedKVNeed(2, 16)
 WIN = PagedKVNeed(2, 16, window=10)
@@ -40,6 +42,46 @@ def test_groups_by_need():
     assert m.group_of_run[4] == 1
     with pytest.raises(ValueError, match="owns none"):
         manager({0: FULL}, borrowed={1: 5})
+
+
+@dataclass(frozen=True)
+class OneVectorNeed(PagedNeed):
+    """A need that is defined here: one vector a token and a count a page."""
+
+    width: int
+    window: int | None = None
+
+    def page_tensors(self, page_size):
+        return {"vector": (page_size, self.width), "count": (1,)}
+
+    def bind(self, group_id, tensors, page_size, dtype):
+        return {"group": group_id, **tensors}
+
+
+def test_a_need_says_what_a_page_holds():
+    needs = {0: OneVectorNeed(6), 1: FULL, 2: OneVectorNeed(6), 3: OneVectorNeed(6, window=8)}
+    m = CacheManager(needs, page_size=4, num_pages=9, n_slots=2, dtype=torch.bfloat16)
+    assert [g.runs for g in m.groups] == [[0, 2], [1], [3]]
+    assert [tuple(g.storage.shape) for g in m.groups] == [(2, 9 * 25), (1, 9 * 2 * 2 * 4 * 16), (1, 9 * 25)]
+    assert CacheManager.bytes_per_page(needs, 4, torch.bfloat16) == (3 * 25 + 2 * 2 * 4 * 16) * 2
+    a, b = m.layer_pages(0), m.layer_pages(2)
+    assert a["group"] == b["group"] == 0 and m.layer_pages(3)["group"] == 2
+    assert tuple(a["vector"].shape) == (9, 4, 6) and tuple(a["count"].shape) == (9, 1)
+    # every tensor of every run has memory of its own, inside the group's storage
+    a["vector"].fill_(1), a["count"].fill_(2), b["vector"].fill_(3), b["count"].fill_(4)
+    assert m.groups[0].storage[0].float().sum() == 9 * 24 * 1 + 9 * 2 and m.groups[0].storage[1].float().sum() == 9 * 24 * 3 + 9 * 4
+    kv = m.layer_pages(1)
+    assert tuple(kv.k.shape) == (9, 2, 4, 16) and tuple(kv.v.shape) == (9, 2, 16, 4)
+    # the books are the same for every kind of page
+    s = m.admit()
+    m.reserve([(s, 14)])
+    m.advance(s, 14)
+    assert [sum(p >= 0 for p in g.tables[s]) for g in m.groups] == [4, 4, 3]
+    m.check()
+    m.free(s)
+    assert m.idle()
+    m.release_storage()
+    assert m.layer_pages(0) is None and m.groups[0].storage is None
 
 
 def test_reserve_advance_free():

@@ -86,7 +86,17 @@ def test_temperature_sampling_with_a_seed(models, dtype):
     if dtype == "float32":
         assert alone[0].output_ids == results[1].output_ids
     else:
-        assert alone[0].output_ids[0][:4] == results[1].output_ids[0][:4]
+        # every token of the run alone is the plain implementation's draw from the same stream,
+        # or a draw within rounding of an interval's edge; and up to the first such draw the two
+        # runs are the same tokens
+        check_against_plain(pc, pw, prompts[1], alone[0].output_ids[0], plain_params, 0, 2e-2)
+        a, b = alone[0].output_ids[0], results[1].output_ids[0]
+        same = next((i for i in range(24) if a[i] != b[i]), 24)
+        assert same >= 4
+        if same < 24:
+            logits = plain_llama.forward(pc, pw, prompts[1] + a[:same])[-1]
+            _, _, margin = plain_llama.sample_token(logits, plain_params, same)
+            assert margin is not None and margin <= 2e-2, (same, margin)
     other = engine.infer_batch([(0, prompts[1], SamplingParams(max_new_tokens=24, temperature=0.8, seed=99))])
     assert other[0].output_ids != results[1].output_ids
     # n samples of one request draw from different streams

@@ -1,7 +1,10 @@
 """The parts alone, and models put together from parts as data: a windowed layer, a
 layer that runs twice, a layer that reads another layer's cache, and toy parts that are
 defined here and registered without touching the framework: a mixer with state of its
-own, a feed-forward that routes tokens to experts, and another position encoding."""
+own, a mixer whose pages hold something else than keys and values, a feed-forward that
+routes tokens to experts, and another position encoding."""
+
+from dataclasses import dataclass
 
 import pytest
 import torch
@@ -13,7 +16,7 @@ import tiny
 from halite_amd.config import LayerRun, LayerSpec, ModelConfig, ModelSpec, PartSpec, ServerConfig, parse_config
 from halite_amd.engine.batch import Segment
 from halite_amd.engine.runner import ModelRunner
-from halite_amd.parts import MIXERS, BuildContext, Decoder, Mixer, ParamDecl, StateNeed
+from halite_amd.parts import MIXERS, BuildContext, Decoder, Mixer, PagedNeed, ParamDecl, StateNeed
 from halite_amd.parts.base import FEED_FORWARDS, NORMS, POSITIONS, Arrangement, FeedForward, PositionEncoding, register_arrangement
 from halite_amd.weights import fill_random
 
@@ -312,6 +315,108 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(gpu, dtype):
     s = runner.admit()
     assert float(runner.cache.state.tensors[0]["sum"][s].abs().sum()) == 0
     runner.free(s)
+
+
+# -- a toy mixer whose pages hold one small vector a token, not keys and values -----------
+
+
+@dataclass(frozen=True)
+class LatentNeed(PagedNeed):
+    width: int
+    window: int | None = None
+
+    def page_tensors(self, page_size):
+        return {"latent": (page_size, self.width)}
+
+    def bind(self, group_id, tensors, page_size, dtype):
+        return LatentPages(group_id, tensors["latent"])
+
+
+@dataclass
+class LatentPages:
+    group_id: int
+    latent: torch.Tensor | None  # [pages, page_size, width]
+
+
+class LookBackParams(BaseModel):
+    hidden_size: int
+    width: int
+    window: int | None = None
+
+
+@MIXERS.register("toy_look_back")
+class ToyLookBack(Mixer):
+    """``y_t = U * mean(D x_s for s in the last `window` tokens up to t)``: what it keeps of a
+    token is ``D x_s``, ``width`` numbers, in pages of its own shape."""
+
+    Params = LookBackParams
+
+    def param_decls(self):
+        p = self.p
+        return {"down.weight": ParamDecl((p.width, p.hidden_size)), "up.weight": ParamDecl((p.hidden_size, p.width))}
+
+    def cache_need(self):
+        return LatentNeed(self.p.width, self.p.window)
+
+    def forward(self, x, ctx, run):
+        group = ctx.group(run.kv.group_id)
+        pages, size = run.kv.latent, group.page_size
+        latent = (x.float() @ self.down_weight.float().T).to(pages.dtype)
+        out = torch.empty((x.shape[0], self.p.width), dtype=torch.float32, device=x.device)
+        for i, (seg, q0, n) in enumerate(zip(ctx.segments, ctx.seg_q_start_host, ctx.seg_q_len_host)):
+            table = group.block_table[i].long()
+            now = torch.arange(seg.start, seg.start + n, device=x.device)
+            pages[table[now // size], now % size] = latent[q0 : q0 + n]
+            first = 0 if self.p.window is None else max(0, seg.start - self.p.window + 1)
+            kept = torch.arange(first, seg.start + n, device=x.device)
+            sums = torch.cumsum(pages[table[kept // size], kept % size].float(), 0)
+            sums = torch.cat((torch.zeros_like(sums[:1]), sums))  # sums[j]: of the kept tokens before first + j
+            lo = now - (self.p.window - 1) if self.p.window is not None else torch.zeros_like(now)
+            lo = torch.clamp(lo, min=first)
+            out[q0 : q0 + n] = (sums[now + 1 - first] - sums[lo - first]) / (now + 1 - lo)[:, None]
+        return (out @ self.up_weight.float().T).to(x.dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_mixer_with_pages_of_another_shape(gpu, dtype):
+    spec = toy_spec(
+        {"far": PartSpec(kind="toy_look_back", hidden_size=64, width=24), "att": attention_spec(),
+         "near": PartSpec(kind="toy_look_back", hidden_size=64, width=24, window=20)},
+        [LayerRun(layer="far"), LayerRun(layer="att"), LayerRun(layer="near"), LayerRun(layer="far")],
+    )
+    runner = make_runner(gpu, spec, dtype, tokens=192)
+    cache = runner.cache
+    assert [g.runs for g in cache.groups] == [[0, 3], [1], [2]]
+    pages = cache.num_pages
+    assert cache.groups[0].storage.shape == (2, pages * 16 * 24) and cache.groups[2].storage.shape == (1, pages * 16 * 24)
+    assert cache.groups[1].storage.shape == (1, pages * 2 * 2 * 16 * 16)
+    needs = {i: runner.model.mixer_of_run(i).cache_need() for i in range(4)}
+    assert cache.bytes_per_page(needs, 16, DT[dtype]) == (3 * 16 * 24 + 2 * 2 * 16 * 16) * DT[dtype].itemsize
+    assert runner.model.runs[0].kv.latent.data_ptr() != runner.model.runs[3].kv.latent.data_ptr()
+    for g in cache.groups:  # a page that was never written, or is read after its time, shows
+        g.storage.fill_(float("nan"))
+    rope_p = dict(rotary_dim=16, theta=10000.0, interleaved=False)
+    round_to = (lambda t: t.to(torch.bfloat16).float()) if dtype == "bfloat16" else (lambda t: t)
+
+    def look_back(part, x, positions, i, run, memo):
+        latent = round_to(x @ part.down_weight.float().cpu().T)
+        w = part.p.window or x.shape[0]
+        mean = torch.stack([latent[max(0, t - w + 1) : t + 1].mean(0) for t in range(x.shape[0])])
+        return mean @ part.up_weight.float().cpu().T
+
+    def att(part, x, positions, i, run, memo):
+        return plain_attention_layer(part, x, positions, rope_p)[0]
+
+    requests = {f"r{i}": [int(t) % 97 for t in tiny.random_tokens(tiny.TINY_A, n, 70 + i)] for i, n in enumerate([60, 3, 35, 18])}
+    ref = {rid: plain_model(runner.model, toks, {"far": look_back, "near": look_back, "att": att}) for rid, toks in requests.items()}
+    replay_all(runner, requests, ref, TOL[dtype], 97)
+    # the windowed group gives pages back while a request runs, the other keeps them
+    slot = runner.admit()
+    runner.step([Segment(slot, 0, requests["r0"][:50], want=[])])
+    held = [sum(p >= 0 for p in g.tables[slot]) for g in cache.groups]
+    assert held == [4, 4, 3], held  # the next query looks back to token 31, on the second page
+    runner.free(slot)
+    assert cache.idle()
 
 
 # -- a toy feed-forward that routes, and another position encoding ------------------------
