@@ -1,15 +1,17 @@
-// C[M, N] = A[M, K] * W[N, K]^T in true float32: plain fused multiply-adds on the
-// vector units, no matrix-core mode of reduced precision.  W has the layout of a
-// bias-free linear layer's weight ([out, in], src/halite/transformers/feedforward.py:
+// C[M, N] = A[M, K] * W[N, K]^T in true float32: float32 multiply-adds on the vector units
+// or the matrix cores' float32 instruction, no mode of reduced precision.  W has the layout
+// of a bias-free linear layer's weight ([out, in], src/halite/transformers/feedforward.py:
 // 204-212; src/halite/transformers/infer/attention.py:21-24).
 //
-// Two kernels.  The tiled one (any M): each output element is one chain of K multiply-adds
-// in index order.  The one for at most 16 rows (decode steps), which the tiled one serves
-// at 1/64 to 1/4 of its tile: a wave takes a few columns of the output, its lanes take
-// every 64th group of four k each (the rows of A come through LDS, shared by the workgroup's
-// four waves), and the lanes' partial sums are added in a fixed tree.
-// In both a token's result depends on its own row alone, not on what else is in the batch;
-// between the two the order of the additions differs, i.e. the last bits may.
+// Three kernels.  At most 16 rows (decode steps): a wave takes a few columns of the output,
+// its lanes take every 64th group of four k each (the rows of A come through LDS, shared by
+// the workgroup's four waves), and the partial sums of the lanes, and of the waves that share
+// columns, are added in a fixed order.  More than 64 rows (prompts): tiles of 128 x 128 on the
+// matrix cores.  Between them, and for sizes and addresses that are no multiples of four:
+// tiles of 64 x 64 on the vector units, each output element one chain of K multiply-adds in
+// index order.
+// In all three a token's result depends on its own row alone, not on what else is in the
+// batch; between them the order of the additions differs, i.e. the last bits may.
 #include "hal_common.h"
 #include "hal_api.h"
 
@@ -70,24 +72,142 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
   }
 }
 
+// ---- many rows: the matrix cores' float32 instruction -----------------------------------------
+// v_mfma_f32_32x32x2_f32 multiplies and adds in float32 (it is the instruction behind the
+// published float32 matrix rate, not one of the reduced-precision modes), at twice the rate of
+// the vector units' multiply-adds.  A workgroup of four waves takes 128 x 128 outputs, a wave
+// 64 x 64 as 2 x 2 products of 32 x 32; k goes through LDS 32 at a time, in two buffers, the
+// next stage on its way to registers while this one is multiplied.
+//
+// The instruction takes, from lane l, A[row l % 32][k l / 32] and B[k l / 32][column l % 32],
+// two k a call.  Which two k of the stage a call gets is free as long as A and B agree: the
+// lower half of the lanes takes the k's 8 s .. 8 s + 3, the upper half 8 s + 4 .. 8 s + 7
+// (s = 0 .. 3), one 16-byte LDS read per operand block and four calls each.  An output element
+// is the sum over k in that order, rounded as the instruction rounds; it depends on its own
+// row of A alone.
+#define MF_BM 128
+#define MF_BN 128
+#define MF_BK 32
+#define MF_KQ (MF_BK / 4)
+#define MF_XCDS 8  // dies of the gfx950 parts that this library is built for (a wrong count costs cache hits only)
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+__global__ void __launch_bounds__(256, 2)
+gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
+                     float* __restrict__ C, int ldc, int M, int N, int K, int tiles_m, int tiles_n) {
+  // [buffer][k / 4][row], a row more than there are so that the stores of a wave (a row's
+  // eight vectors side by side) spread over the banks
+  __shared__ float4 a_s[2][MF_KQ][MF_BM + 1];
+  __shared__ float4 w_s[2][MF_KQ][MF_BN + 1];
+  const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
+  // Workgroups go to the eight dies in turn, each die with a cache of its own: renumber them
+  // so that a die's workgroups are neighbours in the order of tiles (the same columns of W,
+  // rows of A one after the other).
+  int id = blockIdx.x;
+  const int total = tiles_m * tiles_n;
+  if (total % MF_XCDS == 0) id = (id % MF_XCDS) * (total / MF_XCDS) + id / MF_XCDS;
+  const int m0 = (id % tiles_m) * MF_BM, n0 = (id / tiles_m) * MF_BN;
+
+  float4 a_next[4], w_next[4];
+  auto ask = [&](int k0) {  // vector e of a stage: row e / 8, k0 + 4 (e % 8)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = tid + u * 256, r = e / MF_KQ, k = k0 + (e % MF_KQ) * 4;
+      const bool k_in = k < K;  // (K is a multiple of 4)
+      a_next[u] = (k_in && m0 + r < M) ? *(const float4*)(A + (size_t)(m0 + r) * lda + k) : float4{0.f, 0.f, 0.f, 0.f};
+      w_next[u] = (k_in && n0 + r < N) ? *(const float4*)(W + (size_t)(n0 + r) * ldw + k) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = tid + u * 256;
+      a_s[buf][e % MF_KQ][e / MF_KQ] = a_next[u];
+      w_s[buf][e % MF_KQ][e / MF_KQ] = w_next[u];
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  const int rows = (wave / 2) * 64 + lane % 32, cols = (wave % 2) * 64 + lane % 32, half = lane / 32;
+
+  ask(0);
+  put(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += MF_BK, buf ^= 1) {
+    const bool more = k0 + MF_BK < K;
+    if (more) ask(k0 + MF_BK);
+#pragma unroll
+    for (int s = 0; s < MF_KQ / 2; ++s) {
+      const int kq = 2 * s + half;
+      const float4 a0 = a_s[buf][kq][rows], a1 = a_s[buf][kq][rows + 32];
+      const float4 b0 = w_s[buf][kq][cols], b1 = w_s[buf][kq][cols + 32];
+      const float a0v[4] = {a0.x, a0.y, a0.z, a0.w}, a1v[4] = {a1.x, a1.y, a1.z, a1.w};
+      const float b0v[4] = {b0.x, b0.y, b0.z, b0.w}, b1v[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0v[e], b0v[e], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0v[e], b1v[e], acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1v[e], b0v[e], acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1v[e], b1v[e], acc[1][1], 0, 0, 0);
+      }
+    }
+    if (more) put(buf ^ 1);  // (read last in the stage before the one that just ended)
+    __syncthreads();
+  }
+  // element v of a lane's 16: row 8 (v / 4) + 4 (lane / 32) + v % 4, column lane % 32
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int gn = n0 + (wave % 2) * 64 + j * 32 + lane % 32;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int gm = m0 + (wave / 2) * 64 + i * 32 + 8 * (v / 4) + 4 * half + v % 4;
+        if (gm < M && gn < N) C[(size_t)gm * ldc + gn] = acc[i][j][v];
+      }
+    }
+}
+
 // ---- at most 16 rows ------------------------------------------------------------------------
-// A wave computes MB x NC outputs (MB * NC = 64).  Lane l holds the partial sums of the k's
-// 4 (l + 64 i) .. + 3, added in rising k.  Then the 64 sums of a wave are added across the
-// lanes in six halving steps (a lane keeps the half of the values that its bit picks and
-// hands the other half to its partner), after which lane l holds output l whole.
-template <int MB, int NC>
-__global__ void __launch_bounds__(256)
+// A wave computes partial sums of MB x NC outputs (MB * NC = 64).  k is cut into blocks of 256;
+// KW waves of a workgroup share a set of columns and take every KW-th block each (KW = 1: a
+// wave has its columns to itself), and inside a block lane l has the k's 4 l .. 4 l + 3.  A lane
+// adds its products up in rising k.  Then the 64 sums of a wave are added across the lanes in
+// six halving steps (a lane keeps the half of the values that its bit picks and hands the other
+// half to its partner), after which lane l holds output l of its wave's blocks, and the KW
+// waves' sums are added in rising wave number.  The order depends on KW, i.e. on the weight's
+// size, and not on the number of rows.
+//
+// Why KW: a matrix of few columns gives few workgroups (4096 columns: 128 of four waves with
+// eight columns each), and with one wave on half of the compute units, each waiting for 8 KB
+// at a time, memory is asked for too little at once (measured 1.2 TB/s on 4096 x 4096).  With
+// the k's split over the waves such a matrix gives four times the workgroups, and every wave
+// asks for its next block before it works on the one it has.
+template <int MB, int NC, int KW>
+__global__ void __launch_bounds__(256, 2)
 gemm_f32_skinny_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
                        float* __restrict__ C, int ldc, int M, int N, int K) {
   static_assert(MB * NC == HAL_WAVE, "one output per lane");
   // The rows of A go through LDS in pieces of CH k, brought by all four waves together (a
   // wave that read them itself would ask memory for as many bytes of A as of W); the next
   // piece is on its way to registers while this one is worked on.
-  constexpr int CH = 8192 / MB;                // k of a piece: 32 KB of LDS
+  constexpr int CH = 1024;                     // k of a piece: 4 KB of LDS a row
   constexpr int AV = MB * CH / 4 / 256;        // 16-byte vectors of a piece per thread
+  constexpr int BLOCK = HAL_WAVE * 4;          // k of a block
+  constexpr int NB = CH / BLOCK / KW;          // blocks of a piece per wave
+  static_assert(NB >= 1, "a piece has a block for every wave");
   __shared__ __align__(16) float a_s[MB][CH];
+  __shared__ float sums[4][HAL_WAVE];
   const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
-  const int n0 = (blockIdx.x * 4 + wave) * NC;
+  const int kw = wave % KW;  // which of the blocks, and
+  const int n0 = (blockIdx.x * (4 / KW) + wave / KW) * NC;  // which columns
   const bool have_columns = n0 < N;  // (a wave without columns still helps with A)
   const float* wrow[NC];
 #pragma unroll
@@ -103,6 +223,14 @@ gemm_f32_skinny_kernel(const float* __restrict__ A, int lda, const float* __rest
       a_next[u] = (m < M && k < K) ? *(const float4*)(A + (size_t)m * lda + k) : float4{0.f, 0.f, 0.f, 0.f};
     }
   };
+  // this wave's b-th block of the piece at k0 begins at k0 + (b * KW + kw) * BLOCK
+  float4 w_next[NC];
+  auto ask_block = [&](int k) {  // (K is a multiple of 4: a lane's four k are there or not)
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+      w_next[c] = (have_columns && k < K) ? *(const float4*)(wrow[c] + k) : float4{0.f, 0.f, 0.f, 0.f};
+  };
+  ask_block(kw * BLOCK + lane * 4);
   ask_piece(0);
   for (int k0 = 0; k0 < K; k0 += CH) {
     __syncthreads();  // the piece before is read
@@ -113,28 +241,29 @@ gemm_f32_skinny_kernel(const float* __restrict__ A, int lda, const float* __rest
     }
     if (k0 + CH < K) ask_piece(k0 + CH);
     __syncthreads();
-    if (!have_columns) continue;
-    const int k_end = k0 + CH < K ? k0 + CH : K;
-    for (int k = k0 + lane * 4; k < k_end; k += HAL_WAVE * 4) {  // K is a multiple of 4
-      float4 w[NC], a[MB];
+#pragma unroll 1  // (unrolled, the blocks' values of A would wait in registers that are not there)
+    for (int b = 0; b < NB; ++b) {
+      const int at = (b * KW + kw) * BLOCK + lane * 4;  // inside the piece
+      float4 w[NC];
 #pragma unroll
-      for (int c = 0; c < NC; ++c) w[c] = *(const float4*)(wrow[c] + k);
+      for (int c = 0; c < NC; ++c) w[c] = w_next[c];
+      // the block after this one, in this piece or the next (beyond K: zeros, never used)
+      ask_block(b + 1 < NB ? k0 + at + KW * BLOCK : k0 + CH + kw * BLOCK + lane * 4);
 #pragma unroll
-      for (int m = 0; m < MB; ++m) a[m] = *(const float4*)&a_s[m][k - k0];
-#pragma unroll
-      for (int m = 0; m < MB; ++m)
+      for (int m = 0; m < MB; ++m) {
+        const float4 a = *(const float4*)&a_s[m][at];
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
           float s = v[m * NC + c];
-          s = fmaf(a[m].x, w[c].x, s);
-          s = fmaf(a[m].y, w[c].y, s);
-          s = fmaf(a[m].z, w[c].z, s);
-          s = fmaf(a[m].w, w[c].w, s);
+          s = fmaf(a.x, w[c].x, s);
+          s = fmaf(a.y, w[c].y, s);
+          s = fmaf(a.z, w[c].z, s);
+          s = fmaf(a.w, w[c].w, s);
           v[m * NC + c] = s;
         }
+      }
     }
   }
-  if (!have_columns) return;
 #pragma unroll
   for (int half = HAL_WAVE / 2; half >= 1; half /= 2) {
     const bool upper = (lane & half) != 0;
@@ -145,8 +274,34 @@ gemm_f32_skinny_kernel(const float* __restrict__ A, int lda, const float* __rest
       v[i] = keep + __shfl_xor(give, half, HAL_WAVE);
     }
   }
+  float total = v[0];
+  if (KW > 1) {
+    sums[wave][lane] = total;
+    __syncthreads();
+    if (kw != 0) return;
+    total = sums[wave][lane];
+#pragma unroll
+    for (int j = 1; j < KW; ++j) total += sums[wave + j][lane];
+  }
   const int m = lane / NC, c = lane % NC;
-  if (m < M && n0 + c < N) C[(size_t)m * ldc + n0 + c] = v[0];
+  if (m < M && n0 + c < N) C[(size_t)m * ldc + n0 + c] = total;
+}
+
+template <int MB, int NC>
+static void launch_skinny(const float* A, int lda, const float* W, int ldw, float* C, int ldc, int M,
+                          int N, int K, hipStream_t stream) {
+  // as many waves on a set of columns as it takes for 512 workgroups or more, counted for eight
+  // columns a wave whatever NC is: the order of the additions is the same for every M
+  const int alone = (N + 31) / 32;
+  if (alone >= 512)
+    hipLaunchKernelGGL((gemm_f32_skinny_kernel<MB, NC, 1>), dim3((N + 4 * NC - 1) / (4 * NC)), dim3(256), 0,
+                       stream, A, lda, W, ldw, C, ldc, M, N, K);
+  else if (alone >= 256)
+    hipLaunchKernelGGL((gemm_f32_skinny_kernel<MB, NC, 2>), dim3((N + 2 * NC - 1) / (2 * NC)), dim3(256), 0,
+                       stream, A, lda, W, ldw, C, ldc, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_f32_skinny_kernel<MB, NC, 4>), dim3((N + NC - 1) / NC), dim3(256), 0, stream,
+                       A, lda, W, ldw, C, ldc, M, N, K);
 }
 
 extern "C" int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, float* C, int ldc,
@@ -157,13 +312,19 @@ extern "C" int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, fl
   if (M == 0) return 0;
   if (M <= 16 && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && ((uintptr_t)A % 16) == 0 &&
       ((uintptr_t)W % 16) == 0) {
-    if (M <= 8) {
-      hipLaunchKernelGGL((gemm_f32_skinny_kernel<8, 8>), dim3((N + 31) / 32), dim3(256), 0, stream, A, lda,
-                         W, ldw, C, ldc, M, N, K);
-    } else {
-      hipLaunchKernelGGL((gemm_f32_skinny_kernel<16, 4>), dim3((N + 15) / 16), dim3(256), 0, stream, A, lda,
-                         W, ldw, C, ldc, M, N, K);
-    }
+    if (M <= 8)
+      launch_skinny<8, 8>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+    else
+      launch_skinny<16, 4>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
+  if (M > GF_BM && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && ((uintptr_t)A % 16) == 0 &&
+      ((uintptr_t)W % 16) == 0) {
+    const long long tiles_m = (M + MF_BM - 1) / MF_BM, tiles_n = (N + MF_BN - 1) / MF_BN;
+    HAL_REQUIRE(tiles_m * tiles_n < (1ll << 31), "hal_gemm_f32: M=%d N=%d exceed the grid limit", M, N);
+    hipLaunchKernelGGL(gemm_f32_mfma_kernel, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), 0, stream, A, lda,
+                       W, ldw, C, ldc, M, N, K, (int)tiles_m, (int)tiles_n);
     HAL_LAUNCH_CHECK();
     return 0;
   }

@@ -590,7 +590,11 @@ def test_attention_mfma_hundred_thousand_keys(gpu, tiled):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 256, 64), (5, 331, 120), (8, 257, 1000), (9, 130, 36), (16, 1000, 352), (17, 96, 64),
-                                   (64, 200, 352), (130, 96, 1000), (3, 4096, 4096), (2, 50, 30)])
+                                   (64, 200, 352), (130, 96, 1000), (3, 4096, 4096), (2, 50, 30),
+                                   # columns enough for two waves, and for one, on a set of columns
+                                   (7, 8200, 2308), (13, 9001, 260), (4, 16400, 1028), (16, 17003, 520),
+                                   # many rows: tiles of the matrix cores, whole and in part; a k that is no multiple of 4
+                                   (65, 128, 32), (300, 517, 2052), (1024, 260, 1028), (129, 129, 36), (200, 96, 1001)])
 def test_gemm_f32(gpu, M, N, K):
     a, w = rnd(M, K, seed=50), rnd(N, K, seed=51)
     want = (a.double() @ w.double().T).float()
@@ -607,6 +611,22 @@ def test_gemm_f32(gpu, M, N, K):
     if M <= 16:
         assert torch.equal(alone.cpu(), whole[:1].cpu())
     close(alone, whole[:1], 2e-6, "a row alone and in a larger batch")
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 512, 4096), (16, 512, 14336), (48, 512, 4096), (2048, 384, 4096), (1500, 256, 14336)])
+def test_gemm_f32_with_rows_as_long_as_the_models(gpu, M, N, K):
+    """Every kernel of the 32-bit product against the product in 64-bit, at the row lengths
+    of the 8B shape.  One row of W is made of ones and A's entries are positive there, so
+    that a kernel which dropped or doubled a stretch of k would show in a sum without
+    cancellation."""
+    a, w = rnd(M, K, seed=53), rnd(N, K, seed=54)
+    w[5] = 1.0
+    a[3] = a[3].abs()
+    want = (a.double() @ w.double().T).float()
+    got = ops.gemm_f32(a.to(gpu), w.to(gpu)).cpu()
+    close(got, want, 3e-6, "gemm_f32")
+    exact = float(a[3].double().sum())
+    assert abs(float(got[3, 5]) - exact) <= 2e-6 * exact
 
 
 @pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 48, 64])
