@@ -36,17 +36,18 @@ int hal_rope_append(void* qkv, int dtype, int row_stride, const int* positions,
                     void* v_pages, int n_tokens, int H, int K, int D, int rot, int interleaved,
                     int page_size, int n_pages, int tiled, hipStream_t stream);
 
-// `max_kv_len`: no request of the step has more keys (an upper bound will do).
-// `hal_attention_simple_plan` says how the step is cut; if `split`, `part` must bring
-// `part_floats` floats for the pieces' partial sums.
-int hal_attention_simple_plan(int n_tokens, int H, int K, int D, int max_kv_len, int* tq, int* split,
-                              int* rows_per_wave, int* max_pieces, long long* part_floats);
+// `max_kv_len`: no request of the step has more keys (an upper bound will do); `min_q_len`:
+// none has fewer tokens in the step (a lower bound will do, 1 if not known).  They decide how
+// the step is cut, never a result.  `hal_attention_simple_plan` says how; if `split`, `part`
+// must bring `part_floats` floats for the pieces' partial sums.
+int hal_attention_simple_plan(int n_tokens, int H, int K, int D, int max_kv_len, int min_q_len, int* tq,
+                              int* split, int* rows_per_wave, int* max_pieces, long long* part_floats);
 int hal_attention_simple(const void* q, int q_row_stride, void* out, int out_row_stride,
                          int dtype, const int* positions, const int* token_seg,
                          const int* block_table, int bt_stride, const void* k_pages,
                          const void* v_pages, float* part, int n_tokens, int H, int K, int D,
                          int page_size, int n_pages, float scale, int window, int max_kv_len,
-                         hipStream_t stream);
+                         int min_q_len, hipStream_t stream);
 
 int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, float* C, int ldc, int M,
                  int N, int K, hipStream_t stream);

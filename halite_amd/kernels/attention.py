@@ -437,8 +437,10 @@ def paged_attention(ctx, q, q_row_stride, kv, group, n_heads, scale, window):
             f"(dtype {q.dtype}, head size {head_dim}, page size {page_size}, row stride {q_row_stride})"
         )
     # (a step whose launches are recorded serves other lengths later: the block table's width bounds them)
-    most = None if ctx.static is not None or not len(ctx.seg_kv_len_host) else int(ctx.seg_kv_len_host.max())
+    known = ctx.static is None and len(ctx.seg_kv_len_host) > 0
+    most = int(ctx.seg_kv_len_host.max()) if known else None
+    fewest = int(ctx.seg_q_len_host.min()) if known else 1
     return ops.attention_simple(
         q, q_row_stride, ctx.positions, ctx.token_seg, group.block_table, kv.k, kv.v, n_heads, scale, window,
-        max_kv_len=most,
+        max_kv_len=most, min_q_len=fewest,
     )

@@ -327,11 +327,13 @@ def attention_simple(
     scale: float,
     window: int = 0,
     max_kv_len: int | None = None,
+    min_q_len: int = 1,
 ):
     """Paged attention in float32 arithmetic; ``q`` holds the query heads at the start of
     rows of ``q_row_stride`` elements.  ``max_kv_len``: the most keys that a request of the
-    step has (what the block table could hold if it is not given); it decides how the step
-    is cut into workgroups, never a result."""
+    step has (what the block table could hold if it is not given); ``min_q_len``: the fewest
+    tokens that a request has in the step (1 if not known: steps of prompts alone go to the
+    matrix cores).  They decide how the step is cut into workgroups, never a result."""
     lib = library.core_library()
     _dev(q, positions, token_seg, block_table, k_pages, v_pages)
     _i32(positions, "positions"), _i32(token_seg, "token_seg"), _i32(block_table, "block_table")
@@ -344,8 +346,9 @@ def attention_simple(
     if max_kv_len is None:
         max_kv_len = block_table.shape[1] * page_size
     tq, split, rows, pieces, floats = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_longlong()
-    _check(lib, lib.hal_attention_simple_plan(n, n_heads, n_kv, head_dim, max_kv_len, ctypes.byref(tq), ctypes.byref(split),
-                                              ctypes.byref(rows), ctypes.byref(pieces), ctypes.byref(floats)))
+    _check(lib, lib.hal_attention_simple_plan(n, n_heads, n_kv, head_dim, max_kv_len, min_q_len, ctypes.byref(tq),
+                                              ctypes.byref(split), ctypes.byref(rows), ctypes.byref(pieces),
+                                              ctypes.byref(floats)))
     part = torch.empty(floats.value, dtype=torch.float32, device=q.device) if floats.value else None
     _check(
         lib,
@@ -353,7 +356,7 @@ def attention_simple(
             _ptr(q), q_row_stride, _ptr(out), n_heads * head_dim, dtype_code(q.dtype),
             _ptr(positions), _ptr(token_seg), _ptr(block_table), block_table.shape[1],
             _ptr(k_pages), _ptr(v_pages), _ptr(part), n, n_heads, n_kv, head_dim, page_size, n_pages,
-            ctypes.c_float(scale), window, max_kv_len, _stream(),
+            ctypes.c_float(scale), window, max_kv_len, min_q_len, _stream(),
         ),
     )
     return out

@@ -380,8 +380,13 @@ def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use, tiled=Fal
     q = torch.cat(qs).to(dt).to(gpu)
     positions = torch.cat(pos).to(torch.int32).to(gpu)
     token_seg = torch.cat(seg_of).to(torch.int32).to(gpu)
-    if use == "simple":
-        out = ops.attention_simple(q, H * D, positions, token_seg, bt.to(gpu), k_pages, v_pages, H, scale, window)
+    if use in ("simple", "rows"):
+        # as the engine calls it: the fewest tokens of a request decide between the kernel of
+        # the vector units and, for steps of prompts alone, the one of the matrix cores;
+        # "rows" claims many tokens whatever the step holds, which is wrong and must cost time only
+        fewest = 10**6 if use == "rows" else min(new for _, new in segs)
+        out = ops.attention_simple(q, H * D, positions, token_seg, bt.to(gpu), k_pages, v_pages, H, scale, window,
+                                   max_kv_len=max(b + n for b, n in segs), min_q_len=fewest)
     else:
         q_len = np.array([n for _, n in segs], dtype=np.int32)
         kv_len = np.array([b + n for b, n in segs], dtype=np.int32)
@@ -406,14 +411,26 @@ def attention_case(gpu, dtype, H, K, D, page, segs, window, seed, use, tiled=Fal
 
 SHAPES = [(4, 2, 16), (6, 2, 48), (4, 1, 32), (8, 8, 64), (32, 8, 128), (5, 5, 80), (20, 1, 16), (4, 2, 256), (6, 3, 112), (2, 1, 160)]
 SEGS = [[(0, 1)], [(0, 70)], [(63, 1), (0, 33), (64, 64), (129, 2), (200, 1)], [(700, 1), (5, 300)]]
+PROMPTS = [[(0, 200)], [(37, 130), (0, 64), (500, 90)], [(0, 9), (100, 8), (31, 33)], [(1000, 129)]]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("segs", SEGS)
+@pytest.mark.parametrize("segs", SEGS + PROMPTS[:2])
 @pytest.mark.parametrize("H,K,D", SHAPES[:5])
 def test_attention_simple(gpu, dtype, H, K, D, segs):
     for page, window in ((1, 0), (4, 0), (16, 0), (64, 0), (16, 37), (4, 1)):
         attention_case(gpu, dtype, H, K, D, page, segs, window, seed=20, use="simple")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("segs", SEGS + PROMPTS)
+@pytest.mark.parametrize("H,K,D", SHAPES[:7] + [(7, 1, 24), (3, 3, 128), (256, 1, 8)])
+def test_attention_of_many_rows_a_request(gpu, dtype, H, K, D, segs):
+    """The 32-bit kernel on the matrix cores, which steps of prompts alone take: every head
+    size it serves (multiples of 8 up to 128), groups that fill a wave's 32 rows unevenly or
+    are more than a workgroup's 128, and steps that it would not be given (single tokens)."""
+    for page, window in ((1, 0), (4, 0), (16, 0), (64, 0), (16, 37), (4, 1), (8, 70)):
+        attention_case(gpu, dtype, H, K, D, page, segs, window, seed=25, use="rows")
 
 
 @pytest.mark.parametrize("segs", SEGS)
