@@ -1,7 +1,9 @@
-// Paged attention, the plain way: float32 arithmetic on the vector units throughout, any
-// head size that is a multiple of 4 up to 512, any page size, any number of heads and
-// groups, float32 or bf16 storage.  It is the whole attention of the 32-bit path and the
-// fallback of the bf16 path for shapes that the matrix-core kernel refuses.
+// Paged attention in float32 arithmetic throughout: any head size that is a multiple of 4 up
+// to 512, any page size, any number of heads and groups, float32 or bf16 storage.  It is the
+// whole attention of the 32-bit path and the fallback of the bf16 path for shapes that the
+// bf16 matrix-core kernel refuses.  Two kernels: the plain one on the vector units, described
+// first, which serves every step, and further down one on the matrix cores' float32
+// instruction for steps in which every request brings many tokens (prompts).
 //
 // A workgroup of four waves serves up to 16 rows that share their keys: a few neighbouring
 // tokens of one request times the query heads of one key/value head, so the keys and values
