@@ -13,15 +13,17 @@
 // block's loads are in flight while this one is worked on), then wave w takes the rows w,
 // w + 4, ...: a lane is a key for the scores and a dimension for the weighted sum.
 //
-// A row's keys are summed in pieces of 512: a piece starts from nothing, and the pieces'
-// sums are joined in the order of the keys by the log-sum-exp rule.  Where a step has few
-// rows (decoding) every piece is a workgroup of its own and a second kernel joins them;
+// A row's keys are summed in pieces of 512 (of 256 or 128 where a step has so few rows and
+// keys that pieces of 512 would leave the chip empty): a piece starts from nothing, and the
+// pieces' sums are joined in the order of the keys by the log-sum-exp rule.  Where a step has
+// few rows (decoding) every piece is a workgroup of its own and a second kernel joins them;
 // where it has many, one workgroup walks all of a row's pieces and joins as it goes.  Both
 // do the same arithmetic in the same order, and every sum over keys is cut at fixed
 // multiples counted from the request's first key, so a row's result depends on the row's
-// own position, window and request alone, not on what else the step holds.  (The kernel
-// has two builds, blocks of 32 keys for steps of few tokens and of 64 for the others: the
-// same row differs between them by rounding.)
+// own position, window and request alone, not on what else the step holds.  (Between steps
+// that are cut differently the same row differs by rounding: the kernel has two builds,
+// blocks of 32 keys for steps of few tokens and of 64 for the others, and the size of the
+// pieces follows the size of the step.)
 //
 // scores, mask, softmax and weighted sum as in
 // src/halite/transformers/attention.py:647-714; the causal rule for a portion that
@@ -32,7 +34,8 @@
 
 #define PLAIN_THREADS 256
 #define PLAIN_WAVES 4
-#define PLAIN_PIECE 512     // keys of a piece
+#define PLAIN_PIECE_SHIFT 9  // a piece has 512 keys,
+#define PLAIN_PIECE_LEAST 7  // or 256 or 128 where pieces are workgroups of their own and that many fit
 #define PLAIN_PAD 4         // floats between two rows of a tile: 16-byte rows, no bank conflicts
 
 // LDS that one lane of a wave writes and another reads: the wave's LDS operations are done
@@ -91,6 +94,15 @@ __device__ __forceinline__ void plain_join_weights(float M, float m, float& M_ne
 }
 __device__ __forceinline__ float plain_join(float A, float w_old, float a, float w_new) {
   return __fadd_rn(__fmul_rn(A, w_old), __fmul_rn(a, w_new));
+}
+
+// The pieces of a row whose keys are lo .. p, where every piece is a workgroup of its own and
+// a row has room for `slots` of them: the smallest pieces that fit (so that a short range
+// still spreads over the chip), cut at multiples of their size counted from key 0.
+__device__ __forceinline__ int plain_piece_shift(int lo, int p, int slots) {
+  int s = PLAIN_PIECE_LEAST;
+  while (s < PLAIN_PIECE_SHIFT && (p >> s) - (lo >> s) + 1 > slots) ++s;
+  return s;
 }
 
 static inline size_t plain_lds_floats(int D, int keys, int rows) {
@@ -247,9 +259,12 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
     const int n_rows = (tb - ta) * heads_here;
     // the keys this workgroup walks for the run
     int j_begin = lo_min / KEYS * KEYS, j_end = p_max + 1;
+    // (pieces as workgroups: a token a workgroup, so the run's range is the range of its rows)
+    const int piece_shift = split ? plain_piece_shift(lo_min, p_max, max_pieces) : PLAIN_PIECE_SHIFT;
     if (split) {
-      j_begin = max(j_begin, (int)blockIdx.z * PLAIN_PIECE);
-      j_end = min(j_end, ((int)blockIdx.z + 1) * PLAIN_PIECE);
+      const int pc = (lo_min >> piece_shift) + (int)blockIdx.z;
+      j_begin = max(j_begin, pc << piece_shift);
+      j_end = min(j_end, (pc + 1) << piece_shift);
     }
     if (j_begin >= j_end) {  // (the same for every thread)
       ta = tb;
@@ -304,7 +319,7 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
       if (j0 + KEYS < j_end) tiles.fetch(buf ^ 1);
       tiles.ask_place(j0 + 3 * KEYS);
       __syncthreads();
-      const bool piece_ends = (j0 + KEYS) % PLAIN_PIECE == 0 || j0 + KEYS >= j_end;
+      const bool piece_ends = ((j0 + KEYS) & ((1 << piece_shift) - 1)) == 0 || j0 + KEYS >= j_end;
 #pragma unroll
       for (int rr = 0; rr < RW; ++rr) {
         const int r = wave + PLAIN_WAVES * rr;
@@ -373,11 +388,11 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
         if (have_row && piece_ends) {
           // Only pieces that hold keys of the row count (the others would join as nothing,
           // but where pieces are workgroups of their own nobody computes them).
-          const int pc = j0 / PLAIN_PIECE;
-          const bool mine = pc >= lo / PLAIN_PIECE && pc <= p / PLAIN_PIECE;
-          const bool only_piece = lo / PLAIN_PIECE == p / PLAIN_PIECE;
+          const int pc = j0 >> piece_shift;
+          const bool mine = pc >= (lo >> piece_shift) && pc <= (p >> piece_shift);
+          const bool only_piece = (lo >> piece_shift) == (p >> piece_shift);
           if (mine && split && !only_piece) {
-            float* dst = part + (((size_t)(ta + r / heads_here) * H + h_first + r % heads_here) * max_pieces + pc) * (D + 2);
+            float* dst = part + (((size_t)(ta + r / heads_here) * H + h_first + r % heads_here) * max_pieces + blockIdx.z) * (D + 2);
 #pragma unroll
             for (int c = 0; c < R; ++c) {
               const int d = lane + c * HAL_WAVE;
@@ -408,8 +423,8 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
     for (int rr = 0; rr < RW; ++rr) {
       const int r = wave + PLAIN_WAVES * rr;
       const int p = row_p[rr], lo = row_lo[rr];
-      const bool only_piece = lo / PLAIN_PIECE == p / PLAIN_PIECE;
-      if (r >= n_rows || (split && !(only_piece && (int)blockIdx.z == p / PLAIN_PIECE))) continue;
+      const bool only_piece = (lo >> piece_shift) == (p >> piece_shift);
+      if (r >= n_rows || (split && !(only_piece && blockIdx.z == 0))) continue;
       T* op = out + (size_t)(ta + r / heads_here) * out_row_stride + (size_t)(h_first + r % heads_here) * D;
       const float inv = 1.0f / L[rr];
 #pragma unroll
@@ -431,21 +446,37 @@ attention_plain_merge_kernel(T* __restrict__ out, int out_row_stride, const int*
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int p = positions[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-  const int first = lo / PLAIN_PIECE, last = p / PLAIN_PIECE;
+  const int piece_shift = plain_piece_shift(lo, p, max_pieces);
+  const int first = lo >> piece_shift, last = p >> piece_shift;
   if (first == last) return;  // written by the piece's own workgroup
   float M = -INFINITY, L = 0.f, A[R];
 #pragma unroll
   for (int c = 0; c < R; ++c) A[c] = 0.f;
-  for (int pc = first; pc <= last; ++pc) {
-    const float* src = part + (((size_t)t * H + h) * max_pieces + pc) * (D + 2);
-    float M_new, w_old, w_new;
-    plain_join_weights(M, src[D], M_new, w_old, w_new);
-    L = plain_join(L, w_old, src[D + 1], w_new);
-    M = M_new;
+  // eight pieces are asked for at once (the joins wait for each other, the loads need not)
+  constexpr int AHEAD = 8;
+  const float* row = part + ((size_t)t * H + h) * max_pieces * (D + 2);
+  for (int base = first; base <= last; base += AHEAD) {
+    float mm[AHEAD], ll[AHEAD], aa[AHEAD][R];
 #pragma unroll
-    for (int c = 0; c < R; ++c) {
-      const int d = lane + c * HAL_WAVE;
-      if (d < D) A[c] = plain_join(A[c], w_old, src[d], w_new);
+    for (int u = 0; u < AHEAD; ++u) {
+      const float* src = row + (size_t)(min(base + u, last) - first) * (D + 2);
+      mm[u] = src[D];
+      ll[u] = src[D + 1];
+#pragma unroll
+      for (int c = 0; c < R; ++c) {
+        const int d = lane + c * HAL_WAVE;
+        aa[u][c] = d < D ? src[d] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      if (base + u > last) break;
+      float M_new, w_old, w_new;
+      plain_join_weights(M, mm[u], M_new, w_old, w_new);
+      L = plain_join(L, w_old, ll[u], w_new);
+      M = M_new;
+#pragma unroll
+      for (int c = 0; c < R; ++c) A[c] = plain_join(A[c], w_old, aa[u][c], w_new);
     }
   }
   T* op = out + (size_t)t * out_row_stride + (size_t)h * D;
@@ -692,9 +723,18 @@ extern "C" int hal_attention_simple_plan(int n_tokens, int H, int K, int D, int 
   const int chunks = (G + rows_most - 1) / rows_most;
   int together = G >= rows_most ? 1 : rows_most / G;  // tokens whose rows fill a workgroup
   const long long groups = ((long long)n_tokens + together - 1) / together * K * chunks;
-  const int pieces = max(1, (max_kv_len + PLAIN_PIECE - 1) / PLAIN_PIECE);
-  // few workgroups: a token each, and a piece each
-  *split = (groups < 512 && pieces > 1) ? 1 : 0;
+  // Few workgroups: a token each, and a piece each.  A workgroup's walk waits for memory block
+  // after block (4 us a block of 32 keys where it has a compute unit to itself), so a row gets
+  // as many slots for pieces as it takes for 1024 workgroups (at most 64, and no more than
+  // pieces of 128 keys could fill), and the kernel cuts each row's own range into the smallest
+  // pieces that fit its slots.  Pieces of 512 keys always fit (one more where a window's range
+  // begins inside a piece).
+  const int whole = (max_kv_len + (1 << PLAIN_PIECE_SHIFT) - 1) / (1 << PLAIN_PIECE_SHIFT) + 1;
+  const int least = (max_kv_len + (1 << PLAIN_PIECE_LEAST) - 1) / (1 << PLAIN_PIECE_LEAST) + 1;
+  const long long alone = (long long)n_tokens * K * ((G + PLAIN_WAVES - 1) / PLAIN_WAVES);  // groups of a token each
+  const int wanted = alone > 0 ? (int)min((1024 + alone - 1) / alone, (long long)64) : 1;
+  const int pieces = max(whole, min(wanted, least));
+  *split = (groups < 512 && max_kv_len > (1 << PLAIN_PIECE_LEAST)) ? 1 : 0;
   *tq = *split ? 1 : together;
   // a token whose heads are at most four: a row a wave
   *rows_per_wave = (*tq == 1 && G <= PLAIN_WAVES) || D > 256 ? 1 : 4;

@@ -423,6 +423,17 @@ def test_attention_simple(gpu, dtype, H, K, D, segs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("segs", [[(2000, 1), (900, 1), (40, 1), (1199, 2), (383, 1)], [(1300, 1)], [(255, 1), (256, 1), (127, 2)]])
+@pytest.mark.parametrize("H,K,D", SHAPES[:5] + [(20, 1, 16), (4, 2, 256), (2, 1, 320)])
+def test_attention_simple_pieces_of_decode_tokens(gpu, dtype, H, K, D, segs):
+    """Steps of few tokens: every piece of a row's keys is a workgroup of its own and a second
+    kernel joins them; the fewer the rows, the smaller the pieces (512, 256 or 128 keys).  With
+    windows that begin inside a piece, and pages smaller and larger than a block."""
+    for page, window in ((1, 0), (16, 0), (64, 0), (16, 300), (4, 37), (64, 130)):
+        attention_case(gpu, dtype, H, K, D, page, segs, window, seed=27, use="simple")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("segs", SEGS + PROMPTS)
 @pytest.mark.parametrize("H,K,D", SHAPES[:7] + [(7, 1, 24), (3, 3, 128), (256, 1, 8)])
 def test_attention_of_many_rows_a_request(gpu, dtype, H, K, D, segs):
