@@ -6,10 +6,9 @@
 // Three kernels.  At most 16 rows (decode steps): a wave takes a few columns of the output,
 // its lanes take every 64th group of four k each (the rows of A come through LDS, shared by
 // the workgroup's four waves), and the partial sums of the lanes, and of the waves that share
-// columns, are added in a fixed order.  More than 64 rows (prompts): tiles of 128 x 128 on the
-// matrix cores.  Between them, and for sizes and addresses that are no multiples of four:
-// tiles of 64 x 64 on the vector units, each output element one chain of K multiply-adds in
-// index order.
+// columns, are added in a fixed order.  More rows: tiles of 128 rows and 128 or 32 columns on
+// the matrix cores.  For sizes and addresses that are no multiples of four: tiles of 64 x 64
+// on the vector units, each output element one chain of K multiply-adds in index order.
 // In all three a token's result depends on its own row alone, not on what else is in the
 // batch; between them the order of the additions differs, i.e. the last bits may.
 #include "hal_common.h"
@@ -92,13 +91,20 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
 #define MF_XCDS 8  // dies of the gfx950 parts that this library is built for (a wrong count costs cache hits only)
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
+// BN: columns of a workgroup's tile, 128 (a wave takes 64 x 64 as 2 x 2 products) or 32 (a wave
+// takes 32 x 32): the narrow tile is for products of so few rows and columns that tiles of 128
+// columns would leave most of the chip empty.  An output element's sum is the same in both.
+template <int BN>
 __global__ void __launch_bounds__(256, 2)
 gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
                      float* __restrict__ C, int ldc, int M, int N, int K, int tiles_m, int tiles_n) {
+  constexpr int NB = BN == 128 ? 2 : 1;     // 32 x 32 products of a wave, each way
+  constexpr int WV = BN * MF_KQ / 256;      // 16-byte vectors of W's stage per thread
+  static_assert(BN == 128 || BN == 32, "tiles of 128 or 32 columns");
   // [buffer][k / 4][row], a row more than there are so that the stores of a wave (a row's
   // eight vectors side by side) spread over the banks
   __shared__ float4 a_s[2][MF_KQ][MF_BM + 1];
-  __shared__ float4 w_s[2][MF_KQ][MF_BN + 1];
+  __shared__ float4 w_s[2][MF_KQ][BN + 1];
   const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
   // Workgroups go to the eight dies in turn, each die with a cache of its own: renumber them
   // so that a die's workgroups are neighbours in the order of tiles (the same columns of W,
@@ -106,16 +112,21 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restri
   int id = blockIdx.x;
   const int total = tiles_m * tiles_n;
   if (total % MF_XCDS == 0) id = (id % MF_XCDS) * (total / MF_XCDS) + id / MF_XCDS;
-  const int m0 = (id % tiles_m) * MF_BM, n0 = (id / tiles_m) * MF_BN;
+  const int m0 = (id % tiles_m) * MF_BM, n0 = (id / tiles_m) * BN;
 
-  float4 a_next[4], w_next[4];
+  float4 a_next[4], w_next[WV];
   auto ask = [&](int k0) {  // vector e of a stage: row e / 8, k0 + 4 (e % 8)
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int e = tid + u * 256, r = e / MF_KQ, k = k0 + (e % MF_KQ) * 4;
-      const bool k_in = k < K;  // (K is a multiple of 4)
-      a_next[u] = (k_in && m0 + r < M) ? *(const float4*)(A + (size_t)(m0 + r) * lda + k) : float4{0.f, 0.f, 0.f, 0.f};
-      w_next[u] = (k_in && n0 + r < N) ? *(const float4*)(W + (size_t)(n0 + r) * ldw + k) : float4{0.f, 0.f, 0.f, 0.f};
+      const bool in = k < K && m0 + r < M;  // (K is a multiple of 4)
+      a_next[u] = in ? *(const float4*)(A + (size_t)(m0 + r) * lda + k) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < WV; ++u) {
+      const int e = tid + u * 256, r = e / MF_KQ, k = k0 + (e % MF_KQ) * 4;
+      const bool in = k < K && n0 + r < N;
+      w_next[u] = in ? *(const float4*)(W + (size_t)(n0 + r) * ldw + k) : float4{0.f, 0.f, 0.f, 0.f};
     }
   };
   auto put = [&](int buf) {
@@ -123,18 +134,25 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restri
     for (int u = 0; u < 4; ++u) {
       const int e = tid + u * 256;
       a_s[buf][e % MF_KQ][e / MF_KQ] = a_next[u];
+    }
+#pragma unroll
+    for (int u = 0; u < WV; ++u) {
+      const int e = tid + u * 256;
       w_s[buf][e % MF_KQ][e / MF_KQ] = w_next[u];
     }
   };
 
-  f32x16 acc[2][2];
+  f32x16 acc[NB][NB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NB; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-  const int rows = (wave / 2) * 64 + lane % 32, cols = (wave % 2) * 64 + lane % 32, half = lane / 32;
+  // this wave's corner of the tile
+  const int wm = BN == 128 ? (wave / 2) * 64 : wave * 32, wn = BN == 128 ? (wave % 2) * 64 : 0;
+  const int rows = wm + lane % 32, cols = wn + lane % 32, half = lane / 32;
+  const bool wave_has_rows = m0 + wm < M;  // (a wave whose rows are all beyond M only helps to load)
 
   ask(0);
   put(0);
@@ -143,19 +161,24 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restri
   for (int k0 = 0; k0 < K; k0 += MF_BK, buf ^= 1) {
     const bool more = k0 + MF_BK < K;
     if (more) ask(k0 + MF_BK);
+    if (wave_has_rows) {
 #pragma unroll
-    for (int s = 0; s < MF_KQ / 2; ++s) {
-      const int kq = 2 * s + half;
-      const float4 a0 = a_s[buf][kq][rows], a1 = a_s[buf][kq][rows + 32];
-      const float4 b0 = w_s[buf][kq][cols], b1 = w_s[buf][kq][cols + 32];
-      const float a0v[4] = {a0.x, a0.y, a0.z, a0.w}, a1v[4] = {a1.x, a1.y, a1.z, a1.w};
-      const float b0v[4] = {b0.x, b0.y, b0.z, b0.w}, b1v[4] = {b1.x, b1.y, b1.z, b1.w};
+      for (int s = 0; s < MF_KQ / 2; ++s) {
+        const int kq = 2 * s + half;
+        float av[NB][4], bv[NB][4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0v[e], b0v[e], acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0v[e], b1v[e], acc[0][1], 0, 0, 0);
-        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1v[e], b0v[e], acc[1][0], 0, 0, 0);
-        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1v[e], b1v[e], acc[1][1], 0, 0, 0);
+        for (int i = 0; i < NB; ++i) {
+          const float4 a = a_s[buf][kq][rows + 32 * i], b = w_s[buf][kq][cols + 32 * i];
+          av[i][0] = a.x, av[i][1] = a.y, av[i][2] = a.z, av[i][3] = a.w;
+          bv[i][0] = b.x, bv[i][1] = b.y, bv[i][2] = b.z, bv[i][3] = b.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+          for (int i = 0; i < NB; ++i)
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i][e], bv[j][e], acc[i][j], 0, 0, 0);
       }
     }
     if (more) put(buf ^ 1);  // (read last in the stage before the one that just ended)
@@ -163,13 +186,13 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restri
   }
   // element v of a lane's 16: row 8 (v / 4) + 4 (lane / 32) + v % 4, column lane % 32
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NB; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int gn = n0 + (wave % 2) * 64 + j * 32 + lane % 32;
+    for (int j = 0; j < NB; ++j) {
+      const int gn = n0 + wn + j * 32 + lane % 32;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int gm = m0 + (wave / 2) * 64 + i * 32 + 8 * (v / 4) + 4 * half + v % 4;
+        const int gm = m0 + wm + i * 32 + 8 * (v / 4) + 4 * half + v % 4;
         if (gm < M && gn < N) C[(size_t)gm * ldc + gn] = acc[i][j][v];
       }
     }
@@ -319,12 +342,18 @@ extern "C" int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, fl
     HAL_LAUNCH_CHECK();
     return 0;
   }
-  if (M > GF_BM && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && ((uintptr_t)A % 16) == 0 &&
-      ((uintptr_t)W % 16) == 0) {
-    const long long tiles_m = (M + MF_BM - 1) / MF_BM, tiles_n = (N + MF_BN - 1) / MF_BN;
+  if (K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0) {
+    // more than 16 rows: the matrix cores, in tiles of 128 columns where those fill the chip
+    const long long tiles_m = (M + MF_BM - 1) / MF_BM, wide = (N + 127) / 128, narrow = (N + 31) / 32;
+    const bool use_wide = tiles_m * wide >= 256;
+    const long long tiles_n = use_wide ? wide : narrow;
     HAL_REQUIRE(tiles_m * tiles_n < (1ll << 31), "hal_gemm_f32: M=%d N=%d exceed the grid limit", M, N);
-    hipLaunchKernelGGL(gemm_f32_mfma_kernel, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), 0, stream, A, lda,
-                       W, ldw, C, ldc, M, N, K, (int)tiles_m, (int)tiles_n);
+    if (use_wide)
+      hipLaunchKernelGGL(gemm_f32_mfma_kernel<128>, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), 0, stream, A,
+                         lda, W, ldw, C, ldc, M, N, K, (int)tiles_m, (int)tiles_n);
+    else
+      hipLaunchKernelGGL(gemm_f32_mfma_kernel<32>, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), 0, stream, A,
+                         lda, W, ldw, C, ldc, M, N, K, (int)tiles_m, (int)tiles_n);
     HAL_LAUNCH_CHECK();
     return 0;
   }
