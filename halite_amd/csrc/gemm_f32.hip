@@ -3,13 +3,15 @@
 // of a bias-free linear layer's weight ([out, in], src/halite/transformers/feedforward.py:
 // 204-212; src/halite/transformers/infer/attention.py:21-24).
 //
-// Three kernels.  At most 16 rows (decode steps): a wave takes a few columns of the output,
+// Four kernels.  At most 16 rows (decode steps): a wave takes a few columns of the output,
 // its lanes take every 64th group of four k each (the rows of A come through LDS, shared by
 // the workgroup's four waves), and the partial sums of the lanes, and of the waves that share
-// columns, are added in a fixed order.  More rows: tiles of 128 rows and 128 or 32 columns on
-// the matrix cores.  For sizes and addresses that are no multiples of four: tiles of 64 x 64
-// on the vector units, each output element one chain of K multiply-adds in index order.
-// In all three a token's result depends on its own row alone, not on what else is in the
+// columns, are added in a fixed order.  17 to 64 rows: the matrix cores fed straight from
+// memory, k split over a workgroup's waves.  More rows: tiles of 128 rows and 128 or 32
+// columns on the matrix cores, through LDS.  For sizes and addresses that are no multiples of
+// four: tiles of 64 x 64 on the vector units, each output element one chain of K
+// multiply-adds in index order.
+// In all of them a token's result depends on its own row alone, not on what else is in the
 // batch; between them the order of the additions differs, i.e. the last bits may.
 #include "hal_common.h"
 #include "hal_api.h"
@@ -198,6 +200,101 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restri
     }
 }
 
+// ---- 17 to 64 rows: the same instruction, fed from memory -----------------------------------
+// Too many rows for the vector units' kernel below, too few for tiles to fill the chip: what
+// counts is that W streams.  A workgroup takes 32 columns (rows of W) and all rows of A; its
+// waves split k into stretches, one each, and every wave feeds the matrix cores straight from
+// memory: lane l brings 64 bytes of row l % 32 of W (which half of the 128 bytes of a stage:
+// l / 32) and the same of its rows of A, DEPTH stages ahead of the products, with no LDS and no
+// barrier on the way.  W is the first operand, so a lane ends with one row of A and sixteen
+// columns; the waves' sums meet in LDS and are added in rising wave number.
+// MB: blocks of 32 rows of A (M <= 32 MB; built for 1 and 2); WAVES: 4 or 8 (more where few columns leave
+// compute units idle).  An output element's sum depends on K and on WAVES, i.e. on the
+// matrix, and not on the rows beside it.
+template <int MB, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
+gemm_f32_rows_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
+                     float* __restrict__ C, int ldc, int M, int N, int K) {
+  constexpr int DEPTH = MB == 1 ? 4 : 3;  // stages in registers
+  __shared__ float sums[WAVES][32][33];  // [wave][row of A in a block][column], padded
+  const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
+  const int col = lane % 32, half = lane / 32;
+  const int n0 = blockIdx.x * 32;
+  // this wave's stretch of k: whole stages of 32
+  const int stages = (K + 31) / 32, each = (stages + WAVES - 1) / WAVES;
+  const int k_begin = wave * each * 32, k_end = min(K, (wave + 1) * each * 32);
+  const bool w_in = n0 + col < N;
+  const float* wp = W + (size_t)(w_in ? n0 + col : 0) * ldw + 16 * half;
+  const float* ap[MB];
+  bool a_in[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    a_in[b] = 32 * b + col < M;
+    ap[b] = A + (size_t)(a_in[b] ? 32 * b + col : 0) * lda + 16 * half;
+  }
+  float4 wr[DEPTH][4], ar[DEPTH][MB][4];
+  auto ask = [&](int d, int k) {  // (K is a multiple of 4: a vector is inside or outside)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool k_in = k + 16 * half + 4 * j < k_end;
+      wr[d][j] = (k_in && w_in) ? *(const float4*)(wp + k + 4 * j) : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int b = 0; b < MB; ++b)
+        ar[d][b][j] = (k_in && a_in[b]) ? *(const float4*)(ap[b] + k + 4 * j) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  f32x16 acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) ask(d, k_begin + 32 * d);
+  for (int k = k_begin; k < k_end; k += 32 * DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {  // (stages beyond the stretch hold zeros)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float wv[4] = {wr[d][j].x, wr[d][j].y, wr[d][j].z, wr[d][j].w};
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+          const float av[4] = {ar[d][b][j].x, ar[d][b][j].y, ar[d][b][j].z, ar[d][b][j].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[e], av[e], acc[b], 0, 0, 0);
+        }
+      }
+      ask(d, k + 32 * (d + DEPTH));  // (the other stages are on their way meanwhile)
+    }
+  }
+  // element v of a lane's 16: column 8 (v / 4) + 4 half + v % 4 of the workgroup's 32, row `col` of the block
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    __syncthreads();  // the block before is added up
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sums[wave][col][8 * (v / 4) + 4 * half + v % 4] = acc[b][v];
+    __syncthreads();
+    for (int e = tid; e < 32 * 32; e += 64 * WAVES) {
+      const int m = 32 * b + e / 32, n = n0 + e % 32;
+      float total = sums[0][e / 32][e % 32];
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) total += sums[w][e / 32][e % 32];
+      if (m < M && n < N) C[(size_t)m * ldc + n] = total;
+    }
+  }
+}
+
+template <int MB>
+static void launch_rows(const float* A, int lda, const float* W, int ldw, float* C, int ldc, int M, int N,
+                        int K, hipStream_t stream) {
+  const int groups = (N + 31) / 32;
+  if (groups < 256)
+    hipLaunchKernelGGL((gemm_f32_rows_kernel<MB, 8>), dim3(groups), dim3(512), 0, stream, A, lda, W, ldw, C,
+                       ldc, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_f32_rows_kernel<MB, 4>), dim3(groups), dim3(256), 0, stream, A, lda, W, ldw, C,
+                       ldc, M, N, K);
+}
+
 // ---- at most 16 rows ------------------------------------------------------------------------
 // A wave computes partial sums of MB x NC outputs (MB * NC = 64).  k is cut into blocks of 256;
 // KW waves of a workgroup share a set of columns and take every KW-th block each (KW = 1: a
@@ -343,7 +440,14 @@ extern "C" int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, fl
     return 0;
   }
   if (K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0) {
-    // more than 16 rows: the matrix cores, in tiles of 128 columns where those fill the chip
+    if (M <= 64) {  // the matrix cores fed from memory (measured against the tiles below: 8B shape's o-proj
+                    // 44 to 80 us at 17 to 64 rows against 120; at 96 and 128 rows the tiles are the faster)
+      if (M <= 32) launch_rows<1>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+      else launch_rows<2>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+      HAL_LAUNCH_CHECK();
+      return 0;
+    }
+    // more rows: the matrix cores, in tiles of 128 columns where those fill the chip
     const long long tiles_m = (M + MF_BM - 1) / MF_BM, wide = (N + 127) / 128, narrow = (N + 31) / 32;
     const bool use_wide = tiles_m * wide >= 256;
     const long long tiles_n = use_wide ? wide : narrow;

@@ -641,7 +641,8 @@ def test_gemm_f32(gpu, M, N, K):
     close(alone, whole[:1], 2e-6, "a row alone and in a larger batch")
 
 
-@pytest.mark.parametrize("M,N,K", [(8, 512, 4096), (16, 512, 14336), (48, 512, 4096), (2048, 384, 4096), (1500, 256, 14336)])
+@pytest.mark.parametrize("M,N,K", [(8, 512, 4096), (16, 512, 14336), (48, 512, 4096), (2048, 384, 4096), (1500, 256, 14336),
+                                   (17, 9000, 4096), (100, 300, 14336), (128, 96, 4100), (33, 40, 36)])
 def test_gemm_f32_with_rows_as_long_as_the_models(gpu, M, N, K):
     """Every kernel of the 32-bit product against the product in 64-bit, at the row lengths
     of the 8B shape.  One row of W is made of ones and A's entries are positive there, so
