@@ -84,12 +84,13 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
 // two k a call.  Which two k of the stage a call gets is free as long as A and B agree: the
 // lower half of the lanes takes the k's 8 s .. 8 s + 3, the upper half 8 s + 4 .. 8 s + 7
 // (s = 0 .. 3), one 16-byte LDS read per operand block and four calls each.  An output element
-// is the sum over k in that order, rounded as the instruction rounds; it depends on its own
-// row of A alone.
+// is the sum over k in that order, in stretches of 512 that each start from nothing (see the
+// kernel), rounded as the instruction rounds; it depends on its own row of A alone.
 #define MF_BM 128
 #define MF_BN 128
 #define MF_BK 32
 #define MF_KQ (MF_BK / 4)
+#define MF_STRETCH 512  // k of a stretch that is summed from nothing
 #define MF_XCDS 8  // dies of the gfx950 parts that this library is built for (a wrong count costs cache hits only)
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
@@ -112,8 +113,8 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restri
   // so that a die's workgroups are neighbours in the order of tiles (the same columns of W,
   // rows of A one after the other).
   int id = blockIdx.x;
-  const int total = tiles_m * tiles_n;
-  if (total % MF_XCDS == 0) id = (id % MF_XCDS) * (total / MF_XCDS) + id / MF_XCDS;
+  const int n_tiles = tiles_m * tiles_n;
+  if (n_tiles % MF_XCDS == 0) id = (id % MF_XCDS) * (n_tiles / MF_XCDS) + id / MF_XCDS;
   const int m0 = (id % tiles_m) * MF_BM, n0 = (id / tiles_m) * BN;
 
   float4 a_next[4], w_next[WV];
@@ -144,13 +145,16 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restri
     }
   };
 
-  f32x16 acc[NB][NB];
+  // An output element is summed in stretches of MF_STRETCH k, each from nothing, and the
+  // stretches' sums are added in order: one chain of K additions would round K / 2 times on top
+  // of each other (measured: four times the error of this at K = 14,336).
+  f32x16 acc[NB][NB], total[NB][NB];
 #pragma unroll
   for (int i = 0; i < NB; ++i)
 #pragma unroll
     for (int j = 0; j < NB; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = total[i][j][v] = 0.f;
   // this wave's corner of the tile
   const int wm = BN == 128 ? (wave / 2) * 64 : wave * 32, wn = BN == 128 ? (wave % 2) * 64 : 0;
   const int rows = wm + lane % 32, cols = wn + lane % 32, half = lane / 32;
@@ -183,6 +187,17 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restri
               acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i][e], bv[j][e], acc[i][j], 0, 0, 0);
       }
     }
+    if ((k0 + MF_BK) % MF_STRETCH == 0 || !more) {  // (the same for every thread)
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            total[i][j][v] += acc[i][j][v];
+            acc[i][j][v] = 0.f;
+          }
+    }
     if (more) put(buf ^ 1);  // (read last in the stage before the one that just ended)
     __syncthreads();
   }
@@ -195,7 +210,7 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restri
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int gm = m0 + wm + i * 32 + 8 * (v / 4) + 4 * half + v % 4;
-        if (gm < M && gn < N) C[(size_t)gm * ldc + gn] = acc[i][j][v];
+        if (gm < M && gn < N) C[(size_t)gm * ldc + gn] = total[i][j][v];
       }
     }
 }
