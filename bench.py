@@ -313,7 +313,8 @@ def main() -> int:
     ap.add_argument("--prefill-portion", type=int, default=0,
                     help="run the prompt of the prefill measurement in portions of this many tokens (0: whole)")
     ap.add_argument("--steps-ahead", type=int, default=1, choices=[0, 1],
-                    help="scheduler workloads: launch decode steps before the tokens of the step before are read")
+                    help="launch a decode step before the tokens of the step before are read, as the engine does "
+                         "by default (scheduling_steps_ahead); 0: read every step's tokens before the next is put together")
     ap.add_argument("--sampling", default="greedy", choices=["greedy", "temperature", "top_p", "top_k", "all"],
                     help="how the decode steps sample (the contract's line is greedy)")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b"],
@@ -420,14 +421,42 @@ def main() -> int:
                 marks.append((a, b))
             return toks.tolist()
 
-        for _ in range(warmup):
-            last = one_step(last)
-        sync()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            last = one_step(last)
-        sync()
-        dt = time.perf_counter() - t0
+        def steps_launched_ahead(tokens, n):
+            """``n`` steps as the engine runs them with ``scheduling_steps_ahead``: a step is
+            launched with the tokens of the step before still on the device (its segments name
+            their rows there), and the host reads a step's tokens while the next one runs."""
+            feed = torch.tensor(tokens, dtype=torch.int32, device=runner.device)
+            pinned, before = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)], None
+            for i in range(n):
+                segs = [Segment(s, runner.cache.length(s), [row], [0]) for row, s in enumerate(slots)]
+                logits = runner.step(segs, token_feed=feed)
+                feed, _ = sampler.forward(logits, params, seeds, draws)
+                pinned[i % 2].copy_(feed, non_blocking=True)
+                event = torch.cuda.Event()
+                event.record()
+                if before is not None:
+                    before[1].synchronize()
+                    tokens = before[0].tolist()
+                before = (pinned[i % 2], event)
+            before[1].synchronize()
+            return before[0].tolist()
+
+        if args.steps_ahead:
+            last = steps_launched_ahead(last, warmup)
+            sync()
+            t0 = time.perf_counter()
+            last = steps_launched_ahead(last, steps)
+            sync()
+            dt = time.perf_counter() - t0
+        else:
+            for _ in range(warmup):
+                last = one_step(last)
+            sync()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                last = one_step(last)
+            sync()
+            dt = time.perf_counter() - t0
         gpu_s = None
         if families:
             # the GPU's share of a step: a few more steps with events around each (outside
@@ -547,6 +576,7 @@ def main() -> int:
             "prefill_tokens": args.prefill_tokens,
             "page_size": runner.cache.page_size,
             "hip_graph": not args.no_graph,
+            "steps_ahead": args.steps_ahead,
             "sampling": args.sampling,
             "parallelism": "single GPU",
         },
@@ -562,7 +592,7 @@ def main() -> int:
     if gpu_s:
         record["host"] = {"wall_ms": round(gpu_s[1] / EXTRA_MARKED * 1e3, 4), "gpu_ms": round(gpu_s[0] / EXTRA_MARKED * 1e3, 4),
                           "share": round(max(0.0, 1.0 - gpu_s[0] / gpu_s[1]), 4),
-                          "how": f"{EXTRA_MARKED} further steps with HIP events around each"}
+                          "how": f"{EXTRA_MARKED} further steps with HIP events around each, every step's tokens read before the next"}
     if fam:
         # one eager step with events around every kernel wrapper: the weight stream of the
         # products and the cache stream of attention, each against 8 TB/s
