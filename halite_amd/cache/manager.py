@@ -153,6 +153,14 @@ class CacheManager:
         for g in self.groups:
             g.release_passed(slot, new_len)
 
+    def release_unused(self, slot: int) -> int:
+        """Gives back what ``reserve`` took for ``slot`` beyond its length (a step that was
+        prepared and did not come); returns the pages of the tightest group that this freed."""
+        freed = [g.release_beyond(slot, self.lengths[slot]) for g in self.groups]
+        if any(freed):
+            self.version += 1
+        return min(freed, default=0)
+
     def free(self, slot: int) -> None:
         self.version += 1
         for g in self.groups:

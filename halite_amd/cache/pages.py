@@ -154,6 +154,18 @@ class CacheGroup:
         self.pool.free(dead)
         return len(dead)
 
+    def release_beyond(self, slot: int, length: int) -> int:
+        """Gives back the pages behind the one that holds token ``length - 1`` (pages that
+        were taken for tokens that did not come)."""
+        table = self.tables.get(slot)
+        keep = -(-length // self.page_size)
+        if not table or len(table) <= keep:
+            return 0
+        dead = [p for p in table[keep:] if p >= 0]
+        del table[keep:]
+        self.pool.free(dead)
+        return len(dead)
+
     def release_all(self, slot: int) -> int:
         table = self.tables.pop(slot, [])
         self.released.pop(slot, None)

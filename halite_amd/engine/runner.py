@@ -91,6 +91,7 @@ class ModelRunner:
                 pos.tables(self.context_len)
         self._graphs: dict[int, dict] = {}  # batch size -> layout and recorded decode step
         self._ahead = None  # (requests and positions, cache version, context) of a step put together ahead
+        self._pages_taken_ahead: set[int] = set()  # slots for which such steps reserved and may not have come
         self.steps_taken_ahead = 0
         self._token_feed = None
         # graphs replay a model only if every part of it reads what varies on the device
@@ -296,7 +297,15 @@ class ModelRunner:
         )
         ahead = self._take_step_ahead(segments) if graph_step else None
         if ahead is None:  # a step that was put together ahead has its pages already
-            self.cache.reserve(spans)
+            try:
+                self.cache.reserve(spans)
+            except NoSpace:
+                # pages may be held for a step that was prepared ahead and is not the one that came
+                if not self._release_pages_taken_ahead():
+                    raise
+                self.cache.reserve(spans)
+        else:
+            self._pages_taken_ahead.difference_update(s.slot for s in segments)
         logits = None
         try:
             if graph_step:
@@ -340,10 +349,17 @@ class ModelRunner:
             self.cache.reserve([(s.slot, s.start + 1) for s in nxt])
         except NoSpace:
             return
+        self._pages_taken_ahead.update(s.slot for s in nxt)
         ctx = StepContext(nxt, self.cache, self.device, self._staging, static=entry["layout"])
         for run in self.model.runs:
             self.model.mixer_of_run(run.index).prepare(ctx, run)
         self._ahead = (tuple((s.slot, s.start) for s in nxt), self.cache.version, ctx)
+
+    def _release_pages_taken_ahead(self) -> bool:
+        """Gives back the pages of the step that was prepared ahead; whether any came back."""
+        slots, self._pages_taken_ahead = self._pages_taken_ahead, set()
+        live = self.cache.slots.live()
+        return sum(self.cache.release_unused(s) for s in slots if s in live) > 0
 
     def _take_step_ahead(self, segments: list[Segment]):
         ahead, self._ahead = self._ahead, None

@@ -106,6 +106,28 @@ def test_reserve_advance_free():
     m.check()
 
 
+def test_pages_taken_for_tokens_that_did_not_come_are_given_back():
+    m = manager({0: FULL, 1: WIN}, num_pages=9)
+    a, b = m.admit(), m.admit()
+    m.reserve([(a, 6)])
+    m.advance(a, 6)
+    m.reserve([(a, 9)])  # a step ahead: three more tokens, a page more in each group
+    assert [len(g.tables[a]) for g in m.groups] == [3, 3] and m.free_pages() == 5
+    with pytest.raises(NoSpace):
+        m.reserve([(b, 21)])
+    version = m.version
+    assert m.release_unused(a) == 1 and m.version > version
+    assert [len(g.tables[a]) for g in m.groups] == [2, 2] and m.free_pages() == 6
+    assert m.release_unused(a) == 0  # nothing beyond the length is left
+    m.reserve([(b, 21)])
+    m.check()
+    m.reserve([(a, 7)])  # the page that holds token 6 is still there
+    m.advance(a, 7)
+    m.check()
+    m.free(a), m.free(b)
+    assert m.idle()
+
+
 def test_all_or_nothing():
     m = manager(num_pages=5)  # 4 pages of 4 tokens
     a, b = m.admit(), m.admit()

@@ -482,6 +482,38 @@ def test_long_prompts_with_the_heads_of_the_8b_shape(dtype, tmp_path):
         del runner
 
 
+@pytest.mark.parametrize("page_size", [1, 4])
+def test_pages_taken_for_a_step_ahead_come_back_when_another_step_needs_them(folders, page_size):
+    """With graphs a decode step's successor is put together while the GPU works, pages and
+    all.  If another step comes instead, one that needs the pool's last pages for another
+    request, the pages taken ahead are given back: a pool of exactly the trace's peak
+    serves the trace."""
+    folder, requests, ref = folders[("A", "float32")]
+    a, b = requests["r1"], requests["r2"]
+    assert len(a) >= 12 and len(b) >= 9
+    trace = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:9], "want": [8]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[9:10], "want": [0]}], "end": []},  # recorded
+        {"step": 2, "entries": [{"id": "a", "tokens": a[10:11], "want": [0]}], "end": []},  # replayed
+        # replayed; its successor is prepared, with a page for a's thirteenth token (a's 12 fill three pages of 4)
+        {"step": 3, "entries": [{"id": "a", "tokens": a[11:12], "want": [0]}], "end": []},
+        {"step": 4, "entries": [{"id": "b", "tokens": b[:8], "want": [7]}], "end": ["a"]},  # the peak: a's 12 and b's 8
+        {"step": 5, "entries": [{"id": "b", "tokens": b[8:9], "want": [0]}], "end": ["b"]},
+    ]
+    peak = replay.peak_tokens(trace, page_size)
+    assert peak == 20
+    runner = make_runner(folder, "float32", peak, page_size=page_size, use_cudagraph=True)
+    for g in runner.cache.groups:
+        g.storage.fill_(float("nan"))
+    given_back = []
+    release = runner._release_pages_taken_ahead
+    runner._release_pages_taken_ahead = lambda: given_back.append(release()) or given_back[-1]
+    rows = replay.collect(trace, replay.run_trace(runner, trace), CONFIGS["A"]["vocab_size"])
+    replay.compare(rows, {"a": ref["r1"], "b": ref["r2"]}, TOL["float32"])
+    assert given_back == [True]  # (the case is the one that is meant)
+    assert runner.graph_replays >= 1 and runner.cache.idle()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_decode_graph_serves_key_ranges_of_one_piece_and_of_several(dtype, tmp_path):
     """A decode step's attention leaves a short key range whole (one workgroup, no partial
