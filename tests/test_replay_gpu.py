@@ -482,6 +482,66 @@ def test_long_prompts_with_the_heads_of_the_8b_shape(dtype, tmp_path):
         del runner
 
 
+def drawn_configuration(rng) -> dict:
+    """A Llama 3 configuration with every size and option drawn: head sizes that the bf16
+    matrix-core attention serves and others, groups of one to eight heads, widths and
+    vocabularies that are no powers of two."""
+    kv = rng.choice([1, 1, 2, 3, 4])
+    heads = kv * rng.choice([1, 2, 3, 4, 5, 8])
+    cfg = {
+        "architectures": ["LlamaForCausalLM"], "vocab_size": rng.randint(50, 3000), "hidden_size": 8 * rng.randint(2, 40),
+        "num_hidden_layers": rng.randint(1, 3), "num_attention_heads": heads, "num_key_value_heads": kv,
+        "head_dim": rng.choice([16, 32, 48, 64, 80, 96, 112, 128] if rng.random() < 0.7 else [8, 24, 40, 56, 72, 160, 256]),
+        "intermediate_size": 8 * rng.randint(3, 90), "rms_norm_eps": rng.choice([1e-5, 1e-6, 3e-4]),
+        "rope_theta": rng.choice([10000.0, 500000.0, 77777.0]), "max_position_embeddings": rng.choice([96, 300, 700]),
+        "tie_word_embeddings": rng.random() < 0.5,
+    }
+    if rng.random() < 0.5:
+        cfg["rope_scaling"] = {"rope_type": "llama3", "factor": rng.choice([2.0, 8.0, 32.0]), "low_freq_factor": 1.0,
+                               "high_freq_factor": rng.choice([2.0, 4.0]), "original_max_position_embeddings": rng.choice([32, 64, 128])}
+    return cfg
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(12))
+def test_drawn_configurations_under_the_mixed_schedule(dtype, seed, tmp_path):
+    """Configurations, page sizes, request lengths and the trace drawn from a seed: up to four
+    live requests, portions beside decoded tokens, a pool of exactly the trace's peak filled
+    with NaN, with and without graphs.  float32 within the suite's tolerance.  bfloat16 is
+    measured with the yardstick of the check at depth, since the format's cost depends on the
+    configuration: the plain implementation rounding to bfloat16 at the same places; the
+    engine's root mean square distance from float32 arithmetic may be 1.3 times that one's,
+    its largest difference twice that one's (the largest of many scatters)."""
+    import random
+
+    import full_depth_equality as depth
+
+    rng = random.Random(1000 * seed + (dtype == "bfloat16"))
+    cfg = drawn_configuration(rng)
+    page = rng.choice([8, 16, 32, 64, 128] if dtype == "bfloat16" else [1, 4, 8, 16, 32, 64])
+    lengths = [rng.randint(1, cfg["max_position_embeddings"]) for _ in range(rng.randint(2, 6))]
+    weights = tiny.random_weights(cfg, seed=rng.randint(0, 999), std=0.06)
+    requests = {f"r{i}": tiny.random_tokens(cfg, n, rng.randint(0, 9999)) for i, n in enumerate(lengths)}
+    folder = str(tmp_path / "model")
+    tiny.write_model_folder(folder, cfg, weights, torch.float32 if dtype == "float32" else torch.bfloat16)
+    pc, pw = plain_llama.read_model_folder(folder)  # (the stored, i.e. rounded, weights)
+    ref = {rid: plain_llama.forward(pc, pw, toks) for rid, toks in requests.items()}
+    trace = replay.mixed(requests, seed=rng.randint(0, 999))
+    runner = make_runner(folder, dtype, replay.peak_tokens(trace, page), page_size=page, use_cudagraph=rng.random() < 0.5)
+    for g in runner.cache.groups:
+        g.storage.fill_(float("nan"))
+    rows = replay.collect(trace, replay.run_trace(runner, trace), cfg["vocab_size"])
+    assert runner.cache.idle()
+    what = f"{cfg}, pages of {page}, requests of {lengths}"
+    worst, rms, _ = depth.distance(rows, ref)
+    if dtype == "float32":
+        assert worst <= TOL["float32"], what
+        return
+    rounding = {rid: plain_llama.forward(pc, pw, toks, round_to=torch.bfloat16) for rid, toks in requests.items()}
+    e_worst, e_rms, _ = depth.distance({rid: {p: rounding[rid][p] for p in rows[rid]} for rid in rows}, ref)
+    assert rms <= 1.3 * e_rms and worst <= 2.0 * e_worst, f"{what}: largest {worst:.3e} (format {e_worst:.3e}), rms {rms:.3e} (format {e_rms:.3e})"
+
+
 @pytest.mark.parametrize("page_size", [1, 4])
 def test_pages_taken_for_a_step_ahead_come_back_when_another_step_needs_them(folders, page_size):
     """With graphs a decode step's successor is put together while the GPU works, pages and
