@@ -485,14 +485,14 @@ def test_long_prompts_with_the_heads_of_the_8b_shape(dtype, tmp_path):
 def drawn_configuration(rng) -> dict:
     """A Llama 3 configuration with every size and option drawn: head sizes that the bf16
     matrix-core attention serves and others, groups of one to eight heads, widths and
-    vocabularies that are no powers of two."""
+    vocabularies that are no powers of two, some of them no multiples of eight."""
     kv = rng.choice([1, 1, 2, 3, 4])
     heads = kv * rng.choice([1, 2, 3, 4, 5, 8])
     cfg = {
-        "architectures": ["LlamaForCausalLM"], "vocab_size": rng.randint(50, 3000), "hidden_size": 8 * rng.randint(2, 40),
+        "architectures": ["LlamaForCausalLM"], "vocab_size": rng.randint(50, 3000), "hidden_size": rng.choice([8, 8, 2]) * rng.randint(2, 40),
         "num_hidden_layers": rng.randint(1, 3), "num_attention_heads": heads, "num_key_value_heads": kv,
         "head_dim": rng.choice([16, 32, 48, 64, 80, 96, 112, 128] if rng.random() < 0.7 else [8, 24, 40, 56, 72, 160, 256]),
-        "intermediate_size": 8 * rng.randint(3, 90), "rms_norm_eps": rng.choice([1e-5, 1e-6, 3e-4]),
+        "intermediate_size": rng.choice([8, 8, 2]) * rng.randint(3, 90), "rms_norm_eps": rng.choice([1e-5, 1e-6, 3e-4]),
         "rope_theta": rng.choice([10000.0, 500000.0, 77777.0]), "max_position_embeddings": rng.choice([96, 300, 700]),
         "tie_word_embeddings": rng.random() < 0.5,
     }
