@@ -6,8 +6,8 @@
 // Four kernels.  At most 16 rows (decode steps): a wave takes a few columns of the output,
 // its lanes take every 64th group of four k each (the rows of A come through LDS, shared by
 // the workgroup's four waves), and the partial sums of the lanes, and of the waves that share
-// columns, are added in a fixed order.  17 to 64 rows: the matrix cores fed straight from
-// memory, k split over a workgroup's waves.  More rows: tiles of 128 rows and 128 or 32
+// columns, are added in a fixed order.  17 to about 100 rows: the matrix cores, k split over a
+// workgroup's waves, each staging whole rows through LDS of its own.  More rows: tiles of 128 rows and 128 or 32
 // columns on the matrix cores, through LDS.  For sizes and addresses that are no multiples of
 // four: tiles of 64 x 64 on the vector units, each output element one chain of K
 // multiply-adds in index order.
@@ -215,47 +215,59 @@ gemm_f32_mfma_kernel(const float* __restrict__ A, int lda, const float* __restri
     }
 }
 
-// ---- 17 to 64 rows: the same instruction, fed from memory -----------------------------------
+// ---- 17 to 128 rows: the same instruction, k split over a workgroup's waves -----------------
 // Too many rows for the vector units' kernel below, too few for tiles to fill the chip: what
 // counts is that W streams.  A workgroup takes 32 columns (rows of W) and all rows of A; its
-// waves split k into stretches, one each, and every wave feeds the matrix cores straight from
-// memory: lane l brings 64 bytes of row l % 32 of W (which half of the 128 bytes of a stage:
-// l / 32) and the same of its rows of A, DEPTH stages ahead of the products, with no LDS and no
-// barrier on the way.  W is the first operand, so a lane ends with one row of A and sixteen
-// columns; the waves' sums meet in LDS and are added in rising wave number.
-// MB: blocks of 32 rows of A (M <= 32 MB; built for 1 and 2); WAVES: 4 or 8 (more where few columns leave
-// compute units idle).  An output element's sum depends on K and on WAVES, i.e. on the
-// matrix, and not on the rows beside it.
-template <int MB, int WAVES>
-__global__ void __launch_bounds__(64 * WAVES)
+// waves split k into stretches, one each, and work on their own from there: no barrier until
+// the end.  A wave brings a stage (32 k) of its 32 rows of W and of the rows of A in whole rows
+// (a load instruction reads eight rows of 128 bytes: eight cache lines; read in the operands'
+// own order, lane = row, it would touch 32 lines for the same bytes, which measured half the
+// rate), DEPTH stages ahead of the products, puts it into LDS of its own in the order of the
+// tiles above ([k / 4][row]) and reads the operands from there; a wave's LDS operations keep
+// their order, so one buffer will do.  W is the first operand, so a lane ends with one row of
+// A and sixteen columns; the waves' sums meet in LDS and are added in rising wave number.
+// MB: blocks of 32 rows of A (M <= 32 MB).  An output element's sum depends on K and on the
+// number of waves, i.e. on the matrix and on MB, and not on the rows beside it.
+// LDS that one lane of a wave writes and another reads: the wave's LDS operations are done in
+// the order they were issued; this keeps the compiler from moving them across.
+__device__ __forceinline__ void rows_wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int MB, int ROWS_WAVES>
+__global__ void __launch_bounds__(64 * ROWS_WAVES)
 gemm_f32_rows_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
                      float* __restrict__ C, int ldc, int M, int N, int K) {
-  constexpr int DEPTH = MB == 1 ? 4 : 3;  // stages in registers
-  __shared__ float sums[WAVES][32][33];  // [wave][row of A in a block][column], padded
+  constexpr int DEPTH = MB == 1 ? 4 : 2;  // stages in registers
+  constexpr int WS = 33, AS = 32 * MB + 1;  // rows of a stage and one more (the stores spread over the banks)
+  // per wave: W's stage [8][WS] and A's [8][AS] vectors; afterwards the waves' sums [32][33] floats
+  constexpr int PART = MF_KQ * (WS + AS);  // vectors of a wave
+  extern __shared__ float4 stage_s[];      // [ROWS_WAVES][PART]
+  static_assert(sizeof(float4) * PART >= sizeof(float) * 32 * 33, "the sums fit where the stages were");
   const int tid = threadIdx.x, lane = tid % HAL_WAVE, wave = tid / HAL_WAVE;
   const int col = lane % 32, half = lane / 32;
   const int n0 = blockIdx.x * 32;
+  float4* w_s = stage_s + wave * PART;
+  float4* a_s = w_s + MF_KQ * WS;
   // this wave's stretch of k: whole stages of 32
-  const int stages = (K + 31) / 32, each = (stages + WAVES - 1) / WAVES;
+  const int stages = (K + 31) / 32, each = (stages + ROWS_WAVES - 1) / ROWS_WAVES;
   const int k_begin = wave * each * 32, k_end = min(K, (wave + 1) * each * 32);
-  const bool w_in = n0 + col < N;
-  const float* wp = W + (size_t)(w_in ? n0 + col : 0) * ldw + 16 * half;
-  const float* ap[MB];
-  bool a_in[MB];
-#pragma unroll
-  for (int b = 0; b < MB; ++b) {
-    a_in[b] = 32 * b + col < M;
-    ap[b] = A + (size_t)(a_in[b] ? 32 * b + col : 0) * lda + 16 * half;
-  }
-  float4 wr[DEPTH][4], ar[DEPTH][MB][4];
+  // vector e = lane + 64 u of a stage: row e / 8, k 4 (e % 8)
+  const int r0 = lane / MF_KQ, kq0 = lane % MF_KQ;
+  float4 wr[DEPTH][4], ar[DEPTH][4 * MB];
   auto ask = [&](int d, int k) {  // (K is a multiple of 4: a vector is inside or outside)
+    const bool k_in = k + 4 * kq0 < k_end;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const bool k_in = k + 16 * half + 4 * j < k_end;
-      wr[d][j] = (k_in && w_in) ? *(const float4*)(wp + k + 4 * j) : float4{0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < 4; ++u) {
+      const int r = r0 + 8 * u;
+      wr[d][u] = (k_in && n0 + r < N) ? *(const float4*)(W + (size_t)(n0 + r) * ldw + k + 4 * kq0) : float4{0.f, 0.f, 0.f, 0.f};
+    }
 #pragma unroll
-      for (int b = 0; b < MB; ++b)
-        ar[d][b][j] = (k_in && a_in[b]) ? *(const float4*)(ap[b] + k + 4 * j) : float4{0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < 4 * MB; ++u) {
+      const int r = r0 + 8 * u;
+      ar[d][u] = (k_in && r < M) ? *(const float4*)(A + (size_t)r * lda + k + 4 * kq0) : float4{0.f, 0.f, 0.f, 0.f};
     }
   };
   f32x16 acc[MB];
@@ -269,45 +281,66 @@ gemm_f32_rows_kernel(const float* __restrict__ A, int lda, const float* __restri
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {  // (stages beyond the stretch hold zeros)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float wv[4] = {wr[d][j].x, wr[d][j].y, wr[d][j].z, wr[d][j].w};
+      for (int u = 0; u < 4; ++u) w_s[kq0 * WS + r0 + 8 * u] = wr[d][u];
+#pragma unroll
+      for (int u = 0; u < 4 * MB; ++u) a_s[kq0 * AS + r0 + 8 * u] = ar[d][u];
+      rows_wave_sync();  // what one lane put down another reads
+      ask(d, k + 32 * (d + DEPTH));  // (the other stages are on their way meanwhile)
+#pragma unroll
+      for (int s4 = 0; s4 < MF_KQ / 2; ++s4) {
+        const int kq = 2 * s4 + half;
+        const float4 w = w_s[kq * WS + col];
+        const float wv[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int b = 0; b < MB; ++b) {
-          const float av[4] = {ar[d][b][j].x, ar[d][b][j].y, ar[d][b][j].z, ar[d][b][j].w};
+          const float4 a = a_s[kq * AS + 32 * b + col];
+          const float av[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
           for (int e = 0; e < 4; ++e) acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[e], av[e], acc[b], 0, 0, 0);
         }
       }
-      ask(d, k + 32 * (d + DEPTH));  // (the other stages are on their way meanwhile)
+      rows_wave_sync();  // the stage is read before the next one is put down
     }
   }
   // element v of a lane's 16: column 8 (v / 4) + 4 half + v % 4 of the workgroup's 32, row `col` of the block
+  float* sums = (float*)stage_s;  // [wave][32][33], a wave's part where its stages were
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
-    __syncthreads();  // the block before is added up
+    __syncthreads();  // the block before is added up (and, the first time, every wave is done with its stages)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) sums[wave][col][8 * (v / 4) + 4 * half + v % 4] = acc[b][v];
+    for (int v = 0; v < 16; ++v) sums[wave * 4 * PART + col * 33 + 8 * (v / 4) + 4 * half + v % 4] = acc[b][v];
     __syncthreads();
-    for (int e = tid; e < 32 * 32; e += 64 * WAVES) {
+    for (int e = tid; e < 32 * 32; e += 64 * ROWS_WAVES) {
       const int m = 32 * b + e / 32, n = n0 + e % 32;
-      float total = sums[0][e / 32][e % 32];
+      float total = sums[(e / 32) * 33 + e % 32];
 #pragma unroll
-      for (int w = 1; w < WAVES; ++w) total += sums[w][e / 32][e % 32];
+      for (int w = 1; w < ROWS_WAVES; ++w) total += sums[w * 4 * PART + (e / 32) * 33 + e % 32];
       if (m < M && n < N) C[(size_t)m * ldc + n] = total;
     }
   }
 }
 
+template <int MB, int WAVES>
+static int launch_rows_with(const float* A, int lda, const float* W, int ldw, float* C, int ldc, int M, int N,
+                            int K, hipStream_t stream) {
+  const size_t smem = (size_t)WAVES * MF_KQ * (33 + 32 * MB + 1) * sizeof(float4);
+  static bool raised = false;  // more than 64 KB of LDS has to be asked for, once per kernel
+  if (!raised && smem > 64 * 1024) {
+    HAL_CHECK_HIP(hipFuncSetAttribute((const void*)gemm_f32_rows_kernel<MB, WAVES>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    raised = true;
+  }
+  hipLaunchKernelGGL((gemm_f32_rows_kernel<MB, WAVES>), dim3((N + 31) / 32), dim3(64 * WAVES), smem, stream, A,
+                     lda, W, ldw, C, ldc, M, N, K);
+  return 0;
+}
+
+// eight waves a workgroup where few columns leave compute units idle, four otherwise
 template <int MB>
-static void launch_rows(const float* A, int lda, const float* W, int ldw, float* C, int ldc, int M, int N,
-                        int K, hipStream_t stream) {
-  const int groups = (N + 31) / 32;
-  if (groups < 256)
-    hipLaunchKernelGGL((gemm_f32_rows_kernel<MB, 8>), dim3(groups), dim3(512), 0, stream, A, lda, W, ldw, C,
-                       ldc, M, N, K);
-  else
-    hipLaunchKernelGGL((gemm_f32_rows_kernel<MB, 4>), dim3(groups), dim3(256), 0, stream, A, lda, W, ldw, C,
-                       ldc, M, N, K);
+static int launch_rows(const float* A, int lda, const float* W, int ldw, float* C, int ldc, int M, int N,
+                       int K, hipStream_t stream) {
+  if ((N + 31) / 32 < 256) return launch_rows_with<MB, 8>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+  return launch_rows_with<MB, 4>(A, lda, W, ldw, C, ldc, M, N, K, stream);
 }
 
 // ---- at most 16 rows ------------------------------------------------------------------------
@@ -455,10 +488,15 @@ extern "C" int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, fl
     return 0;
   }
   if (K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0) {
-    if (M <= 64) {  // the matrix cores fed from memory (measured against the tiles below: 8B shape's o-proj
-                    // 44 to 80 us at 17 to 64 rows against 120; at 96 and 128 rows the tiles are the faster)
-      if (M <= 32) launch_rows<1>(A, lda, W, ldw, C, ldc, M, N, K, stream);
-      else launch_rows<2>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+    // up to 96 rows, and up to 128 on matrices of few columns: k split over a workgroup's waves (measured
+    // against the tiles below on the 8B shape's matrices: o-proj 31 / 50 / 74 / 100 us at 32 / 64 / 96 / 128
+    // rows against 120; gate and up together 129 / 204 / 287 / 414 us against 275 to 368)
+    if (M <= 96 || (M <= 128 && (N + 127) / 128 < 128)) {
+      if (M <= 32 ? launch_rows<1>(A, lda, W, ldw, C, ldc, M, N, K, stream)
+          : M <= 64 ? launch_rows<2>(A, lda, W, ldw, C, ldc, M, N, K, stream)
+          : M <= 96 ? launch_rows_with<3, 4>(A, lda, W, ldw, C, ldc, M, N, K, stream)
+                    : launch_rows_with<4, 4>(A, lda, W, ldw, C, ldc, M, N, K, stream))
+        return 1;
       HAL_LAUNCH_CHECK();
       return 0;
     }
