@@ -422,3 +422,35 @@ def test_stop_strings_through_the_engine(models, ahead):
     with pytest.raises(ValueError, match="tokenizer"):
         InferenceEngine.from_pretrained(folder, server, ModelConfig(dtype="float32")).infer_batch(
             [(prompts[0], {"max_new_tokens": 3, "stop": "ab"})])
+
+
+def test_the_bench_line_keeps_its_contract():
+    """One JSON line with the keys that whoever runs ``bench.py`` reads (here with one layer,
+    a short context and a short prompt, so that it takes seconds); more than one GPU is
+    refused in one line with exit status 2."""
+    cmd = [sys.executable, os.path.join(ROOT, "bench.py"), "--layers", "1", "--steps", "4", "--warmup", "2",
+           "--context", "1024", "--prefill-tokens", "256", "--no-extras"]
+    proc = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = proc.stdout.strip().split("\n")
+    assert len(lines) == 1
+    rec = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "prefill", "roofline", "points"):
+        assert key in rec, key
+    assert rec["n_gpus"] == 1 and rec["steps"] == 4 and rec["warmup"] == 2 and rec["higher_is_better"] is True
+    assert rec["dtype"] == "bf16" and rec["unit"] == "tok/s" and rec["value"] > 0
+    assert abs(rec["value"] - 8 / rec["ms_per_step"] * 1e3) < 0.01 * rec["value"]
+    config = rec["config"]
+    assert len(config) <= 20 and all(not isinstance(v, (dict, list)) for v in config.values())
+    assert config["layers"] == 1 and config["layers_of_model"] == 32 and config["global_batch"] == 8 and config["seq_len"] == 1024
+    for key in ("hidden_size", "heads", "kv_heads", "head_dim", "intermediate_size", "vocab_size"):
+        assert config[key] > 0
+    assert set(rec["prefill"]) >= {"value", "tokens", "ms", "frac"} and rec["prefill"]["tokens"] == 256
+    roof = rec["roofline"]
+    assert roof["bound"] == "hbm" and roof["unit"] == "GB/s" and roof["peak"] == 8000.0
+    assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
+    assert rec["points"]["decode_b1"] > 0 and rec["points"]["decode_b64"] > 0
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], cwd=ROOT, capture_output=True,
+                          text=True, timeout=120)
+    assert proc.returncode == 2 and len((proc.stdout + proc.stderr).strip().split("\n")) == 1
